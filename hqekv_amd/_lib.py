@@ -1,0 +1,125 @@
+"""ctypes binding of libhqekv.so (the C ABI declared in include/hqekv.h).
+
+The product path has no CPU fallback: if the shared library is missing, or a call fails,
+an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from pathlib import Path
+from typing import Optional
+
+import torch
+
+_PKG = Path(__file__).resolve().parent
+_LIB_PATH = Path(os.environ.get("HQEKV_LIB", _PKG / "libhqekv.so"))
+
+MAX_SEGS = 8
+
+# every symbol include/hqekv.h declares
+EXPORTS = (
+    "hqekv_version", "hqekv_last_error",
+    "hqekv_quant_pack_rows", "hqekv_quant_pack_k_tokenmajor", "hqekv_dequant_unpack_rows", "hqekv_pack_i32",
+    "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group",
+    "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
+    "hqekv_decode_attn",
+)
+
+
+class Seg(C.Structure):
+    """Mirror of ``struct hqekv_seg``."""
+    _fields_ = [
+        ("bits", C.c_int32),
+        ("token_major", C.c_int32),
+        ("n_tokens", C.c_int64),
+        ("pos_base", C.c_int64),
+        ("data", C.c_void_p),
+        ("scale", C.c_void_p),
+        ("zero", C.c_void_p),
+        ("idx", C.c_void_p),
+    ]
+
+
+_lib: Optional[C.CDLL] = None
+
+_i64, _int, _vp = C.c_int64, C.c_int, C.c_void_p
+_SEGP = C.POINTER(Seg)
+
+_PROTOS = {
+    "hqekv_version": (C.c_int, []),
+    "hqekv_last_error": (C.c_char_p, []),
+    "hqekv_quant_pack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
+    "hqekv_quant_pack_k_tokenmajor": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
+    "hqekv_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
+    "hqekv_pack_i32": (C.c_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "hqekv_gemv_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64, _int]),
+    "hqekv_gemv_uniform_group": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
+    "hqekv_qk_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "hqekv_scale_softmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, C.c_float, _vp]),
+    "hqekv_pv_workspace_bytes": (_i64, [_SEGP, _int, _i64, _i64, _i64, _i64]),
+    "hqekv_pv_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "hqekv_decode_attn": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
+}
+
+
+def lib_path() -> Path:
+    return _LIB_PATH
+
+
+def load() -> C.CDLL:
+    """Load libhqekv.so once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build it with `python -m hqekv_amd.build` "
+                "(there is no CPU fallback for the HIP path)")
+        lib = C.CDLL(str(_LIB_PATH))
+        for name, (res, args) in _PROTOS.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    """Turn a non-zero return code into the exception the reference's callers expect."""
+    if rc == 0:
+        return
+    msg = load().hqekv_last_error().decode("utf-8", "replace")
+    if rc < 0:
+        raise ValueError(f"{what}: {msg} (code {rc})")
+    raise RuntimeError(f"{what}: HIP error {rc}: {msg}")
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU: the HIP path has no CPU fallback")
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def make_segs(items) -> "C.Array[Seg]":
+    """items: iterable of dicts with keys bits, n_tokens, data, scale, zero, idx, pos_base, token_major."""
+    items = list(items)
+    if len(items) > MAX_SEGS:
+        raise ValueError("too many segments")
+    arr = (Seg * max(1, len(items)))()
+    for s, it in zip(arr, items):
+        s.bits = it["bits"]
+        s.token_major = int(it.get("token_major", 0))
+        s.n_tokens = it["n_tokens"]
+        s.pos_base = int(it.get("pos_base", 0))
+        s.data = ptr(it["data"])
+        s.scale = ptr(it.get("scale"))
+        s.zero = ptr(it.get("zero"))
+        s.idx = ptr(it.get("idx"))
+    return arr

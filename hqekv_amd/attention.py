@@ -1,0 +1,189 @@
+"""Host glue between the reference's 42-field cache tuple and the hybrid HIP launches.
+
+The tuple layout is the reference's (quant/quant_matmul_hq.py:34-38):
+  0 sixteen_K (B,Hkv,D,T16)  1 sixteen_K_idx  2 sixteen_V (B,Hkv,T16,D)  3 sixteen_V_idx
+  K class b at base 4/12/20/28 (8/4/2/1 bit): code, idx, scale, zero;  V class at 8/16/24/32
+  36 outliers  37 outliers_idx  38 V_token_norm  39 new_K (B,Hkv,Tn,D)  40 new_V  41 kv_seq_len
+Each populated class becomes one ``hqekv_seg``; the kernels read the tensors where they lie.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+BITS = (8, 4, 2)
+K_BASE = {8: 4, 4: 12, 2: 20, 1: 28}
+V_BASE = {8: 8, 4: 16, 2: 24, 1: 32}
+K16, K16_IDX, V16, V16_IDX = 0, 1, 2, 3
+NEW_K, NEW_V, KV_SEQ_LEN = 39, 40, 41
+
+
+def _idx(t: Optional[torch.Tensor], n: int, dev) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    if t.dtype != torch.int64:
+        t = t.to(torch.int64)
+    if t.device != dev:
+        t = t.to(dev)
+    t = t.contiguous()
+    if t.numel() != n:
+        raise ValueError(f"index of length {t.numel()} for a class of {n} tokens")
+    return t
+
+
+def _f16_k_item(k16: torch.Tensor, idx, keep: list) -> dict:
+    """fp16 K class (B,Hkv,D,T): read channel-major, or token-major if it is a transposed view."""
+    B, H, D, T = k16.shape
+    if k16.is_contiguous():
+        data, tm = k16, 0
+    elif k16.stride(2) == 1 and k16.transpose(2, 3).is_contiguous():
+        data, tm = k16, 1  # memory is (B,Hkv,T,D)
+    else:
+        data, tm = k16.contiguous(), 0
+    keep.append(data)
+    return dict(bits=16, n_tokens=T, data=data, idx=idx, token_major=tm)
+
+
+def key_segments(pkv: tuple, dev, Tall: int, keep: list) -> Tuple[List[dict], int, int]:
+    items = []
+    nh_kv = D = None
+    if pkv[K16] is not None:
+        k = pkv[K16]
+        nh_kv, D = k.shape[1], k.shape[2]
+        items.append(_f16_k_item(k, _idx(pkv[K16_IDX], k.shape[3], dev), keep))
+    for b in BITS:
+        base = K_BASE[b]
+        if pkv[base] is not None:
+            code = pkv[base].contiguous()
+            sc, zr = pkv[base + 2].contiguous(), pkv[base + 3].contiguous()
+            n = code.shape[3] * (32 // b)
+            nh_kv, D = code.shape[1], code.shape[2]
+            idx = _idx(pkv[base + 1], n, dev)
+            keep += [code, sc, zr, idx]
+            items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx))
+    if pkv[K_BASE[1]] is not None:
+        raise NotImplementedError("the 1-bit normal-quantile class is not built")
+    new_K = pkv[NEW_K]
+    if new_K is not None and new_K.shape[2] > 0:
+        nk = new_K.contiguous()
+        keep.append(nk)
+        nh_kv, D = nk.shape[1], nk.shape[3]
+        n = nk.shape[2]
+        items.append(dict(bits=16, n_tokens=n, data=nk, idx=None, pos_base=Tall - n, token_major=1))
+    return items, nh_kv, D
+
+
+def value_segments(pkv: tuple, dev, Tall: int, keep: list) -> Tuple[List[dict], int, int]:
+    items = []
+    nh_kv = D = None
+    if pkv[V16] is not None:
+        v = pkv[V16].contiguous()
+        nh_kv, D = v.shape[1], v.shape[3]
+        idx = _idx(pkv[V16_IDX], v.shape[2], dev)
+        keep += [v, idx]
+        items.append(dict(bits=16, n_tokens=v.shape[2], data=v, idx=idx))
+    for b in BITS:
+        base = V_BASE[b]
+        if pkv[base] is not None:
+            code = pkv[base].contiguous()
+            sc, zr = pkv[base + 2].contiguous(), pkv[base + 3].contiguous()
+            n = code.shape[2]
+            nh_kv, D = code.shape[1], code.shape[3] * (32 // b)
+            idx = _idx(pkv[base + 1], n, dev)
+            keep += [code, sc, zr, idx]
+            items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx))
+    if pkv[V_BASE[1]] is not None:
+        raise NotImplementedError("the 1-bit normal-quantile class is not built")
+    new_V = pkv[NEW_V]
+    if new_V is not None and new_V.shape[2] > 0:
+        nv = new_V.contiguous()
+        keep.append(nv)
+        nh_kv, D = nv.shape[1], nv.shape[3]
+        n = nv.shape[2]
+        items.append(dict(bits=16, n_tokens=n, data=nv, idx=None, pos_base=Tall - n))
+    return items, nh_kv, D
+
+
+def value_length(pkv: tuple) -> int:
+    """Sum of the V class lengths plus the residual (quant/hqe_matmul.py:379-402)."""
+    n = 0
+    if pkv[V16] is not None:
+        n += pkv[V16].shape[2]
+    for b in (8, 4, 2, 1):
+        if pkv[V_BASE[b]] is not None:
+            n += pkv[V_BASE[b]].shape[2]
+    if pkv[NEW_V] is not None:
+        n += pkv[NEW_V].shape[2]
+    return n
+
+
+def _mask_arg(mask, B: int, Hq: int, Tall: int, dev, keep: list):
+    """-> (pointer or None, row stride in elements) for an additive fp16 mask."""
+    if mask is None:
+        return None, 0
+    if not torch.is_tensor(mask):
+        if float(mask) == 0.0:
+            return None, 0
+        mask = torch.full((1, 1, 1, Tall), float(mask), dtype=torch.float16, device=dev)
+    mask = mask.to(device=dev, dtype=torch.float16)
+    while mask.dim() < 4:
+        mask = mask.unsqueeze(0)
+    if mask.shape[-1] != Tall or mask.shape[-2] != 1:
+        mask = mask.expand(*mask.shape[:-2], 1, Tall) if mask.shape[-1] in (1, Tall) else mask
+        if mask.shape[-1] != Tall:
+            raise ValueError(f"mask last dim {mask.shape[-1]} != {Tall}")
+    if mask.shape[0] == 1 and mask.shape[1] == 1:
+        m = mask.reshape(Tall).contiguous()
+        keep.append(m)
+        return m.data_ptr(), 0
+    m = mask.expand(B, Hq, 1, Tall).contiguous()
+    keep.append(m)
+    return m.data_ptr(), Tall
+
+
+def workspace_for(v_segs, n_v: int, B: int, Hq: int, Hkv: int, D: int, dev) -> torch.Tensor:
+    need = _lib.load().hqekv_pv_workspace_bytes(v_segs, n_v, B, Hq, Hkv, D)
+    if need < 0:
+        raise ValueError("invalid segment table")
+    return torch.empty(max(need, 16) // 4, dtype=torch.float32, device=dev)
+
+
+def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool):
+    """q (B,Hq,1,D) fp16 -> (attn_weights (B,Hq,1,Tall) fp16 probabilities, attn_output (B,Hq,1,D) fp16).
+
+    One qk launch over all K classes, the scale/mask/clamp/softmax pass, one p.V launch over all
+    V classes plus the fixed-order combine, on torch's current stream.
+    """
+    _lib.require_gpu(q, "q")
+    if q.dtype != torch.float16:
+        raise TypeError("q must be float16 (the cache is fp16 by definition)")
+    if q.dim() != 4 or q.shape[2] != 1:
+        raise ValueError("q must be (B, Hq, 1, D): only single-token decode is computed")
+    B, Hq, _, D = q.shape
+    dev = q.device
+    keep: list = []
+    k_items, hk, dk = key_segments(pkv, dev, Tall, keep)
+    v_items, hv, dv = value_segments(pkv, dev, Tall, keep)
+    Hkv = hk if hk is not None else hv
+    if Hkv is None:
+        raise ValueError("invalid past_key_value")
+    for d_ in (dk, dv):
+        if d_ is not None and d_ != D:
+            raise ValueError("head_dim of the cache does not match q")
+    qc = q.contiguous()
+    weights = (torch.zeros if zero_init else torch.empty)(B, Hq, 1, Tall, dtype=torch.float16, device=dev)
+    out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev)
+    k_segs, v_segs = _lib.make_segs(k_items), _lib.make_segs(v_items)
+    mptr, mstride = _mask_arg(mask, B, Hq, Tall, dev, keep)
+    with torch.cuda.device(dev):
+        ws = workspace_for(v_segs, len(v_items), B, Hq, Hkv, D, dev)
+        rc = _lib.load().hqekv_decode_attn(
+            k_segs, len(k_items), v_segs, len(v_items), qc.data_ptr(), mptr, mstride,
+            weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4,
+            _lib.stream_ptr(dev))
+    _lib.check(rc, "decode_attention")
+    return weights, out

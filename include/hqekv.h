@@ -1,0 +1,161 @@
+/*
+ * libhqekv -- C ABI of the MI355X (gfx950) quantized-KV decode-attention path.
+ *
+ * Plain pointers and sizes only: every pointer is a DEVICE pointer unless stated otherwise,
+ * `stream` is a hipStream_t passed as void* (NULL = the null stream).  The library never
+ * allocates or frees device memory, never synchronises, never switches device and keeps no
+ * pointer after a call returns.  Outputs and workspaces are owned by the caller.
+ *
+ * Return value of every int function: 0 = ok, < 0 = invalid argument (HQEKV_E_*),
+ * > 0 = a hipError_t raised by the launch.  hqekv_last_error() returns a thread-local
+ * description of the last non-zero return.
+ *
+ * Storage layouts are the reference's cache layouts, consumed as stored (no transposes):
+ *   K class, b bits : code (B,Hkv,D,T/pf) int32, scale/zero (B,Hkv,D,T/32) fp16, pf = 32/b
+ *   V class, b bits : code (B,Hkv,T,D/pf) int32, scale/zero (B,Hkv,T,D/32) fp16
+ *   fp16 K class    : (B,Hkv,D,T) fp16 (channel-major);  fp16 V class: (B,Hkv,T,D)
+ *   residual new_K / new_V : (B,Hkv,T,D) fp16 (token-major)
+ * Codes are packed LSB first: word j holds elements j*pf .. j*pf+pf-1 of the last axis.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * reference checkout).
+ */
+#ifndef HQEKV_H
+#define HQEKV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HQEKV_OK 0
+#define HQEKV_E_ARG (-1)      /* bad size / bits / null pointer            */
+#define HQEKV_E_ALIGN (-2)    /* pointer or stride not aligned as required */
+#define HQEKV_E_WORKSPACE (-3)/* workspace too small                       */
+#define HQEKV_E_UNSUPPORTED (-4)
+
+#define HQEKV_MAX_SEGS 8
+#define HQEKV_GROUP 32
+
+int hqekv_version(void);
+const char *hqekv_last_error(void);
+
+/* ------------------------------------------------------------------ quantise / pack
+ * Replaces uniform_group_quantize_pack_last_dim (quant/pack_unpack.py:156-193: the
+ * min/max/scale/sub/div/clamp/round torch chain plus the Triton _pack_along_last_dim
+ * kernel at :16-51) with one pass.
+ *
+ * x is (n_outer, n_rows, L) fp16 with a contiguous last axis; groups of 32 along L.
+ * Strides are in ELEMENTS of the respective array (fp16 for x/scale/zero, int32 words for
+ * code), so the outputs may be windows of larger, capacity-sized cache buffers (append).
+ * Requires L % 32 == 0, x 16-byte aligned rows (x strides % 8 == 0).
+ */
+int hqekv_quant_pack_rows(const void *x, int64_t x_outer_stride, int64_t x_row_stride,
+                          void *code, int64_t code_outer_stride, int64_t code_row_stride,
+                          void *scale, void *zero, int64_t sz_outer_stride, int64_t sz_row_stride,
+                          int64_t n_outer, int64_t n_rows, int64_t L, int bits, void *stream);
+
+/* Same quantiser for K handed over token-major: x is (n_outer, T, D) fp16 (what the model
+ * produces), groups are 32 consecutive TOKENS of one channel, outputs are channel-major:
+ * code (n_outer, D, T/pf), scale/zero (n_outer, D, T/32).  Replaces the
+ * `.transpose(2, 3)` + reshape copy + quantiser of quant_new_K (quant/hqe_2.py:31-35).
+ * Requires T % 32 == 0, D % 2 == 0.
+ */
+int hqekv_quant_pack_k_tokenmajor(const void *x, int64_t x_outer_stride, int64_t x_token_stride,
+                                  void *code, int64_t code_outer_stride, int64_t code_row_stride,
+                                  void *scale, void *zero, int64_t sz_outer_stride, int64_t sz_row_stride,
+                                  int64_t n_outer, int64_t T, int64_t D, int bits, void *stream);
+
+/* Replaces uniform_group_dequantize_unpack_last_dim (quant/pack_unpack.py:316-333):
+ * out = rnd16(rnd16(fp16(code) * scale) + zero), (n_outer, n_rows, L) fp16.
+ * scale == NULL: plain unpack_along_last_dim (quant/pack_unpack.py:255-295), codes as fp16.
+ */
+int hqekv_dequant_unpack_rows(const void *code, int64_t code_outer_stride, int64_t code_row_stride,
+                              const void *scale, const void *zero, int64_t sz_outer_stride,
+                              int64_t sz_row_stride, void *out, int64_t out_outer_stride,
+                              int64_t out_row_stride, int64_t n_outer, int64_t n_rows, int64_t L,
+                              int bits, void *stream);
+
+/* Replaces pack_along_last_dim (quant/pack_unpack.py:16-70): q is (n_rows, L) int32 codes,
+ * code is (n_rows, L/pf) int32, both contiguous. */
+int hqekv_pack_i32(const void *q, void *code, int64_t n_rows, int64_t L, int bits, void *stream);
+
+/* ------------------------------------------------------------------ per-class GEMV
+ * Replaces gemv_forward_cuda_uniform_group (quant/csrc/gemv_cuda.h:46-54, launched from
+ * cuda_bmm_fA_qB_uniform_group, quant/matmul.py:263-299) and
+ * gemv_forward_cuda_wv_uniform_group (gemv_cuda.h:235-243), WITHOUT the three
+ * transpose().contiguous() copies of matmul.py:293-295:
+ *
+ *   out[b,hq,n] = sum_k fA[b,hq,k] * (scale[b,hkv,k,n/32] * code[b,hkv,k,n] + zero[b,hkv,k,n/32])
+ *
+ * fA (B,Hq,K) fp16, code (B,Hkv,K,N/pf) int32, scale/zero (B,Hkv,K,N/32) fp16, out (B,Hq,N)
+ * fp16; hkv = hq / (Hq/Hkv).  fp32 accumulation, one rounding to fp16.
+ * q.K^T is K = head_dim, N = tokens;  p.V is K = tokens, N = head_dim.
+ * `workspace` is needed only when hqekv_gemv_workspace_bytes() > 0 (split-K partials).
+ */
+int64_t hqekv_gemv_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N, int bits);
+int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale, const void *zero,
+                             void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N,
+                             int bits, void *workspace, int64_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------ hybrid (all classes, one launch)
+ * One segment = one precision class of one layer's cache.  `idx` maps element j of the class
+ * to its position in the compacted sequence (int64, shared by all batch rows and heads,
+ * quant/csrc/gemv_cuda_uniform.cu:945); idx == NULL means position = pos_base + j (used for
+ * the fp16 residual at the tail).  Evicted tokens are simply absent from every segment.
+ */
+typedef struct hqekv_seg {
+  int32_t bits;          /* 16, 8, 4 or 2                                              */
+  int32_t token_major;   /* K segments with bits == 16 only: 1 = (B,Hkv,T,D) residual   */
+  int64_t n_tokens;      /* multiple of 32 unless bits == 16                           */
+  int64_t pos_base;      /* used when idx == NULL                                      */
+  const void *data;      /* codes (int32) or fp16 values                               */
+  const void *scale;     /* NULL when bits == 16                                       */
+  const void *zero;
+  const int64_t *idx;    /* (n_tokens) or NULL                                         */
+} hqekv_seg;
+
+/* Replaces gemv_forward_cuda_qk_group_hq (quant/csrc/gemv_cuda.h:78-109; kernel
+ * quant/csrc/gemv_cuda_uniform.cu:941-1228), i.e. cuda_bmm_forward_qk_group_hq
+ * (quant/matmul.py:351-434): raw scores q.K^T scattered through idx.
+ * q (B,Hq,D) fp16 -> scores (B,Hq,Tall) fp16 (row stride Tall).  `segs` is a HOST pointer.
+ */
+int hqekv_qk_hybrid(const hqekv_seg *segs, int nseg, const void *q, void *scores, int64_t B,
+                    int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, void *stream);
+
+/* Replaces the torch epilogue of qkv_matmul (quant/quant_matmul_hq.py:100-103):
+ * w = rnd16(w * (1/sqrt(D))) ; w += mask ; w = max(w, -65504) ; softmax in fp32 ; round to fp16.
+ * In place on scores (B*Hq rows of Tall).  mask may be NULL; otherwise fp16 with
+ * mask_row_stride elements between (b,hq) rows (0 = one row broadcast to all).
+ */
+int hqekv_scale_softmax(void *scores, const void *mask, int64_t mask_row_stride, int64_t n_rows,
+                        int64_t Tall, float inv_sqrt_d, void *stream);
+
+/* Replaces gemv_forward_cuda_wv_group_hq (quant/csrc/gemv_cuda.h:139-170; kernel
+ * quant/csrc/gemv_cuda_wv_uniform.cu:347-745), i.e. cuda_bmm_forward_wv_group_hq
+ * (quant/matmul.py:507-579): out[b,hq,:] = sum over segments of p[b,hq,idx[j]] * V[j,:].
+ * p (B,Hq,Tall) fp16, out (B,Hq,D) fp16.  Split-K over tokens with a deterministic,
+ * fixed-order combine (no float atomics).  `segs` is a HOST pointer.
+ */
+int64_t hqekv_pv_workspace_bytes(const hqekv_seg *segs, int nseg, int64_t B, int64_t Hq,
+                                 int64_t Hkv, int64_t D);
+int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, int64_t B,
+                    int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, void *workspace,
+                    int64_t workspace_bytes, void *stream);
+
+/* The whole decode-attention layer-step: qk_hybrid -> scale_softmax -> pv_hybrid on one
+ * stream.  Replaces qkv_matmul / qkv_matmul_hq (quant/quant_matmul_hq.py:23-174) and
+ * qkv_matmul_hqe_2 (quant/hqe_matmul.py:354-451).  attn_weights (B,Hq,Tall) fp16 receives
+ * the probabilities (the caller's importance tracker needs them, model/llama_hqe.py:200).
+ */
+int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
+                      const void *q, const void *mask, int64_t mask_row_stride,
+                      void *attn_weights, void *attn_out, int64_t B, int64_t Hq, int64_t Hkv,
+                      int64_t D, int64_t Tall, void *workspace, int64_t workspace_bytes,
+                      void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HQEKV_H */

@@ -1,0 +1,317 @@
+"""CPU oracle for the quantized-KV decode-attention path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, on the CPU and with plain torch tensor ops, what the reference
+computes on its GPU path.  It is imported by ``tests/``, by ``__graft_entry__.smoke()``
+and by the ``cpu_baseline`` leg of ``bench.py`` -- never by the product package.
+
+Every function cites the reference lines it follows (paths relative to the reference
+checkout).  How each function is pinned (known answers, closed forms, brute force) is
+listed next to it; the checks themselves live in ``tests/test_oracle.py`` and
+``tests/golden/``.
+
+Pinned:
+  pack_along_last_dim / unpack_along_last_dim   closed form, round trip, KAT 0xE4E4E4E4
+  uniform_group_quantize_pack_last_dim          arange(128) known answer, 8-bit identity,
+                                                invariants (min->0, 0<=c<=qmax, |x-dq|<=s/2)
+  uniform_group_dequantize_unpack_last_dim      closed form on hand-computed values
+  gemv_uniform_group                            special cases that collapse to integer
+                                                mat-vec / torch.matmul
+  qkv_matmul                                    permutation invariance against dense attention
+  compress_cache / rerank_after_eviction        brute force against Python sets
+
+Parity unpinned (no reference fixture exists and only a run of the original GPU stack
+could pin it): the last-bit behaviour of ``fp16_tensor / python_int`` on the GPU, which
+ATen evaluates as multiply-by-reciprocal.  ``scalar_div='recip'`` restates that rule,
+``scalar_div='true'`` is the CPU rule; the GPU test-suite checks the HIP kernels against
+torch's own on-device op chain to close the gap.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+BITS = (8, 4, 2)
+
+# --------------------------------------------------------------------------- pack / unpack
+
+
+def pack_along_last_dim(data: torch.Tensor, bit: int) -> torch.Tensor:
+    """word[..., j] = OR_i (q[..., j*pf+i] << (i*bit)), LSB first, int32.
+
+    Follows quant/pack_unpack.py:40-51 (Triton ``_pack_along_last_dim``) and the
+    wrapper at :53-70.
+    """
+    pf = 32 // bit
+    assert data.dtype == torch.int32 and data.shape[-1] % pf == 0
+    q = data.reshape(*data.shape[:-1], data.shape[-1] // pf, pf).to(torch.int64)
+    word = torch.zeros(q.shape[:-1], dtype=torch.int64)
+    for i in range(pf):
+        word |= (q[..., i] & ((1 << 32) - 1)) << (i * bit)
+    word &= (1 << 32) - 1
+    # reinterpret the unsigned 32-bit payload as int32 (the sign bit is just payload)
+    word = torch.where(word >= (1 << 31), word - (1 << 32), word)
+    return word.to(torch.int32)
+
+
+def unpack_codes(code: torch.Tensor, bit: int) -> torch.Tensor:
+    """Integer codes ``(word >> i*bit) & (0xFF >> (8-bit))`` as int32, last dim * pf.
+
+    quant/pack_unpack.py:272-278.
+    """
+    pf = 32 // bit
+    mask = 0xFF >> (8 - bit)
+    w = code.to(torch.int64) & ((1 << 32) - 1)
+    shifts = torch.arange(pf, dtype=torch.int64) * bit
+    c = (w.unsqueeze(-1) >> shifts) & mask
+    return c.reshape(*code.shape[:-1], code.shape[-1] * pf).to(torch.int32)
+
+
+def unpack_along_last_dim(code: torch.Tensor, bit: int) -> torch.Tensor:
+    """Codes stored as fp16 (quant/pack_unpack.py:281-295)."""
+    return unpack_codes(code, bit).to(torch.float16)
+
+
+# --------------------------------------------------------------------------- quantise
+
+
+def _div_scalar_fp16(x: torch.Tensor, divisor: int, scalar_div: str) -> torch.Tensor:
+    """``fp16_tensor / python_int``.
+
+    'recip': what ATen's GPU true-divide does for a CPU scalar divisor -- the fp32
+    reciprocal is formed first, then an fp32 multiply, then one rounding to fp16.
+    'true' : fp32 divide then one rounding to fp16 (the CPU rule).
+    """
+    xf = x.to(torch.float32)
+    if scalar_div == "recip":
+        inv = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(float(divisor), dtype=torch.float32)
+        return (xf * inv).to(torch.float16)
+    if scalar_div == "true":
+        return (xf / float(divisor)).to(torch.float16)
+    raise ValueError("scalar_div must be 'recip' or 'true'")
+
+
+def uniform_group_quantize_pack_last_dim(
+    data: torch.Tensor, group_size: int, bit: int, scalar_div: str = "recip"
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Asymmetric min/max group quantiser over the last dim; quant/pack_unpack.py:156-193.
+
+    fp16 op chain, each arrow one rounding to fp16:
+      mn, mx -> (mx - mn) -> / qmax -> scale ;  x - mn -> / scale -> clamp -> round-half-even
+    A group with mx == mn gives 0/0 = NaN, which the GPU's float->int conversion turns
+    into code 0; the oracle states that explicitly.  Does not mutate ``data``.
+    """
+    B, nh, D, T = data.shape
+    assert data.dtype == torch.float16 and T % group_size == 0
+    qmax = 2 ** bit - 1
+    g = data.reshape(B * nh * D, T // group_size, group_size).clone()
+    mn = g.min(dim=-1, keepdim=True)[0]
+    mx = g.max(dim=-1, keepdim=True)[0]
+    scale = _div_scalar_fp16(mx - mn, qmax, scalar_div)
+    v = (g - mn) / scale                      # fp16 subtract, fp16 divide (each rounded once)
+    v = v.clamp(0, qmax).round()
+    v = torch.nan_to_num(v, nan=0.0)
+    q = v.to(torch.int32).reshape(B, nh, D, T)
+    code = pack_along_last_dim(q, bit)
+    shp = (B, nh, D, T // group_size)
+    return code, scale.reshape(shp), mn.reshape(shp)
+
+
+def uniform_group_dequantize_unpack_last_dim(
+    code: torch.Tensor, scale: torch.Tensor, mn: torch.Tensor, group_size: int, bit: int
+) -> torch.Tensor:
+    """x = rnd16(rnd16(fp16(c) * scale) + mn); quant/pack_unpack.py:316-333."""
+    B, nh, D, Td = code.shape
+    T = Td * (32 // bit)
+    x = unpack_along_last_dim(code, bit).reshape(B, nh, D, T // group_size, group_size)
+    x = x * scale.unsqueeze(-1)
+    x = x + mn.unsqueeze(-1)
+    return x.reshape(B, nh, D, T)
+
+
+def uniform_group_fake_quant(data: torch.Tensor, group_size: int, bit: int, scalar_div: str = "recip"):
+    """quant/pack_unpack.py:134-154 (quantise then dequantise without packing)."""
+    if bit == 0:
+        return 0
+    code, s, z = uniform_group_quantize_pack_last_dim(data, group_size, bit, scalar_div)
+    return uniform_group_dequantize_unpack_last_dim(code, s, z, group_size, bit)
+
+
+# --------------------------------------------------------------------------- GEMV
+
+
+def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """(B, Hkv, a, b) -> (B, Hkv*n_rep, a, b), each KV head repeated n_rep times in place.
+
+    transformers' ``repeat_kv`` as used at quant/quant_matmul_hq.py:19,81.
+    """
+    if n_rep == 1:
+        return x
+    B, H, a, b = x.shape
+    return x[:, :, None].expand(B, H, n_rep, a, b).reshape(B, H * n_rep, a, b)
+
+
+def gemv_uniform_group(group_size, fA, qB, scales, zeros, bits) -> torch.Tensor:
+    """C[b,hq,m,n] = sum_k fA[b,hq,m,k] * dq(qB)[b,hq//n_rep,k,n], fp32 accumulate, fp16 out.
+
+    The reference's definition of a correct ``cuda_bmm_fA_qB_uniform_group``
+    (quant/matmul.py:263-299): dequantise with the library's own unpack, ``repeat_kv``,
+    ``torch.matmul`` (quant/cuda_hq_test.py:82,242; quant/matmul.py:819-832).
+    """
+    n_rep = fA.shape[1] // qB.shape[1]
+    dq = uniform_group_dequantize_unpack_last_dim(qB, scales, zeros, group_size, bits)
+    return torch.matmul(fA.float(), repeat_kv(dq, n_rep).float()).to(torch.float16)
+
+
+# --------------------------------------------------------------------------- hybrid attention
+
+# slot bases of the 42-field cache tuple (quant/quant_matmul_hq.py:34-38)
+K16, K16_IDX, V16, V16_IDX = 0, 1, 2, 3
+K_BASE = {8: 4, 4: 12, 2: 20, 1: 28}
+V_BASE = {8: 8, 4: 16, 2: 24, 1: 32}
+V_TOKEN_NORM, NEW_K, NEW_V, KV_SEQ_LEN = 38, 39, 40, 41
+
+
+def empty_cache(new_K=None, new_V=None, kv_seq_len=0) -> tuple:
+    """``(None,)*39 + (K, V, len)`` -- the cache right after prefill (model/llama_hqe.py:186)."""
+    return (None,) * 39 + (new_K, new_V, kv_seq_len)
+
+
+def _scale_clamp_softmax(w: torch.Tensor, head_dim: int, mask, scalar_div: str) -> torch.Tensor:
+    """quant/quant_matmul_hq.py:100-103: ``/= sqrt(D)`` (fp16), ``+= mask`` (fp16),
+    ``max(., finfo.min)``, fp32 softmax, round to fp16."""
+    if scalar_div == "recip":
+        inv = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(head_dim ** 0.5, dtype=torch.float32)
+        w = (w.float() * inv).to(torch.float16)
+    else:
+        w = (w.float() / (head_dim ** 0.5)).to(torch.float16)
+    if mask is not None:
+        w = w + mask
+    w = torch.max(w, torch.tensor(torch.finfo(torch.float16).min, dtype=torch.float16))
+    return torch.softmax(w.float(), dim=-1).to(torch.float16)
+
+
+def qkv_matmul(
+    q: torch.Tensor,
+    past_key_value: tuple,
+    attention_mask,
+    head_dim: int,
+    quant_strategy: str = "uniform_group",
+    block_size: int = 32,
+    group_size: int = 32,
+    *,
+    use_mask: bool = True,
+    scalar_div: str = "recip",
+    round_per_class: bool = True,
+):
+    """Hybrid decode attention over the 42-tuple: quant/quant_matmul_hq.py:23-120 and
+    quant/hqe_matmul.py:354-451 (``use_mask=False`` restates the latter, which skips the mask).
+
+    ``round_per_class=True`` keeps the reference's ``attn_output +=`` in fp16 after every
+    class; ``False`` accumulates every class in fp32 and rounds once (what a fused kernel does).
+    Only the uniform classes (16/8/4/2) are restated; a populated 1-bit class raises.
+    """
+    if quant_strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
+        raise ValueError("invalid quant_strategy")
+    pkv = past_key_value
+    if pkv[K_BASE[1]] is not None or pkv[V_BASE[1]] is not None:
+        raise NotImplementedError("1-bit normal-quantile class is outside the oracle")
+    new_K, new_V = pkv[NEW_K], pkv[NEW_V]
+    B, Hq, _, D = q.shape
+    real_len = 0
+    nh_kv = None
+    if pkv[V16] is not None:
+        nh_kv = pkv[V16].shape[1]
+        real_len += pkv[V16].shape[2]
+    for b in BITS:
+        v = pkv[V_BASE[b]]
+        if v is not None:
+            nh_kv = v.shape[1]
+            real_len += v.shape[2]
+    new_len = 0
+    if new_V is not None:
+        nh_kv = new_V.shape[1]
+        new_len = new_V.shape[2]
+        real_len += new_len
+    if real_len == 0:
+        raise ValueError("invalid past_key_value")
+    n_rep = Hq // nh_kv
+    w = torch.zeros(B, Hq, 1, real_len, dtype=torch.float16)
+    if pkv[K16] is not None:
+        w[..., pkv[K16_IDX]] = torch.matmul(q.float(), repeat_kv(pkv[K16], n_rep).float()).half()
+    for b in BITS:
+        base = K_BASE[b]
+        if pkv[base] is not None:
+            w[..., pkv[base + 1]] = gemv_uniform_group(block_size, q, pkv[base], pkv[base + 2], pkv[base + 3], b)
+    if new_K is not None:
+        w[..., real_len - new_len:] = torch.matmul(
+            q.float(), repeat_kv(new_K, n_rep).transpose(2, 3).float()).half()
+    w = _scale_clamp_softmax(w, head_dim, attention_mask if use_mask else None, scalar_div)
+
+    acc32 = torch.zeros(B, Hq, 1, D, dtype=torch.float32)
+    acc16 = torch.zeros(B, Hq, 1, D, dtype=torch.float16)
+
+    def _add(part32):
+        nonlocal acc32, acc16
+        acc32 = acc32 + part32
+        acc16 = acc16 + part32.half()
+
+    if pkv[V16] is not None:
+        _add(torch.matmul(w[..., pkv[V16_IDX]].float(), repeat_kv(pkv[V16], n_rep).float()))
+    for b in BITS:
+        base = V_BASE[b]
+        if pkv[base] is not None:
+            dq = uniform_group_dequantize_unpack_last_dim(pkv[base], pkv[base + 2], pkv[base + 3], group_size, b)
+            _add(torch.matmul(w[..., pkv[base + 1]].float(), repeat_kv(dq, n_rep).float()))
+    if new_V is not None:
+        _add(torch.matmul(w[..., real_len - new_len:].float(), repeat_kv(new_V, n_rep).float()))
+    out = acc16 if round_per_class else acc32.half()
+    return w, out
+
+
+# --------------------------------------------------------------------------- policy helpers
+
+
+def calculate_token_range(new_cache: Optional[torch.Tensor], token_range: Optional[torch.Tensor]):
+    """Per-token sum over (batch, head) of max_d - min_d, appended to the running vector.
+    model/public_func.py:58-73."""
+    if new_cache is None:
+        return None
+    r = (new_cache.max(dim=-1)[0] - new_cache.min(dim=-1)[0]).sum(0).sum(0)
+    return r if token_range is None else torch.cat((token_range, r), dim=-1)
+
+
+def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tensor) -> torch.Tensor:
+    """Token indices of 32-token blocks ordered by descending mean importance.
+    model/public_func.py:92-106 (the in-place divide of the caller's tensor is not reproduced)."""
+    bi = importance.reshape(block_num, -1)
+    bi = (bi / bi.shape[1]).sum(dim=-1)
+    _, order = torch.sort(bi, descending=True, stable=True)
+    return (order.reshape(-1, 1) * block_size + torch.arange(block_size, dtype=order.dtype)).flatten()
+
+
+def make_sum_equal(array: torch.Tensor, array_sum: int, start_idx: int = 4) -> torch.Tensor:
+    """Repair rounded block counts so they sum to ``array_sum`` (model/public_func.py:259-268):
+    the surplus is taken from index ``start_idx`` walking down; a deficit is added to it."""
+    a = array.clone()
+    sub = int(a.sum()) - int(array_sum)
+    for i in range(start_idx, -1, -1):
+        if int(a[i]) - sub < 0:
+            sub -= int(a[i])
+            a[i] = 0
+        else:
+            a[i] -= sub
+            break
+    return a
+
+
+def rerank_after_eviction(idx_per_class: Sequence[Optional[torch.Tensor]]) -> List[Optional[torch.Tensor]]:
+    """Replace every surviving position by its rank among all survivors (quant/hqe_2.py:661-670).
+    Written with a Python dict instead of the reference's all-pairs compare."""
+    alive = sorted(int(v) for t in idx_per_class if t is not None for v in t.tolist())
+    rank = {v: r for r, v in enumerate(alive)}
+    out = []
+    for t in idx_per_class:
+        out.append(None if t is None else torch.tensor([rank[int(v)] for v in t.tolist()], dtype=torch.int64))
+    return out

@@ -1,0 +1,142 @@
+"""Hybrid decode attention (all precision classes in one launch, evicted tokens absent) against the
+CPU oracle.  Probabilities and outputs: 1e-3 relative + 2e-3 absolute with fp32 accumulation."""
+import pytest
+import torch
+
+from hqekv_amd import synth
+from oracle import hqe_oracle as O
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-3, 2e-3
+
+
+def _close(a, b, what=""):
+    torch.testing.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, msg=lambda m: f"{what}: {m}")
+
+
+def _case(B, Hq, Hkv, T, D, fractions, residual, seed, permute=False):
+    q, K, V = synth.make_qkv(B, Hq, Hkv, T, D, seed)
+    classes = synth.split_blocks(T - residual, fractions, seed)
+    override = None
+    if permute:  # arbitrary int64 positions, as the reference's kernel scripts feed (quant/cuda_hq_test.py:21-22)
+        pos, kept = synth.survivor_positions(classes, T - residual)
+        perm = torch.randperm(kept, generator=torch.Generator().manual_seed(seed))
+        override, start = {}, 0
+        for b, p in pos.items():
+            override[b] = perm[start:start + p.numel()]
+            start += p.numel()
+    cache = synth.build_cache(K, V, classes, residual, O.uniform_group_quantize_pack_last_dim, override)
+    return q, cache
+
+
+CASES = [
+    dict(B=1, Hq=8, Hkv=2, T=1024, D=128, fractions=(0.1, 0.2, 0.3, 0.3, 0.1), residual=0, seed=1),
+    dict(B=2, Hq=8, Hkv=2, T=2048 + 17, D=128, fractions=(0.05, 0.15, 0.3, 0.3, 0.2), residual=17, seed=2),
+    dict(B=1, Hq=32, Hkv=8, T=4096, D=128, fractions=(0.0, 0.0, 0.0, 1.0, 0.0), residual=128, seed=1235),  # config 1
+    dict(B=1, Hq=4, Hkv=4, T=512 + 31, D=128, fractions=(0.25, 0.0, 0.5, 0.0, 0.25), residual=31, seed=4),
+    dict(B=1, Hq=16, Hkv=2, T=1024, D=128, fractions=(0.0, 1.0, 0.0, 0.0, 0.0), residual=0, seed=5),
+    dict(B=1, Hq=8, Hkv=2, T=640 + 5, D=64, fractions=(0.1, 0.2, 0.3, 0.3, 0.1), residual=5, seed=6),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: f"B{c['B']}Hq{c['Hq']}T{c['T']}D{c['D']}s{c['seed']}")
+@pytest.mark.parametrize("permute", [False, True], ids=["blockidx", "randperm"])
+def test_hqe2_matches_oracle(dev, case, permute):
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    q, cache = _case(permute=permute, **case)
+    w_ref, o_ref = O.qkv_matmul(q, cache, None, case["D"], use_mask=False)
+    _, o_ref32 = O.qkv_matmul(q, cache, None, case["D"], use_mask=False, round_per_class=False)
+    w, o = qkv_matmul_hqe_2(q.to(dev), synth.cache_to(cache, dev), None, case["D"], "uniform_group")
+    assert w.shape == w_ref.shape and o.shape == o_ref.shape and w.dtype == torch.float16
+    _close(w, w_ref, "attn_weights")
+    _close(o, o_ref, "attn_output vs per-class fp16 accumulation")
+    _close(o, o_ref32, "attn_output vs fp32 accumulation")
+    # the probabilities of every (b, h) row sum to one
+    torch.testing.assert_close(w.float().sum(-1).cpu(), torch.ones(case["B"], case["Hq"], 1), rtol=0, atol=5e-3)
+
+
+def test_qkv_matmul_with_mask(dev):
+    from hqekv_amd.quant_matmul_hq import qkv_matmul, qkv_matmul_hq
+    case = CASES[1]
+    q, cache = _case(**case)
+    Tall = cache[41]
+    g = torch.Generator().manual_seed(3)
+    mask = torch.zeros(case["B"], 1, 1, Tall, dtype=torch.float16)
+    mask[..., torch.randperm(Tall, generator=g)[:Tall // 4]] = torch.finfo(torch.float16).min
+    w_ref, o_ref = O.qkv_matmul(q, cache, mask, case["D"])
+    for fn in (qkv_matmul, qkv_matmul_hq):
+        w, o = fn(q.to(dev), synth.cache_to(cache, dev), mask.to(dev), case["D"], "uniform_group")
+        _close(w, w_ref, "attn_weights")
+        _close(o, o_ref, "attn_output")
+        assert (w.cpu()[mask.expand_as(w_ref) < 0] == 0).all()
+    w0, o0 = qkv_matmul(q.to(dev), synth.cache_to(cache, dev), 0, case["D"], "uniform_group")
+    w_ref0, o_ref0 = O.qkv_matmul(q, cache, None, case["D"])
+    _close(w0, w_ref0)
+    _close(o0, o_ref0)
+
+
+def test_fused_wrappers_match_oracle(dev):
+    """cuda_bmm_forward_qk_group_hq / wv_group_hq with shuffled idx, the shape of quant/cuda_hq_test.py."""
+    from hqekv_amd.matmul import cuda_bmm_forward_qk_group_hq, cuda_bmm_forward_wv_group_hq
+    case = dict(B=1, Hq=32, Hkv=8, T=2048 + 95, D=128, fractions=(0.05, 0.0, 0.15, 0.8, 0.0), residual=95, seed=9)
+    q, cache = _case(permute=True, **case)
+    c = synth.cache_to(cache, dev)
+    Tall = cache[41]
+    scores = cuda_bmm_forward_qk_group_hq(32, 8, q.to(dev), c[0], c[1], c[4], c[5], c[6], c[7], c[12], c[13], c[14],
+                                          c[15], c[20], c[21], c[22], c[23], None, None, None, None, c[39])
+    # reference definition: dequantise everything, place by idx, matmul
+    D = case["D"]
+    dqK = torch.zeros(1, 8, Tall, D, dtype=torch.float16)
+    dqK[:, :, cache[1]] = cache[0].transpose(2, 3)
+    for b, base in ((4, 12), (2, 20)):
+        dq = O.uniform_group_dequantize_unpack_last_dim(cache[base], cache[base + 2], cache[base + 3], 32, b)
+        dqK[:, :, cache[base + 1]] = dq.transpose(2, 3)
+    dqK[:, :, Tall - 95:] = cache[39]
+    ref = torch.matmul(q.float(), O.repeat_kv(dqK, 4).transpose(2, 3).float())
+    torch.testing.assert_close(scores.float().cpu(), ref, rtol=2e-3, atol=2e-2)  # raw scores are O(50)
+
+    p = torch.softmax(torch.randn(1, 32, 1, Tall, generator=torch.Generator().manual_seed(1)) * 2, -1).half()
+    out = cuda_bmm_forward_wv_group_hq(32, 8, p.to(dev), c[2], c[3], c[8], c[9], c[10], c[11], c[16], c[17], c[18],
+                                       c[19], c[24], c[25], c[26], c[27], None, None, None, None, c[40])
+    dqV = torch.zeros(1, 8, Tall, D, dtype=torch.float16)
+    dqV[:, :, cache[3]] = cache[2]
+    for b, base in ((4, 16), (2, 24)):
+        dqV[:, :, cache[base + 1]] = O.uniform_group_dequantize_unpack_last_dim(
+            cache[base], cache[base + 2], cache[base + 3], 32, b)
+    dqV[:, :, Tall - 95:] = cache[40]
+    ref = torch.matmul(p.float(), O.repeat_kv(dqV, 4).float())
+    _close(out, ref, "attn_output")
+
+
+def test_all_fp16_equals_dense_attention(dev):
+    """Permutation invariance: with every class at fp16 and tokens shuffled between positions, the
+    result must equal dense attention over the permuted sequence."""
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    q, K, V = synth.make_qkv(1, 8, 2, 512, 128, 77)
+    perm = torch.randperm(480, generator=torch.Generator().manual_seed(5))
+    t = [None] * 42
+    t[0], t[1] = K[:, :, :480].transpose(2, 3).contiguous(), perm
+    t[2], t[3] = V[:, :, :480].contiguous(), perm.clone()
+    t[39], t[40], t[41] = K[:, :, 480:].contiguous(), V[:, :, 480:].contiguous(), 512
+    w, o = qkv_matmul_hqe_2(q.to(dev), synth.cache_to(tuple(t), dev), None, 128, "uniform_group")
+    Kp, Vp = K.clone(), V.clone()
+    Kp[:, :, perm], Vp[:, :, perm] = K[:, :, :480], V[:, :, :480]
+    s = torch.matmul(q.float(), O.repeat_kv(Kp, 4).transpose(2, 3).float()).half()
+    s = (s.float() * (1.0 / 128 ** 0.5)).half()
+    pr = torch.softmax(s.float(), -1).half()
+    _close(w, pr)
+    _close(o, torch.matmul(pr.float(), O.repeat_kv(Vp, 4).float()))
+
+
+def test_errors(dev):
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    from hqekv_amd.quant_matmul_hq import qkv_matmul
+    q = torch.zeros(1, 4, 1, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError, match="invalid past_key_value"):
+        qkv_matmul_hqe_2(q, (None,) * 41 + (0,), None, 128, "uniform_group")
+    with pytest.raises(ValueError, match="invalid quant_strategy"):
+        qkv_matmul_hqe_2(q, (None,) * 41 + (0,), None, 128, "bogus")
+    with pytest.raises(ValueError, match="invalid quant_strategy"):
+        qkv_matmul(q, (None,) * 41 + (0,), None, 128, "bogus")
+    with pytest.raises(ValueError, match="invalid past_key_value"):
+        qkv_matmul(q, (None,) * 41 + (0,), None, 128, "uniform_group")

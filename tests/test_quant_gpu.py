@@ -1,0 +1,150 @@
+"""HIP quantise/pack/unpack kernels against the CPU oracle: bit-exact codes, scales and zeros."""
+import pytest
+import torch
+
+from oracle import hqe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _data(shape, seed, outliers=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(*shape, generator=g)
+    if outliers:
+        x[..., 3::32, :] *= 10.0
+    return x.half()
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_quant_rows_bit_exact(dev, bit):
+    from hqekv_amd import pack_unpack as P
+    x = _data((2, 3, 96, 256), 10 + bit)
+    code, scale, mn = P.uniform_group_quantize_pack_last_dim(x.to(dev), 32, bit)
+    oc, os_, om = O.uniform_group_quantize_pack_last_dim(x, 32, bit)
+    assert code.dtype == torch.int32 and scale.dtype == torch.float16
+    assert torch.equal(code.cpu(), oc)
+    assert torch.equal(scale.cpu().view(torch.int16), os_.view(torch.int16))
+    assert torch.equal(mn.cpu().view(torch.int16), om.view(torch.int16))
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_quant_k_transposed_view_bit_exact(dev, bit):
+    """K reaches the quantiser as the transpose(2, 3) view of token-major memory (quant/hqe_2.py:32-35)."""
+    from hqekv_amd import pack_unpack as P
+    k = _data((2, 2, 160, 128), 20 + bit, outliers=False)  # (B, H, T, D)
+    k[..., 5] *= 10.0
+    kd = k.to(dev)
+    before = kd.clone()
+    code, scale, mn = P.uniform_group_quantize_pack_last_dim(kd.transpose(2, 3), 32, bit)
+    assert torch.equal(kd, before), "the input must not be modified"
+    oc, os_, om = O.uniform_group_quantize_pack_last_dim(k.transpose(2, 3).contiguous(), 32, bit)
+    assert torch.equal(code.cpu(), oc)
+    assert torch.equal(scale.cpu().view(torch.int16), os_.view(torch.int16))
+    assert torch.equal(mn.cpu().view(torch.int16), om.view(torch.int16))
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_quant_matches_torch_chain_on_device(dev, bit):
+    """The reference's own torch op chain (quant/pack_unpack.py:166-175) evaluated ON THE GPU, which pins
+    the tensor / python-int rule and the fp32 divide of the device against the HIP kernel."""
+    from hqekv_amd import pack_unpack as P
+    x = _data((1, 8, 128, 1024), 30 + bit).to(dev)
+    code, scale, mn = P.uniform_group_quantize_pack_last_dim(x, 32, bit)
+    g = x.reshape(8 * 128, 1024 // 32, 32).clone()
+    t_mn = torch.min(g, dim=-1, keepdim=True)[0]
+    t_mx = torch.max(g, dim=-1, keepdim=True)[0]
+    t_scale = (t_mx - t_mn) / (2 ** bit - 1)
+    g.sub_(t_mn)
+    g.div_(t_scale)
+    q = g.clamp_(0, 2 ** bit - 1).round_().to(torch.int32).view(1, 8, 128, 1024)
+    assert torch.equal(scale.reshape(-1), t_scale.reshape(-1))
+    assert torch.equal(mn.reshape(-1), t_mn.reshape(-1))
+    assert torch.equal(code.cpu(), O.pack_along_last_dim(q.cpu(), bit))
+
+
+def test_quant_degenerate_and_extreme_groups(dev):
+    from hqekv_amd import pack_unpack as P
+    x = torch.zeros(1, 1, 4, 64, dtype=torch.float16)
+    x[0, 0, 0, :32] = 1.5                      # constant group -> scale 0, codes 0
+    x[0, 0, 1, :] = torch.linspace(-60000, 60000, 64).half()
+    x[0, 0, 2, 0] = 6e-8                       # denormal range
+    x[0, 0, 3, :] = torch.arange(64).half() / 1024
+    for bit in (2, 4, 8):
+        code, scale, mn = P.uniform_group_quantize_pack_last_dim(x.to(dev), 32, bit)
+        oc, os_, om = O.uniform_group_quantize_pack_last_dim(x, 32, bit)
+        assert torch.equal(code.cpu(), oc), bit
+        assert torch.equal(scale.cpu().view(torch.int16), os_.view(torch.int16)), bit
+        assert torch.equal(mn.cpu().view(torch.int16), om.view(torch.int16)), bit
+        dq = P.uniform_group_dequantize_unpack_last_dim(code, scale, mn, 32, bit)
+        assert torch.equal(dq.cpu()[0, 0, 0, :32], x[0, 0, 0, :32])
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_dequant_and_unpack_bit_exact(dev, bit):
+    from hqekv_amd import pack_unpack as P
+    x = _data((1, 2, 64, 512), 40 + bit)
+    oc, os_, om = O.uniform_group_quantize_pack_last_dim(x, 32, bit)
+    dq = P.uniform_group_dequantize_unpack_last_dim(oc.to(dev), os_.to(dev), om.to(dev), 32, bit)
+    ref = O.uniform_group_dequantize_unpack_last_dim(oc, os_, om, 32, bit)
+    assert torch.equal(dq.cpu().view(torch.int16), ref.view(torch.int16))
+    un = P.unpack_along_last_dim(oc.to(dev), bit)
+    assert torch.equal(un.cpu(), O.unpack_along_last_dim(oc, bit))
+    fq = P.uniform_group_fake_quant(x.to(dev), 32, bit)
+    assert torch.equal(fq.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_pack_roundtrip(dev, bit):
+    from hqekv_amd import pack_unpack as P
+    g = torch.Generator().manual_seed(bit)
+    q = torch.randint(0, 2 ** bit, (2, 2, 16, 128), generator=g, dtype=torch.int32)
+    code = P.pack_along_last_dim(q.to(dev), bit)
+    assert torch.equal(code.cpu(), O.pack_along_last_dim(q, bit))
+    assert torch.equal(P.unpack_along_last_dim(code, bit).cpu().to(torch.int32), q)
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_append_into_capacity_window(dev, bit):
+    """Quantise new tokens straight into a window of capacity-sized cache buffers: the bytes written
+    equal a stand-alone quantisation and nothing outside the window changes."""
+    from hqekv_amd import pack_unpack as P
+    pf = 32 // bit
+    B, H, D, cap, old, new = 1, 2, 128, 512, 192, 128
+    k_new = _data((B, H, new, D), 50 + bit, outliers=False)
+    code = torch.full((B, H, D, cap // pf), -1, dtype=torch.int32, device=dev)
+    scale = torch.full((B, H, D, cap // 32), -1.0, dtype=torch.float16, device=dev)
+    mn = torch.full_like(scale, -1.0)
+    P.quantize_pack_into(k_new.to(dev).transpose(2, 3), bit,
+                         code[..., old // pf:(old + new) // pf], scale[..., old // 32:(old + new) // 32],
+                         mn[..., old // 32:(old + new) // 32])
+    oc, os_, om = O.uniform_group_quantize_pack_last_dim(k_new.transpose(2, 3).contiguous(), 32, bit)
+    assert torch.equal(code[..., old // pf:(old + new) // pf].cpu(), oc)
+    assert torch.equal(scale[..., old // 32:(old + new) // 32].cpu(), os_)
+    assert torch.equal(mn[..., old // 32:(old + new) // 32].cpu(), om)
+    assert (code[..., :old // pf] == -1).all() and (code[..., (old + new) // pf:] == -1).all()
+    assert (scale[..., :old // 32] == -1).all() and (scale[..., (old + new) // 32:] == -1).all()
+    # V: token rows appended into (B, H, cap, D/pf)
+    v_new = _data((B, H, new, D), 60 + bit, outliers=False)
+    vcode = torch.full((B, H, cap, D // pf), -1, dtype=torch.int32, device=dev)
+    vs = torch.full((B, H, cap, D // 32), -1.0, dtype=torch.float16, device=dev)
+    vz = torch.full_like(vs, -1.0)
+    P.quantize_pack_into(v_new.to(dev), bit, vcode[:, :, old:old + new], vs[:, :, old:old + new], vz[:, :, old:old + new])
+    oc, os_, om = O.uniform_group_quantize_pack_last_dim(v_new, 32, bit)
+    assert torch.equal(vcode[:, :, old:old + new].cpu(), oc)
+    assert torch.equal(vs[:, :, old:old + new].cpu(), os_) and torch.equal(vz[:, :, old:old + new].cpu(), om)
+    assert (vcode[:, :, :old] == -1).all() and (vcode[:, :, old + new:] == -1).all()
+
+
+def test_argument_errors(dev):
+    from hqekv_amd import pack_unpack as P
+    x = torch.zeros(1, 1, 2, 64, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        P.uniform_group_quantize_pack_last_dim(x, 32, 3)
+    with pytest.raises(ValueError):
+        P.uniform_group_quantize_pack_last_dim(x, 64, 2)
+    with pytest.raises(ValueError):
+        P.uniform_group_quantize_pack_last_dim(x[..., :48], 32, 2)
+    with pytest.raises(TypeError):
+        P.uniform_group_quantize_pack_last_dim(x.float(), 32, 2)
+    with pytest.raises(RuntimeError):
+        P.uniform_group_quantize_pack_last_dim(x.cpu(), 32, 2)
