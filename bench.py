@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Decode-attention benchmark over the hybrid quantized KV cache (one MI355X).
+
+A step is ONE decode-attention layer-step (q.K^T over every precision class, scale+softmax, p.V over
+every class, split-K combine) on one layer's cache.  Steps cycle through ``--layers`` distinct layer
+caches (default 32, like the 32 decoder layers of Llama-3.1-8B) so no step finds its cache in L2 or in
+the 256 MB Infinity Cache.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line: metric/value are microseconds per layer-step; ``roofline`` prices the dominant
+kernel's algorithmic bytes against the 8 TB/s HBM peak using its average duration measured live with
+HIP events; ``cpu_baseline`` times the CPU restatement of the reference's unpack + dequant +
+torch.matmul path on the same layer-0 inputs on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "us/layer decode-attn & achieved HBM GB/s (% of peak) at 32k ctx, 1 GPU"
+
+WORKLOADS = {
+    "c1": "Llama-3.1-8B shape, B=1, ctx 4096: 3968 tokens 2-bit + 128 fp16 residual",
+    "c2": "Llama-3.1-8B shape, B=1, ctx 32768 hybrid: fp16 5% / 8-bit 15% / 4-bit 30% / 2-bit 30% / evicted 20%",
+    "c4": "Qwen3-8B shape, B=8, ctx 65536 hybrid: fp16 10% / 4-bit 20% / 2-bit 50% / evicted 20%",
+}
+
+
+def side_bytes(pkv, k_side: bool) -> int:
+    """Algorithmic bytes of the K side (q.K^T launch) or V side (p.V launch) of one layer-step."""
+    if k_side:
+        slots = (0, 1, 4, 5, 6, 7, 12, 13, 14, 15, 20, 21, 22, 23, 39)
+    else:
+        slots = (2, 3, 8, 9, 10, 11, 16, 17, 18, 19, 24, 25, 26, 27, 40)
+    return sum(pkv[i].numel() * pkv[i].element_size() for i in slots if torch.is_tensor(pkv[i]))
+
+
+def build_layers(name: str, n_layers: int, dev):
+    from hqekv_amd import synth
+    from hqekv_amd.pack_unpack import uniform_group_quantize_pack_last_dim as hip_quant
+    cfg = synth.CONFIGS[name]
+    layers = []
+    q0 = cpu_cache = None
+    for l in range(n_layers):
+        if l == 0:
+            # layer 0 is the CPU-seeded configuration, also handed to the CPU baseline
+            q, K, V = synth.make_qkv(cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["T"], cfg["D"], cfg["seed"])
+            q, K, V = q.to(dev), K.to(dev), V.to(dev)
+        else:
+            g = torch.Generator(device=dev).manual_seed(cfg["seed"] + 1000 * l)
+            K = torch.randn(cfg["B"], cfg["Hkv"], cfg["T"], cfg["D"], generator=g, device=dev)
+            V = torch.randn(cfg["B"], cfg["Hkv"], cfg["T"], cfg["D"], generator=g, device=dev).half()
+            for c in synth.OUTLIER_CHANNELS:
+                K[..., c] *= 10.0
+            K = K.half()
+            q = torch.randn(cfg["B"], cfg["Hq"], 1, cfg["D"], generator=g, device=dev).half()
+        classes = synth.split_blocks(cfg["T"] - cfg["residual"], cfg["fractions"], cfg["seed"] + 1000 * l)
+        cache = synth.build_cache(K, V, classes, cfg["residual"], hip_quant)
+        layers.append((q, cache))
+        del K, V
+    return layers
+
+
+def time_region(fn, sync):
+    sync()
+    t0 = time.perf_counter()
+    fn()
+    sync()
+    return time.perf_counter() - t0
+
+
+def event_avg_us(launch, n_launches: int, reps: int) -> float:
+    """Average duration of one launch: HIP events on the launch stream around back-to-back launches."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = []
+    for _ in range(reps):
+        e0.record()
+        launch()
+        e1.record()
+        e1.synchronize()
+        best.append(e0.elapsed_time(e1) * 1e3 / n_launches)
+    return statistics.median(best)
+
+
+def cpu_baseline(name: str, n_iter: int = 5):
+    """The reference's CPU-expressible path (unpack + dequant + torch.matmul) on layer 0."""
+    from hqekv_amd import synth
+    from oracle import hqe_oracle as O
+    cores = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(cores)
+    cfg = synth.CONFIGS[name]
+    B = cfg["B"]
+    sample = "one layer-step, all batch rows"
+    scale = 1.0
+    if name == "c4":  # bounded sample: one batch row, scaled by B
+        cfg = dict(cfg, B=1)
+        sample = f"one layer-step of ONE batch row, time x{B}"
+        scale = float(B)
+    q, K, V = synth.make_qkv(cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["T"], cfg["D"], cfg["seed"])
+    classes = synth.split_blocks(cfg["T"] - cfg["residual"], cfg["fractions"], cfg["seed"])
+    cache = synth.build_cache(K, V, classes, cfg["residual"], O.uniform_group_quantize_pack_last_dim)
+    times = []
+    ref = None
+    for i in range(n_iter + 1):
+        t0 = time.perf_counter()
+        ref = O.qkv_matmul(q, cache, None, cfg["D"], use_mask=False)
+        if i:
+            times.append(time.perf_counter() - t0)
+    return dict(value=statistics.median(times) * 1e6 * scale, unit="us/layer", cores=cores, kind="port",
+                sample=f"{sample}; median of {n_iter} after 1 warm-up; torch {torch.__version__} CPU ops"), (q, cache, ref)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=640)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--layers", type=int, default=None, help="distinct layer caches cycled through")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs the decode-attention path on ONE GPU; --gpus {args.gpus} is not "
+              "supported (no collectives or sharding are part of this path)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+
+    from hqekv_amd import synth
+    from hqekv_amd.attention import DecodePlan
+
+    dev = torch.device("cuda:0")
+    n_layers = args.layers or {"c1": 64, "c2": 32, "c4": 4}[args.workload]
+    layers = build_layers(args.workload, n_layers, dev)
+    plans = [DecodePlan(q, cache) for q, cache in layers]
+    qs = [q.contiguous() for q, _ in layers]
+    cfg = synth.CONFIGS[args.workload]
+    pkv0 = layers[0][1]
+    alg_bytes = synth.algorithmic_bytes(pkv0, cfg["Hq"])
+    k_bytes, v_bytes = side_bytes(pkv0, True), side_bytes(pkv0, False)
+
+    def step(i):
+        plans[i % n_layers].run(qs[i % n_layers])
+
+    sync = torch.cuda.synchronize
+    for i in range(args.warmup):
+        step(i)
+    sync()
+
+    K = args.steps
+    rounds, rem = divmod(K, n_layers)
+    graph = None
+    if not args.no_graph and rounds > 0:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(n_layers):
+                step(i)
+        graph.replay()
+        sync()
+
+    def timed():
+        if graph is not None:
+            for _ in range(rounds):
+                graph.replay()
+            for i in range(rem):
+                step(i)
+        else:
+            for i in range(K):
+                step(i)
+
+    elapsed = time_region(timed, sync)
+    us_per_step = elapsed / K * 1e6
+
+    # per-kernel averages (HIP events on the launch stream), back-to-back over all layers
+    reps = 5
+    qk_us = event_avg_us(lambda: [p.run_qk(q) for p, q in zip(plans, qs)], n_layers, reps)
+    sm_us = event_avg_us(lambda: [p.run_softmax() for p in plans], n_layers, reps)
+    for p, q in zip(plans, qs):  # leave valid probabilities behind for the p.V timing
+        p.run(q)
+    pv_us = event_avg_us(lambda: [p.run_pv() for p in plans], n_layers, reps)
+    dominant = "qk_hybrid_kernel" if qk_us >= pv_us else "pv_hybrid_kernel"
+    dom_us, dom_bytes = (qk_us, k_bytes) if qk_us >= pv_us else (pv_us, v_bytes)
+    achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(args.workload, {}).get(dominant)
+        except Exception:
+            traffic = None
+
+    out = {
+        "metric": METRIC,
+        "value": round(us_per_step, 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_per_step / 1e3, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {WORKLOADS[args.workload]}", "B": cfg["B"], "Hq": cfg["Hq"],
+                   "Hkv": cfg["Hkv"], "head_dim": cfg["D"], "context": cfg["T"], "kept_tokens": pkv0[41],
+                   "layers_cycled": n_layers, "launch": "eager" if graph is None else "hip-graph replay",
+                   "algorithmic_bytes_per_step": alg_bytes},
+        "achieved_GBps": round(alg_bytes / (us_per_step * 1e-6) / 1e9, 1),
+        "pct_of_hbm_peak": round(alg_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS * 100, 2),
+        "kernels_us": {"qk_hybrid_kernel": round(qk_us, 3), "scale_softmax_kernel": round(sm_us, 3),
+                       "pv_hybrid_kernel+combine": round(pv_us, 3)},
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "bytes_per_launch": dom_bytes, "avg_us": round(dom_us, 3)},
+    }
+
+    if not args.no_cpu:
+        base, (q_cpu, cache_cpu, ref) = cpu_baseline(args.workload)
+        out["cpu_baseline"] = base
+        # parity of layer 0 against the oracle on the same seeded inputs (c4: first batch row)
+        w, o = plans[0].run(qs[0])
+        sync()
+        if q_cpu.shape[0] == cfg["B"]:
+            out["parity_layer0"] = {
+                "attn_weights_max_abs": float((w.float().cpu() - ref[0].float()).abs().max()),
+                "attn_output_max_abs": float((o.float().cpu() - ref[1].float()).abs().max()),
+            }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -187,3 +187,59 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
             _lib.stream_ptr(dev))
     _lib.check(rc, "decode_attention")
     return weights, out
+
+
+class DecodePlan:
+    """Pre-validated launch plan for one layer's cache: segment tables, outputs and the split-K
+    workspace are built once, so a decode step is a single C call (three kernel launches plus the
+    combine) with no per-step Python work.  Holds references to every tensor it points into.
+    """
+
+    def __init__(self, q_like: torch.Tensor, pkv: tuple, mask=None, Tall: Optional[int] = None):
+        _lib.require_gpu(q_like, "q")
+        B, Hq, _, D = q_like.shape
+        self.dev = q_like.device
+        self.Tall = int(Tall) if Tall is not None else value_length(pkv)
+        self._keep: list = []
+        k_items, hk, _ = key_segments(pkv, self.dev, self.Tall, self._keep)
+        v_items, hv, _ = value_segments(pkv, self.dev, self.Tall, self._keep)
+        self.Hkv = hk if hk is not None else hv
+        if self.Hkv is None:
+            raise ValueError("invalid past_key_value")
+        self.B, self.Hq, self.D = B, Hq, D
+        self.n_k, self.n_v = len(k_items), len(v_items)
+        self.k_segs, self.v_segs = _lib.make_segs(k_items), _lib.make_segs(v_items)
+        self.weights = torch.zeros(B, Hq, 1, self.Tall, dtype=torch.float16, device=self.dev)
+        self.out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=self.dev)
+        self.mask_ptr, self.mask_stride = _mask_arg(mask, B, Hq, self.Tall, self.dev, self._keep)
+        with torch.cuda.device(self.dev):
+            self.ws = workspace_for(self.v_segs, self.n_v, B, Hq, self.Hkv, D, self.dev)
+        self._lib = _lib.load()
+        self.inv_sqrt_d = 1.0 / (D ** 0.5)
+
+    def run(self, q: torch.Tensor, stream: Optional[int] = None):
+        st = _lib.stream_ptr(self.dev) if stream is None else stream
+        rc = self._lib.hqekv_decode_attn(
+            self.k_segs, self.n_k, self.v_segs, self.n_v, q.data_ptr(), self.mask_ptr, self.mask_stride,
+            self.weights.data_ptr(), self.out.data_ptr(), self.B, self.Hq, self.Hkv, self.D, self.Tall,
+            self.ws.data_ptr(), self.ws.numel() * 4, st)
+        if rc:
+            _lib.check(rc, "DecodePlan.run")
+        return self.weights, self.out
+
+    # the three stages on their own, for per-kernel timing
+    def run_qk(self, q: torch.Tensor, stream: Optional[int] = None):
+        st = _lib.stream_ptr(self.dev) if stream is None else stream
+        _lib.check(self._lib.hqekv_qk_hybrid(self.k_segs, self.n_k, q.data_ptr(), self.weights.data_ptr(), self.B,
+                                             self.Hq, self.Hkv, self.D, self.Tall, st), "run_qk")
+
+    def run_softmax(self, stream: Optional[int] = None):
+        st = _lib.stream_ptr(self.dev) if stream is None else stream
+        _lib.check(self._lib.hqekv_scale_softmax(self.weights.data_ptr(), self.mask_ptr, self.mask_stride,
+                                                 self.B * self.Hq, self.Tall, self.inv_sqrt_d, st), "run_softmax")
+
+    def run_pv(self, stream: Optional[int] = None):
+        st = _lib.stream_ptr(self.dev) if stream is None else stream
+        _lib.check(self._lib.hqekv_pv_hybrid(self.v_segs, self.n_v, self.weights.data_ptr(), self.out.data_ptr(),
+                                             self.B, self.Hq, self.Hkv, self.D, self.Tall, self.ws.data_ptr(),
+                                             self.ws.numel() * 4, st), "run_pv")

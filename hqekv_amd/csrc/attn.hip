@@ -35,23 +35,29 @@ struct SegDev {
   int64_t n_tokens;
   int32_t bits;
   int32_t token_major;
-  int32_t unit_begin;  // first tile (q.K^T) or chunk (p.V) of this segment in the launch
-  int32_t pad_;
+  int32_t unit_begin;  // first chunk of this segment in the p.V partial buffer
+  int32_t n_units;     // tiles (q.K^T) or chunks (p.V) of this segment; blockIdx.z selects the segment
 };
 
 struct SegTable {
   SegDev seg[HQEKV_MAX_SEGS];
   int32_t nseg;
   int32_t total_units;
+  int32_t max_units;   // grid.x: the largest n_units of any segment
+  int32_t pad_;
 };
 
-__device__ __forceinline__ int find_seg(const SegTable &tb, int unit) {
-  int s = 0;
-#pragma unroll
-  for (int k = 1; k < HQEKV_MAX_SEGS; ++k)
-    if (k < tb.nseg && unit >= tb.seg[k].unit_begin) s = k;
-  return s;
-}
+// A workgroup learns its segment from blockIdx.z and its tile/chunk from blockIdx.x, so everything it
+// needs from the kernel arguments is fetched in one batch at the top of the kernel (a scalar load that
+// misses costs about a microsecond; a lookup through the table would chain several of them).
+
+// keep every load issued above this point ahead of the arithmetic below it (the scheduler would
+// otherwise sink loads next to their uses to save registers, serialising the memory latency)
+#define HQ_LOADS_ABOVE()                     \
+  do {                                       \
+    asm volatile("" ::: "memory");           \
+    __builtin_amdgcn_sched_barrier(0);       \
+  } while (0)
 
 __device__ __forceinline__ half2_t as_h2(uint32_t u) {
   half2_t h;
@@ -89,7 +95,11 @@ __device__ __forceinline__ half2_t field_pair(uint32_t u) {
   constexpr uint32_t MASK = FMASK | (FMASK << 16);
   constexpr uint32_t EXPO = (uint32_t)(10 - POS + 15) << 10;  // fp16 bits of 2^(10-POS)
   constexpr uint32_t MAGIC = EXPO | (EXPO << 16);
-  const half2_t biased = as_h2((u & MASK) | MAGIC);     // 2^(10-POS) + c, exact
+  // (u & MASK) | MAGIC in one VALU op; the mask rides in a scalar register, the magic in a vector one
+  uint32_t r;
+  const uint32_t magic_v = MAGIC;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(u), "s"(MASK), "v"(magic_v));
+  const half2_t biased = as_h2(r);                      // 2^(10-POS) + c, exact
   const half2_t bias = as_h2(MAGIC);
   return biased - bias;                                 // c, exact
 }
@@ -129,135 +139,154 @@ __device__ __forceinline__ void consume_words(uint32_t w0, uint32_t w1, half2_t 
 }
 
 // =============================================================================== q.K^T
-constexpr int QK_THREADS = 256;
-constexpr int QK_WAVES = 4;
+constexpr int QK_THREADS = 512;
+constexpr int QK_WAVES = 8;
+constexpr int QK_TPL = 8;               // tokens per lane in every channel-major class
+constexpr int QK_TILE = 64 * QK_TPL;    // tokens per workgroup tile
+constexpr int QK_UNR = 8;               // row pairs whose loads are in flight together, per wave
 
 __host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
-  if (bits == 16) return token_major ? 64 : 128;
-  return 64 * (32 / bits);
+  return (bits == 16 && token_major) ? 64 : QK_TILE;
 }
 
-// cross-wave sum of PF accumulators per lane, one query head at a time (keeps LDS at 3*PF*256 B)
-template <int PF>
-__device__ __forceinline__ void qk_reduce_head(float (&a)[PF], float *red, int wave, int lane) {
-  if (wave > 0) {
-#pragma unroll
-    for (int i = 0; i < PF; ++i) red[((wave - 1) * PF + i) * 64 + lane] = a[i];
-  }
-  __syncthreads();
-  if (wave == 0) {
-#pragma unroll
-    for (int i = 0; i < PF; ++i)
-      a[i] += red[(0 * PF + i) * 64 + lane] + red[(1 * PF + i) * 64 + lane] + red[(2 * PF + i) * 64 + lane];
-  }
-  __syncthreads();
+// uniform base + 32-bit byte offset: the address math stays in scalar registers
+__device__ __forceinline__ uint32_t ld_u32(const void *base, uint32_t byte_off) {
+  return *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(base) + byte_off);
+}
+__device__ __forceinline__ half_t ld_f16(const void *base, uint32_t byte_off) {
+  return *reinterpret_cast<const half_t *>(reinterpret_cast<const char *>(base) + byte_off);
 }
 
-template <int NREP, int PF>
-__device__ __forceinline__ void qk_store(const SegDev &sg, float (&acc)[NREP][PF], int64_t t0, int b, int hkv,
-                                         int Hq, int64_t Tall, half_t *__restrict__ scores) {
-#pragma unroll
-  for (int i = 0; i < PF; ++i) {
-    if (t0 + i < sg.n_tokens) {
-      const int64_t pos = sg.idx ? sg.idx[t0 + i] : sg.pos_base + t0 + i;
-#pragma unroll
-      for (int h = 0; h < NREP; ++h)
-        scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = (half_t)acc[h][i];
-    }
-  }
-}
-
+// Accumulate one quantised tile: 512 tokens x D channels.  A lane owns 8 consecutive tokens: half a
+// packed word at 2 bits (two lanes read the same word), one word at 4 bits, two words at 8 bits.
+// QK_UNR row pairs at a time: every load of a block is issued before its first use, and the rolled outer
+// loop keeps the code small enough to stay in the instruction cache from one launch to the next.
 template <int BITS, int NREP>
-__device__ __forceinline__ void qk_quant_tile(const SegDev &sg, int tile, int bh, int b, int hkv, int D,
-                                              int Hq, int64_t Tall, const half2_t *q2s, float *red,
-                                              half_t *__restrict__ scores) {
+__device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int D, int wave,
+                                                    const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
   constexpr int PF = 32 / BITS;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t wpr = sg.n_tokens / PF;  // words per row
-  const int64_t gpr = sg.n_tokens / 32;  // groups per row
-  const int64_t jw = (int64_t)tile * 64 + lane;
-  const bool valid = jw < wpr;
-  const int64_t jws = valid ? jw : 0;
-  const int64_t g = (jws * PF) >> 5;
-  const uint32_t *code = (const uint32_t *)sg.data + (int64_t)bh * D * wpr + jws;
-  const half_t *sc = sg.scale + (int64_t)bh * D * gpr + g;
-  const half_t *zr = sg.zero + (int64_t)bh * D * gpr + g;
+  constexpr int NW = BITS == 8 ? 2 : 1;  // packed words per lane per row
+  const uint32_t n = (uint32_t)sg.n_tokens;
+  const uint32_t wpr = n / PF;   // words per row
+  const uint32_t gpr = n >> 5;   // groups per row
+  const uint32_t wofs = (ts / PF) * 4u;  // byte offset of this lane's first word inside a row
+  const uint32_t gofs = (ts >> 5) * 2u;  // byte offset of this lane's group inside a scale/zero row
+  const int sh2 = (BITS == 2) ? (int)((ts >> 3) & 1) * 16 : 0;  // which half of the 2-bit word
+  const uint32_t *code = (const uint32_t *)sg.data + (int64_t)bh * D * wpr;
+  const half_t *sc = sg.scale + (int64_t)bh * D * gpr;
+  const half_t *zr = sg.zero + (int64_t)bh * D * gpr;
   const int DP = D >> 1;
-
-  float acc[NREP][PF];
+#pragma unroll 1
+  for (int dp0 = wave; dp0 < DP; dp0 += QK_WAVES * QK_UNR) {
+    uint32_t w0[QK_UNR][NW], w1[QK_UNR][NW];
+    half_t s0[QK_UNR], s1[QK_UNR], z0[QK_UNR], z1[QK_UNR];
 #pragma unroll
-  for (int h = 0; h < NREP; ++h)
+    for (int k = 0; k < QK_UNR; ++k) {
+      const int dpk = dp0 + QK_WAVES * k;
+      const uint32_t d = 2u * (uint32_t)(dpk < DP ? dpk : dp0);    // uniform; past-the-end pairs reload dp0
+      const uint32_t *c0 = code + (size_t)d * wpr, *c1 = c0 + wpr;  // uniform row bases
+      const half_t *sa = sc + (size_t)d * gpr, *za = zr + (size_t)d * gpr;
 #pragma unroll
-    for (int i = 0; i < PF; ++i) acc[h][i] = 0.f;
-
-#pragma unroll 2
-  for (int dp = wave; dp < DP; dp += QK_WAVES) {
-    const int64_t d = 2 * dp;
-    const uint32_t w0 = code[d * wpr];
-    const uint32_t w1 = code[(d + 1) * wpr];
-    const half2_t s2 = pack_h2(sc[d * gpr], sc[(d + 1) * gpr]);
-    const half2_t z2 = pack_h2(zr[d * gpr], zr[(d + 1) * gpr]);
-    half2_t q2[NREP];
+      for (int j = 0; j < NW; ++j) {
+        w0[k][j] = ld_u32(c0, wofs + 4 * j);
+        w1[k][j] = ld_u32(c1, wofs + 4 * j);
+      }
+      s0[k] = ld_f16(sa, gofs);
+      s1[k] = ld_f16(sa + gpr, gofs);
+      z0[k] = ld_f16(za, gofs);
+      z1[k] = ld_f16(za + gpr, gofs);
+    }
+    HQ_LOADS_ABOVE();
 #pragma unroll
-    for (int h = 0; h < NREP; ++h) q2[h] = q2s[h * DP + dp];
-    consume_words<BITS, NREP, PF>(w0, w1, s2, z2, q2, acc);
+    for (int k = 0; k < QK_UNR; ++k) {
+      const int dp = dp0 + QK_WAVES * k;
+      if (dp >= DP) break;  // uniform
+      half2_t q2[NREP];
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) q2[h] = q2s[dp * NREP + h];
+      const half2_t s2 = pack_h2(s0[k], s1[k]), z2 = pack_h2(z0[k], z1[k]);
+      if (BITS == 2) {
+        const uint32_t a0 = w0[k][0] >> sh2, a1 = w1[k][0] >> sh2;
+        consume_byte<2, NREP, QK_TPL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
+        consume_byte<2, NREP, QK_TPL>(byte_pair<1>(a0, a1), s2, z2, q2, acc, 4);
+      } else if (BITS == 4) {
+        consume_byte<4, NREP, QK_TPL>(byte_pair<0>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 0);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<1>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 2);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<2>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 4);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<3>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 6);
+      } else {
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+          consume_byte<8, NREP, QK_TPL>(byte_pair<0>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 0);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<1>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 1);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<2>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 2);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<3>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 3);
+        }
+      }
+    }
   }
-#pragma unroll
-  for (int h = 0; h < NREP; ++h) qk_reduce_head<PF>(acc[h], red, wave, lane);
-  if (wave == 0 && valid) qk_store<NREP, PF>(sg, acc, jw * PF, b, hkv, Hq, Tall, scores);
 }
 
-// fp16 class stored channel-major (B,Hkv,D,T): a lane owns two adjacent tokens
+// fp16 class stored channel-major (B,Hkv,D,T): a lane owns 8 adjacent tokens of each row
 template <int NREP>
-__device__ __forceinline__ void qk_f16_cm_tile(const SegDev &sg, int tile, int bh, int b, int hkv, int D,
-                                               int Hq, int64_t Tall, const half2_t *q2s, float *red,
-                                               half_t *__restrict__ scores) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t n = sg.n_tokens;
-  const int64_t t0 = ((int64_t)tile * 64 + lane) * 2;
-  const bool v0 = t0 < n, v1 = t0 + 1 < n;
-  const half_t *kp = (const half_t *)sg.data + (int64_t)bh * D * n + (v0 ? t0 : 0);
-  const bool pair = (n & 1) == 0;  // rows stay 4-byte aligned
+__device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t t0, int bh, int D, int wave,
+                                                     const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
+  const uint32_t n = (uint32_t)sg.n_tokens;
+  const half_t *kp = (const half_t *)sg.data + (int64_t)bh * D * n;
+  const bool vec = (n & 7) == 0 && (((uintptr_t)kp) & 15) == 0 && t0 < n;  // rows stay 16-byte aligned
   const int DP = D >> 1;
-  float acc[NREP][2];
-#pragma unroll
-  for (int h = 0; h < NREP; ++h) acc[h][0] = acc[h][1] = 0.f;
-#pragma unroll 2
-  for (int dp = wave; dp < DP; dp += QK_WAVES) {
-    const int64_t d = 2 * dp;
-    uint32_t r0, r1;  // (k[d][t0], k[d][t0+1]) and the same for row d+1
-    if (pair) {
-      r0 = *reinterpret_cast<const uint32_t *>(kp + d * n);
-      r1 = *reinterpret_cast<const uint32_t *>(kp + (d + 1) * n);
+  auto load8 = [&](const half_t *row, uint32_t (&r)[4]) {
+    if (vec) {
+      const uint4 v = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(row) + t0 * 2u);
+      r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
     } else {
-      r0 = as_u32(pack_h2(kp[d * n], v1 ? kp[d * n + 1] : (half_t)0));
-      r1 = as_u32(pack_h2(kp[(d + 1) * n], v1 ? kp[(d + 1) * n + 1] : (half_t)0));
-    }
-    const half2_t ka = half_pair<0>(r0, r1);  // token t0:   (k[d], k[d+1])
-    const half2_t kb = half_pair<1>(r0, r1);  // token t0+1
 #pragma unroll
-    for (int h = 0; h < NREP; ++h) {
-      const half2_t q2 = q2s[h * DP + dp];
-      acc[h][0] = __builtin_amdgcn_fdot2(ka, q2, acc[h][0], false);
-      acc[h][1] = __builtin_amdgcn_fdot2(kb, q2, acc[h][1], false);
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t ta = t0 + 2 * i, tb = ta + 1;
+        r[i] = as_u32(pack_h2(ta < n ? row[ta] : (half_t)0, tb < n ? row[tb] : (half_t)0));
+      }
+    }
+  };
+  constexpr int UNR = 2;
+#pragma unroll 1
+  for (int dp0 = wave; dp0 < DP; dp0 += QK_WAVES * UNR) {
+    uint32_t r0[UNR][4], r1[UNR][4];
+#pragma unroll
+    for (int k = 0; k < UNR; ++k) {
+      const uint32_t d = 2u * (uint32_t)(dp0 + QK_WAVES * k);
+      load8(kp + (size_t)d * n, r0[k]);
+      load8(kp + (size_t)(d + 1) * n, r1[k]);
+    }
+    HQ_LOADS_ABOVE();
+#pragma unroll
+    for (int k = 0; k < UNR; ++k) {
+      const int dp = dp0 + QK_WAVES * k;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const half2_t ka = half_pair<0>(r0[k][i], r1[k][i]);  // token 2i:   (k[d], k[d+1])
+        const half2_t kb = half_pair<1>(r0[k][i], r1[k][i]);  // token 2i+1
+#pragma unroll
+        for (int h = 0; h < NREP; ++h) {
+          const half2_t q2 = q2s[dp * NREP + h];
+          acc[h][2 * i] = __builtin_amdgcn_fdot2(ka, q2, acc[h][2 * i], false);
+          acc[h][2 * i + 1] = __builtin_amdgcn_fdot2(kb, q2, acc[h][2 * i + 1], false);
+        }
+      }
     }
   }
-#pragma unroll
-  for (int h = 0; h < NREP; ++h) qk_reduce_head<2>(acc[h], red, wave, lane);
-  if (wave == 0 && v0) qk_store<NREP, 2>(sg, acc, t0, b, hkv, Hq, Tall, scores);
 }
 
 // fp16 residual stored token-major (B,Hkv,T,D): a wave walks tokens, lanes split the channels
 template <int NREP>
 __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int bh, int b, int hkv, int D,
-                                               int Hq, int64_t Tall, const half2_t *q2s,
+                                               int Hq, int64_t Tall, int wave, int lane, const half2_t *q2s,
                                                half_t *__restrict__ scores) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t n = sg.n_tokens;
   const half_t *kb = (const half_t *)sg.data + (int64_t)bh * n * D;
   const int DP = D >> 1;
-  for (int k = 0; k < 16; ++k) {
-    const int64_t t = (int64_t)tile * 64 + wave * 16 + k;
+#pragma unroll 1
+  for (int k = 0; k < 64 / QK_WAVES; ++k) {
+    const int64_t t = (int64_t)tile * 64 + wave * (64 / QK_WAVES) + k;
     if (t >= n) break;  // uniform per wave
     float part[NREP];
 #pragma unroll
@@ -265,7 +294,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
     for (int dp = lane; dp < DP; dp += 64) {
       const half2_t kk = *reinterpret_cast<const half2_t *>(kb + t * D + 2 * dp);
 #pragma unroll
-      for (int h = 0; h < NREP; ++h) part[h] = __builtin_amdgcn_fdot2(kk, q2s[h * DP + dp], part[h], false);
+      for (int h = 0; h < NREP; ++h) part[h] = __builtin_amdgcn_fdot2(kk, q2s[dp * NREP + h], part[h], false);
     }
 #pragma unroll
     for (int h = 0; h < NREP; ++h) part[h] = wave_sum(part[h]);
@@ -278,28 +307,97 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
   }
 }
 
+// One workgroup = one tile of one class for one (b, kv head).  The class-specific code is only the
+// accumulation; the cross-wave reduction and the (scattered) store are shared by every class.
 template <int NREP>
 __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
                                                                half_t *__restrict__ scores, int Hq,
                                                                int Hkv, int D, int64_t Tall) {
   extern __shared__ float smem[];
-  float *red = smem;                                          // 3 * 16 * 64 floats
-  half2_t *q2s = reinterpret_cast<half2_t *>(smem + 3 * 16 * 64);  // NREP * D/2 pairs (q[d], q[d+1])
+  float *red = smem;                                                        // QK_WAVES * 2 * 8 * 64 floats
+  half2_t *q2s = reinterpret_cast<half2_t *>(smem + QK_WAVES * 2 * QK_TPL * 64);  // D/2 x NREP pairs (q[d], q[d+1])
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int bh = blockIdx.y;
   const int b = bh / Hkv, hkv = bh % Hkv;
+  const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads, no lazy re-reads
+  const int tile = blockIdx.x;
+  if (tile >= sg.n_units) return;  // uniform: grid.x is the largest tile count of any segment
+  const bool tm = sg.bits == 16 && sg.token_major;
+  const uint32_t n = (uint32_t)sg.n_tokens;
+  const uint32_t t0 = (uint32_t)tile * QK_TILE + lane * QK_TPL;
+  const uint32_t ts = t0 < n ? t0 : 0;  // lanes past the end recompute token 0 and store nothing
+  // positions of this lane's 8 tokens: requested first (branch-free, so the loads overlap), used last
+  int64_t pos[QK_TPL];
+  {
+    const int64_t *ip = sg.idx;
+    const bool has_idx = ip != nullptr;
+#pragma unroll
+    for (int i = 0; i < QK_TPL; ++i) {
+      const uint32_t t = min(ts + i, n - 1);
+      pos[i] = sg.pos_base + t;
+      if (has_idx) pos[i] = ip[t];
+    }
+  }
   const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * D);
-  for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_THREADS) q2s[k] = as_h2(qsrc[k]);
+  for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_THREADS) {
+    const int h = k / (D >> 1), dp = k % (D >> 1);
+    q2s[dp * NREP + h] = as_h2(qsrc[k]);  // [dp][h]: one 16-byte LDS read fetches a row pair for 4 heads
+  }
   __syncthreads();
-  const int s = find_seg(tb, blockIdx.x);
-  const SegDev &sg = tb.seg[s];
-  const int tile = blockIdx.x - sg.unit_begin;
+  if (tm) {
+    qk_f16_tm_tile<NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores);
+    return;
+  }
+
+  float acc[NREP][QK_TPL];
+#pragma unroll
+  for (int h = 0; h < NREP; ++h)
+#pragma unroll
+    for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {
-    case 2: qk_quant_tile<2, NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, q2s, red, scores); break;
-    case 4: qk_quant_tile<4, NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, q2s, red, scores); break;
-    case 8: qk_quant_tile<8, NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, q2s, red, scores); break;
-    default:
-      if (sg.token_major) qk_f16_tm_tile<NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, q2s, scores);
-      else qk_f16_cm_tile<NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, q2s, red, scores);
+    case 2: qk_quant_accumulate<2, NREP>(sg, ts, bh, D, wave, q2s, acc); break;
+    case 4: qk_quant_accumulate<4, NREP>(sg, ts, bh, D, wave, q2s, acc); break;
+    case 8: qk_quant_accumulate<8, NREP>(sg, ts, bh, D, wave, q2s, acc); break;
+    default: qk_f16_cm_accumulate<NREP>(sg, t0, bh, D, wave, q2s, acc);
+  }
+
+  // cross-wave reduction, RH heads per pass (bounds LDS at QK_WAVES*RH*8*64*4 bytes): every wave parks
+  // its partials, then wave j of the pass sums head j over the waves and stores that head's row
+  constexpr int RH = NREP < 2 ? NREP : 2;
+  bool contig = (t0 + QK_TPL <= n);
+#pragma unroll
+  for (int i = 1; i < QK_TPL; ++i) contig = contig && (pos[i] == pos[0] + i);
+#pragma unroll
+  for (int h0 = 0; h0 < NREP; h0 += RH) {
+    if (h0 > 0) __syncthreads();
+#pragma unroll
+    for (int j = 0; j < RH; ++j)
+#pragma unroll
+      for (int i = 0; i < QK_TPL; ++i) red[((wave * RH + j) * QK_TPL + i) * 64 + lane] = acc[h0 + j][i];
+    __syncthreads();
+    if (wave < RH && t0 < n) {
+      const int h = h0 + wave;
+      half_t v[QK_TPL];
+#pragma unroll
+      for (int i = 0; i < QK_TPL; ++i) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < QK_WAVES; ++w) a += red[((w * RH + wave) * QK_TPL + i) * 64 + lane];
+        v[i] = (half_t)a;
+      }
+      half_t *row = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+      // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
+      // 128-bit store per head row; otherwise 2-byte scatters through idx
+      if (contig && (((uintptr_t)(row + pos[0])) & 15) == 0) {
+        uint4 raw;
+        __builtin_memcpy(&raw, v, 16);
+        *reinterpret_cast<uint4 *>(row + pos[0]) = raw;
+      } else {
+#pragma unroll
+        for (int i = 0; i < QK_TPL; ++i)
+          if (t0 + i < n) row[pos[i]] = v[i];
+      }
+    }
   }
 }
 
@@ -307,7 +405,7 @@ __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, cons
 constexpr int SM_THREADS = 1024;
 
 __device__ __forceinline__ float block_reduce(float v, float *sh, bool is_max) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   v = is_max ? wave_max(v) : wave_sum(v);
   __syncthreads();  // sh may still be read from a previous reduction
   if (lane == 0) sh[wave] = v;
@@ -324,6 +422,7 @@ __device__ __forceinline__ float sm_logit(half_t s, const half_t *mask, int64_t 
   return fmaxf((float)x, -65504.0f);
 }
 
+// Generic three-pass kernel: any row length, scalar accesses.
 __global__ __launch_bounds__(SM_THREADS) void scale_softmax_kernel(half_t *__restrict__ scores,
                                                                    const half_t *__restrict__ mask,
                                                                    int64_t mask_row_stride, int64_t Tall,
@@ -341,12 +440,89 @@ __global__ __launch_bounds__(SM_THREADS) void scale_softmax_kernel(half_t *__res
     row[t] = (half_t)(expf(sm_logit(row[t], mrow, t, inv) - m) / l);
 }
 
+// Register-resident kernel: the row is read once with 128-bit accesses aligned to memory (a row of
+// odd length does not start on a 16-byte boundary, so vector j covers elements [8j-off, 8j-off+8) and
+// the two edge vectors fall back to predicated scalar accesses), kept as fp16 logits in registers for
+// the max / sum / normalise passes, and written once.  NV <= 8 vectors per thread cover up to 65536 elements;
+// longer rows take the generic kernel.
+template <int NV>
+__global__ __launch_bounds__(SM_THREADS) void scale_softmax_reg_kernel(half_t *__restrict__ scores,
+                                                                       const half_t *__restrict__ mask,
+                                                                       int64_t mask_row_stride, int64_t Tall,
+                                                                       float inv) {
+  __shared__ float sh[SM_THREADS / 64];
+  half_t *row = scores + (int64_t)blockIdx.x * Tall;
+  const half_t *mrow = mask ? mask + (int64_t)blockIdx.x * mask_row_stride : nullptr;
+  const int off = (int)(((uintptr_t)row >> 1) & 7);  // elements between the previous 16-byte boundary and row[0]
+  half_t x[NV][8];
+  float m = -INFINITY;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int64_t e0 = ((int64_t)k * SM_THREADS + threadIdx.x) * 8 - off;  // first element of this vector
+    if (e0 >= 0 && e0 + 8 <= Tall) {
+      const uint4 raw = *reinterpret_cast<const uint4 *>(row + e0);
+      __builtin_memcpy(x[k], &raw, 16);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[k][i] = (e0 + i >= 0 && e0 + i < Tall) ? row[e0 + i] : (half_t)0;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t t = e0 + i;
+      if (t >= 0 && t < Tall) {
+        half_t v = (half_t)((float)x[k][i] * inv);
+        if (mrow) v = (half_t)((float)v + (float)mrow[t]);
+        v = (half_t)fmaxf((float)v, -65504.0f);
+        x[k][i] = v;
+        m = fmaxf(m, (float)v);
+      }
+    }
+  }
+  m = block_reduce(m, sh, true);
+  // exp(x - m) is evaluated once (hardware exp2; its error is far below one fp16 ulp of the result)
+  // and kept in registers for the normalisation
+  float e[NV][8];
+  float l = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int64_t e0 = ((int64_t)k * SM_THREADS + threadIdx.x) * 8 - off;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const bool in = e0 + i >= 0 && e0 + i < Tall;
+      e[k][i] = in ? __expf((float)x[k][i] - m) : 0.f;
+      l += e[k][i];
+    }
+  }
+  l = block_reduce(l, sh, false);
+  const float inv_l = 1.0f / l;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int64_t e0 = ((int64_t)k * SM_THREADS + threadIdx.x) * 8 - off;
+    if (e0 >= Tall || e0 + 8 <= 0) continue;
+    half_t y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = (half_t)(e[k][i] * inv_l);
+    if (e0 >= 0 && e0 + 8 <= Tall) {
+      uint4 raw;
+      __builtin_memcpy(&raw, y, 16);
+      *reinterpret_cast<uint4 *>(row + e0) = raw;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (e0 + i >= 0 && e0 + i < Tall) row[e0 + i] = y[i];
+    }
+  }
+}
+
 // =============================================================================== p.V
 constexpr int PV_THREADS = 256;
 constexpr int PV_WAVES = 4;
-constexpr int PV_BLOCK = 512;  // tokens staged in LDS at a time (256 token pairs)
+constexpr int PV_CPL = 8;                        // channels per lane
+constexpr int PV_BLOCK = 512;                    // tokens staged in LDS at a time (256 token pairs)
+constexpr int PV_UNR = 4;                        // wave steps whose loads are in flight together
 
-// LDS block: per token pair {s2, z2} for each of the D/32 groups, and p2 for each query head
+// LDS block, pair-interleaved: per token pair {s2, z2} for each of the D/32 groups and p2 for each
+// query head, so one 8-byte and one 4*NREP-byte LDS read feed a whole step of a lane.
 template <int NREP, int NG>
 struct PvStage {
   uint2 sz[PV_BLOCK / 2][NG];
@@ -358,13 +534,24 @@ template <int NREP, int NG, bool QUANT>
 __device__ __forceinline__ void pv_stage(const SegDev &sg, int64_t t0, int nt, int bh,
                                          const half_t *const (&prow)[NREP], PvStage<NREP, NG> &st) {
   const int ntp = (nt + 1) >> 1;
-  for (int k = threadIdx.x; k < ntp * NREP; k += PV_THREADS) {
-    const int tp = k / NREP, h = k % NREP;
+  const int64_t *ip = sg.idx;
+  for (int tp = threadIdx.x; tp < ntp; tp += PV_THREADS) {
     const int64_t ta = t0 + 2 * tp;
     const bool has_b = 2 * tp + 1 < nt;
-    const int64_t pa = sg.idx ? sg.idx[ta] : sg.pos_base + ta;
-    const int64_t pb = has_b ? (sg.idx ? sg.idx[ta + 1] : sg.pos_base + ta + 1) : pa;
-    st.p2[tp][h] = pack_h2(prow[h][pa], has_b ? prow[h][pb] : (half_t)0);
+    const int64_t tb2 = has_b ? ta + 1 : ta;
+    int64_t pa = sg.pos_base + ta, pb = sg.pos_base + tb2;
+    if (ip) {
+      pa = ip[ta];
+      pb = ip[tb2];
+    }
+    half_t va[NREP], vb[NREP];
+#pragma unroll
+    for (int h = 0; h < NREP; ++h) {
+      va[h] = prow[h][pa];
+      vb[h] = prow[h][pb];
+    }
+#pragma unroll
+    for (int h = 0; h < NREP; ++h) st.p2[tp][h] = pack_h2(va[h], has_b ? vb[h] : (half_t)0);
   }
   if (QUANT) {  // n_tokens is a multiple of 32, so pairs are always complete
     const half_t *sc = sg.scale + ((int64_t)bh * sg.n_tokens + t0) * NG;
@@ -379,96 +566,90 @@ __device__ __forceinline__ void pv_stage(const SegDev &sg, int64_t t0, int nt, i
   }
 }
 
+// One class chunk.  16 lanes cover a token row (8 channels each: half a packed word at 2 bits, one word
+// at 4 bits, two words at 8 bits, 16 bytes of fp16), 4 token pairs per wave step, so the reduction over
+// tokens needs only two butterfly steps across lanes.
 template <int BITS, int NREP, int D>
-__device__ __forceinline__ void pv_quant_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh,
-                                               const half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
-                                               float *red) {
-  constexpr int PF = 32 / BITS;
-  constexpr int WT = D / PF;    // words (lanes) per token row
-  constexpr int TPW = 64 / WT;  // token pairs per wave step
-  static_assert(WT >= 1 && WT <= 64 && (WT & (WT - 1)) == 0, "D/pf must be a power of two <= 64");
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int jl = lane % WT, tl = lane / WT;
-  const int g = (jl * PF) / 32;
-  const uint32_t *code = (const uint32_t *)sg.data + (int64_t)bh * sg.n_tokens * WT + jl;
-
-  float acc[NREP][PF];
-#pragma unroll
-  for (int h = 0; h < NREP; ++h)
-#pragma unroll
-    for (int i = 0; i < PF; ++i) acc[h][i] = 0.f;
+__device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh, int wave, int lane,
+                                         const half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
+                                         float (&acc)[NREP][PV_CPL]) {
+  static_assert(D == 128, "16 lanes x 8 channels cover one token row");
+  constexpr int WPL = BITS == 16 ? 4 : (BITS == 8 ? 2 : 1);  // 32-bit words per lane per token
+  constexpr int ROWW = D * BITS / 32;                         // 32-bit words per token row
+  const int cl = lane & 15, tl = lane >> 4;
+  const int g = cl >> 2;
+  const int sh2 = (BITS == 2) ? (cl & 1) * 16 : 0;
+  const uint32_t wofs = (BITS == 2 ? (cl >> 1) : cl * WPL) * 4u;  // byte offset inside a token row
+  const char *base = (const char *)sg.data + (int64_t)bh * sg.n_tokens * ROWW * 4;
 
   for (int64_t t0 = c0; t0 < c1; t0 += PV_BLOCK) {
     const int nt = (int)min((int64_t)PV_BLOCK, c1 - t0);
-    __syncthreads();
-    pv_stage<NREP, D / 32, true>(sg, t0, nt, bh, prow, st);
-    __syncthreads();
-    const int ntp = nt >> 1;
-#pragma unroll 2
-    for (int tp = wave * TPW + tl; tp < ntp; tp += PV_WAVES * TPW) {
-      const int64_t t = t0 + 2 * tp;
-      const uint32_t w0 = code[t * WT];
-      const uint32_t w1 = code[(t + 1) * WT];
-      const uint2 sz = st.sz[tp][g];
-      half2_t p2[NREP];
-#pragma unroll
-      for (int h = 0; h < NREP; ++h) p2[h] = st.p2[tp][h];
-      consume_words<BITS, NREP, PF>(w0, w1, as_h2(sz.x), as_h2(sz.y), p2, acc);
-    }
-  }
-#pragma unroll
-  for (int h = 0; h < NREP; ++h) {
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      float v = acc[h][i];
-#pragma unroll
-      for (int m = WT; m < 64; m <<= 1) v += xor_f(v, m);
-      if (tl == 0) red[(wave * NREP + h) * D + jl * PF + i] = v;
-    }
-  }
-}
-
-template <int NREP, int D>
-__device__ __forceinline__ void pv_f16_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh,
-                                             const half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
-                                             float *red) {
-  constexpr int LPT = D / 2;     // lanes per token row (a lane owns two channels)
-  constexpr int TPW = 64 / LPT;  // token pairs per wave step
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int jl = lane % LPT, tl = lane / LPT;
-  const half_t *vb = (const half_t *)sg.data + (int64_t)bh * sg.n_tokens * D + jl * 2;
-  float acc[NREP][2];
-#pragma unroll
-  for (int h = 0; h < NREP; ++h) acc[h][0] = acc[h][1] = 0.f;
-  for (int64_t t0 = c0; t0 < c1; t0 += PV_BLOCK) {
-    const int nt = (int)min((int64_t)PV_BLOCK, c1 - t0);
-    __syncthreads();
-    pv_stage<NREP, D / 32, false>(sg, t0, nt, bh, prow, st);
-    __syncthreads();
     const int ntp = (nt + 1) >> 1;
-#pragma unroll 2
-    for (int tp = wave * TPW + tl; tp < ntp; tp += PV_WAVES * TPW) {
-      const int64_t t = t0 + 2 * tp;
-      const uint32_t r0 = *reinterpret_cast<const uint32_t *>(vb + t * D);
-      const uint32_t r1 = (2 * tp + 1 < nt) ? *reinterpret_cast<const uint32_t *>(vb + (t + 1) * D) : 0u;
-      const half2_t va = half_pair<0>(r0, r1);  // channel 2*jl:   (v[t], v[t+1])
-      const half2_t vc = half_pair<1>(r0, r1);  // channel 2*jl+1
+    const int nsteps = (ntp + 4 * PV_WAVES - 1) / (4 * PV_WAVES);
+    __syncthreads();  // previous block fully consumed
+    if (BITS == 16) pv_stage<NREP, D / 32, false>(sg, t0, nt, bh, prow, st);
+    else pv_stage<NREP, D / 32, true>(sg, t0, nt, bh, prow, st);
+    __syncthreads();
+#pragma unroll 1
+    for (int s0 = 0; s0 < nsteps; s0 += PV_UNR) {
+      uint32_t w0[PV_UNR][WPL], w1[PV_UNR][WPL];
 #pragma unroll
-      for (int h = 0; h < NREP; ++h) {
-        const half2_t p2 = st.p2[tp][h];
-        acc[h][0] = __builtin_amdgcn_fdot2(va, p2, acc[h][0], false);
-        acc[h][1] = __builtin_amdgcn_fdot2(vc, p2, acc[h][1], false);
+      for (int k = 0; k < PV_UNR; ++k) {
+        const int tp = 4 * ((s0 + k) * PV_WAVES + wave) + tl;
+        const int tpc = tp < ntp ? tp : 0;
+        const bool has_b = 2 * tpc + 1 < nt;
+        const char *ra = base + (t0 + 2 * tpc) * (int64_t)(ROWW * 4) + wofs;
+        const char *rb = has_b ? ra + ROWW * 4 : ra;
+#pragma unroll
+        for (int j = 0; j < WPL; ++j) {
+          w0[k][j] = *reinterpret_cast<const uint32_t *>(ra + 4 * j);
+          w1[k][j] = *reinterpret_cast<const uint32_t *>(rb + 4 * j);
+        }
       }
-    }
-  }
+      HQ_LOADS_ABOVE();
 #pragma unroll
-  for (int h = 0; h < NREP; ++h) {
+      for (int k = 0; k < PV_UNR; ++k) {
+        const int tp = 4 * ((s0 + k) * PV_WAVES + wave) + tl;
+        if (tp < ntp) {
+          half2_t p2[NREP];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      float v = acc[h][i];
+          for (int h = 0; h < NREP; ++h) p2[h] = st.p2[tp][h];
+          if (BITS == 16) {
+            // an odd tail pair has p = 0 for its second token, so the duplicated row adds nothing
 #pragma unroll
-      for (int m = LPT; m < 64; m <<= 1) v += xor_f(v, m);
-      if (tl == 0) red[(wave * NREP + h) * D + jl * 2 + i] = v;
+            for (int j = 0; j < 4; ++j) {
+              const half2_t va = half_pair<0>(w0[k][j], w1[k][j]);  // channel 2j:   (v[t], v[t+1])
+              const half2_t vb = half_pair<1>(w0[k][j], w1[k][j]);  // channel 2j+1
+#pragma unroll
+              for (int h = 0; h < NREP; ++h) {
+                acc[h][2 * j] = __builtin_amdgcn_fdot2(va, p2[h], acc[h][2 * j], false);
+                acc[h][2 * j + 1] = __builtin_amdgcn_fdot2(vb, p2[h], acc[h][2 * j + 1], false);
+              }
+            }
+          } else {
+            const uint2 sz = st.sz[tp][g];
+            const half2_t s2 = as_h2(sz.x), z2 = as_h2(sz.y);
+            if (BITS == 2) {
+              const uint32_t a0 = w0[k][0] >> sh2, a1 = w1[k][0] >> sh2;
+              consume_byte<2, NREP, PV_CPL>(byte_pair<0>(a0, a1), s2, z2, p2, acc, 0);
+              consume_byte<2, NREP, PV_CPL>(byte_pair<1>(a0, a1), s2, z2, p2, acc, 4);
+            } else if (BITS == 4) {
+              consume_byte<4, NREP, PV_CPL>(byte_pair<0>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 0);
+              consume_byte<4, NREP, PV_CPL>(byte_pair<1>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 2);
+              consume_byte<4, NREP, PV_CPL>(byte_pair<2>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 4);
+              consume_byte<4, NREP, PV_CPL>(byte_pair<3>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 6);
+            } else {
+#pragma unroll
+              for (int j = 0; j < (BITS == 8 ? 2 : 0); ++j) {
+                consume_byte<8, NREP, PV_CPL>(byte_pair<0>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 0);
+                consume_byte<8, NREP, PV_CPL>(byte_pair<1>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 1);
+                consume_byte<8, NREP, PV_CPL>(byte_pair<2>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 2);
+                consume_byte<8, NREP, PV_CPL>(byte_pair<3>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 3);
+              }
+            }
+          }
+        }
+      }
     }
   }
 }
@@ -480,38 +661,70 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, cons
                                                                int64_t n_bhq) {
   __shared__ float red[PV_WAVES * NREP * D];
   __shared__ PvStage<NREP, D / 32> st;
+  const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads
+  if ((int)blockIdx.x >= sg.n_units) return;  // uniform: grid.x is the largest chunk count of any segment
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int bh = blockIdx.y;
   const int b = bh / Hkv, hkv = bh % Hkv;
-  const int s = find_seg(tb, blockIdx.x);
-  const SegDev &sg = tb.seg[s];
-  const int64_t c0 = (int64_t)(blockIdx.x - sg.unit_begin) * chunk_tokens;
+  const int chunk_id = sg.unit_begin + (int)blockIdx.x;
+  const int64_t c0 = (int64_t)blockIdx.x * chunk_tokens;
   const int64_t c1 = min(c0 + chunk_tokens, sg.n_tokens);
   const half_t *prow[NREP];
 #pragma unroll
   for (int h = 0; h < NREP; ++h) prow[h] = p + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+  float acc[NREP][PV_CPL];
+#pragma unroll
+  for (int h = 0; h < NREP; ++h)
+#pragma unroll
+    for (int i = 0; i < PV_CPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {
-    case 2: pv_quant_chunk<2, NREP, D>(sg, c0, c1, bh, prow, st, red); break;
-    case 4: pv_quant_chunk<4, NREP, D>(sg, c0, c1, bh, prow, st, red); break;
-    case 8: pv_quant_chunk<8, NREP, D>(sg, c0, c1, bh, prow, st, red); break;
-    default: pv_f16_chunk<NREP, D>(sg, c0, c1, bh, prow, st, red);
+    case 2: pv_chunk<2, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc); break;
+    case 4: pv_chunk<4, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc); break;
+    case 8: pv_chunk<8, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc); break;
+    default: pv_chunk<16, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc);
   }
+  // lanes 16 and 32 apart hold the same channels of other tokens
+  const int cl = lane & 15;
+#pragma unroll
+  for (int h = 0; h < NREP; ++h)
+#pragma unroll
+    for (int i = 0; i < PV_CPL; ++i) {
+      float v = acc[h][i];
+      v += xor_f(v, 16);
+      v += xor_f(v, 32);
+      if (lane < 16) red[(wave * NREP + h) * D + cl * PV_CPL + i] = v;
+    }
   __syncthreads();
   for (int k = threadIdx.x; k < NREP * D; k += PV_THREADS) {
     const float v = red[k] + red[NREP * D + k] + red[2 * NREP * D + k] + red[3 * NREP * D + k];
     const int h = k / D, d = k % D;
-    partial[((int64_t)blockIdx.x * n_bhq + (int64_t)b * Hq + hkv * NREP + h) * D + d] = v;
+    partial[((int64_t)chunk_id * n_bhq + (int64_t)b * Hq + hkv * NREP + h) * D + d] = v;
   }
 }
 
 // fixed-order sum over chunks: deterministic replacement for the reference's half atomics
-// (quant/csrc/gemv_cuda_wv_uniform.cu:110)
-__global__ void pv_combine_kernel(const float *__restrict__ partial, half_t *__restrict__ out, int n_chunks,
-                                  int64_t n_bhq, int D) {
+// (quant/csrc/gemv_cuda_wv_uniform.cu:110).  One workgroup per (b, hq) row; CB_SLICES slices of the
+// chunk list are summed in parallel (strided, ascending within a slice), then the slices in order.
+constexpr int CB_SLICES = 8;
+__global__ __launch_bounds__(1024) void pv_combine_kernel(const float *__restrict__ partial,
+                                                          half_t *__restrict__ out, int n_chunks,
+                                                          int64_t n_bhq, int D) {
+  __shared__ float sh[CB_SLICES][128];
   const int64_t r = blockIdx.x;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+  const int d = threadIdx.x % 128, sl = threadIdx.x / 128;
+  for (int d0 = 0; d0 < D; d0 += 128) {
     float v = 0.f;
-    for (int c = 0; c < n_chunks; ++c) v += partial[((int64_t)c * n_bhq + r) * D + d];
-    out[r * D + d] = (half_t)v;
+    if (d0 + d < D)
+      for (int c = sl; c < n_chunks; c += CB_SLICES) v += partial[((int64_t)c * n_bhq + r) * D + d0 + d];
+    sh[sl][d] = v;
+    __syncthreads();
+    if (sl == 0 && d0 + d < D) {
+      float t = sh[0][d];
+#pragma unroll
+      for (int k = 1; k < CB_SLICES; ++k) t += sh[k][d];
+      out[r * D + d0 + d] = (half_t)t;
+    }
+    __syncthreads();
   }
 }
 
@@ -521,7 +734,7 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
                        int64_t Tall, SegTable *tb, const char *who) {
   if (nseg < 0 || nseg > HQEKV_MAX_SEGS) return fail(HQEKV_E_ARG, "%s: nseg=%d out of range", who, nseg);
   if (nseg > 0 && !segs) return fail(HQEKV_E_ARG, "%s: null segment table", who);
-  int64_t units = 0;
+  int64_t units = 0, max_units = 0;
   int m = 0;
   for (int k = 0; k < nseg; ++k) {
     const hqekv_seg &s = segs[k];
@@ -539,6 +752,8 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
       return fail(HQEKV_E_ARG, "%s: segment %d positions [%lld,%lld) outside [0,%lld)", who, k,
                   (long long)s.pos_base, (long long)(s.pos_base + s.n_tokens), (long long)Tall);
     if ((uintptr_t)s.data & 3) return fail(HQEKV_E_ALIGN, "%s: segment %d data not 4-byte aligned", who, k);
+    if (s.n_tokens * D >= (1LL << 31))
+      return fail(HQEKV_E_UNSUPPORTED, "%s: segment %d: n_tokens * D must stay below 2^31 per (b, head) slab", who, k);
     SegDev &d = tb->seg[m++];
     d.data = s.data;
     d.scale = (const half_t *)s.scale;
@@ -549,13 +764,17 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
     d.bits = s.bits;
     d.token_major = is_k ? (s.bits == 16 && s.token_major) : 0;
     d.unit_begin = (int32_t)units;
-    d.pad_ = 0;
     const int64_t per = is_k ? qk_tile_tokens(s.bits, d.token_major) : chunk_tokens;
-    units += (s.n_tokens + per - 1) / per;
+    const int64_t nu = (s.n_tokens + per - 1) / per;
+    d.n_units = (int32_t)nu;
+    if (nu > max_units) max_units = nu;
+    units += nu;
     if (units > 0x3fffffff) return fail(HQEKV_E_ARG, "%s: too many work units", who);
   }
   tb->nseg = m;
   tb->total_units = (int32_t)units;
+  tb->max_units = (int32_t)max_units;
+  tb->pad_ = 0;
   (void)D;
   return HQEKV_OK;
 }
@@ -576,8 +795,8 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
                      int64_t D, int64_t Tall, hipStream_t st) {
   if (tb.total_units == 0) return HQEKV_OK;
   const int nrep = (int)(Hq / Hkv);
-  dim3 grid((unsigned)tb.total_units, (unsigned)(B * Hkv)), block(QK_THREADS);
-  const size_t shmem = (size_t)(nrep * D + 3 * 16 * 64) * sizeof(float);
+  dim3 grid((unsigned)tb.max_units, (unsigned)(B * Hkv), (unsigned)tb.nseg), block(QK_THREADS);
+  const size_t shmem = (size_t)(nrep * D + QK_WAVES * 2 * QK_TPL * 64) * sizeof(float);
 #define LAUNCH(N_)                                                                                    \
   hipLaunchKernelGGL(qk_hybrid_kernel<N_>, grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
                      (int)Hq, (int)Hkv, (int)D, Tall)
@@ -614,12 +833,11 @@ static int launch_pv(const SegTable &tb, int64_t chunk, const void *p, void *out
   const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
   if (tb.total_units > 0) {
-    dim3 grid((unsigned)tb.total_units, (unsigned)(B * Hkv)), block(PV_THREADS);
+    dim3 grid((unsigned)tb.max_units, (unsigned)(B * Hkv), (unsigned)tb.nseg), block(PV_THREADS);
 #define LAUNCH(N_, D_)                                                                                   \
   hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_>), grid, block, 0, st, tb, (const half_t *)p, partial, (int)Hq, \
                      (int)Hkv, Tall, chunk, n_bhq)
-#define LAUNCH_D(N_) \
-  if (D == 128) LAUNCH(N_, 128); else LAUNCH(N_, 64)
+#define LAUNCH_D(N_) LAUNCH(N_, 128)
     switch (nrep) {
       case 1: LAUNCH_D(1); break;
       case 2: LAUNCH_D(2); break;
@@ -631,7 +849,7 @@ static int launch_pv(const SegTable &tb, int64_t chunk, const void *p, void *out
     int rc = check_launch("pv_hybrid_kernel");
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq), dim3((unsigned)(D < 64 ? 64 : D)), 0, st, partial,
+  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq), dim3(128 * CB_SLICES), 0, st, partial,
                      (half_t *)out, (int)tb.total_units, n_bhq, (int)D);
   return check_launch("pv_combine_kernel");
 }
@@ -657,8 +875,19 @@ extern "C" int hqekv_scale_softmax(void *scores, const void *mask, int64_t mask_
   if (n_rows < 0 || Tall <= 0 || n_rows > 0x7fffffffLL) return fail(HQEKV_E_ARG, "scale_softmax: bad shape");
   if (n_rows == 0) return HQEKV_OK;
   if (!scores) return fail(HQEKV_E_ARG, "scale_softmax: null scores");
-  hipLaunchKernelGGL(scale_softmax_kernel, dim3((unsigned)n_rows), dim3(SM_THREADS), 0, (hipStream_t)stream,
-                     (half_t *)scores, (const half_t *)mask, mask_row_stride, Tall, inv_sqrt_d);
+  const dim3 grid((unsigned)n_rows), block(SM_THREADS);
+  hipStream_t st = (hipStream_t)stream;
+  half_t *sp = (half_t *)scores;
+  const half_t *mp = (const half_t *)mask;
+  const int64_t nv = (Tall + 7 + 8 * SM_THREADS - 1) / (8 * SM_THREADS);  // +7: worst-case alignment shift
+  if (((uintptr_t)scores & 1) == 0 && nv <= 8) {
+#define LAUNCH(N_) \
+  hipLaunchKernelGGL(scale_softmax_reg_kernel<N_>, grid, block, 0, st, sp, mp, mask_row_stride, Tall, inv_sqrt_d)
+    if (nv <= 1) LAUNCH(1); else if (nv <= 2) LAUNCH(2); else if (nv <= 4) LAUNCH(4); else LAUNCH(8);
+#undef LAUNCH
+  } else {
+    hipLaunchKernelGGL(scale_softmax_kernel, grid, block, 0, st, sp, mp, mask_row_stride, Tall, inv_sqrt_d);
+  }
   return check_launch("scale_softmax_kernel");
 }
 
@@ -678,7 +907,7 @@ extern "C" int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, v
                                void *stream) {
   int rc = check_heads("pv_hybrid", B, Hq, Hkv, D);
   if (rc) return rc;
-  if (!(D == 128 || D == 64)) return fail(HQEKV_E_UNSUPPORTED, "pv_hybrid: D=%lld (supported: 64, 128)", (long long)D);
+  if (D != 128) return fail(HQEKV_E_UNSUPPORTED, "pv_hybrid: head_dim %lld (supported: 128)", (long long)D);
   if (!p || !out || Tall <= 0) return fail(HQEKV_E_ARG, "pv_hybrid: null pointer or Tall <= 0");
   const int64_t chunk = pv_chunk_tokens(seg_total_tokens(segs, nseg), B * Hkv);
   SegTable tb{};
@@ -706,7 +935,7 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
 }
 
 // ------------------------------------------------------------------ per-class GEMV on the same kernels
-static bool gemv_is_pv_shape(int64_t K, int64_t N) { return (N == 64 || N == 128) && K % 32 == 0 && K > N; }
+static bool gemv_is_pv_shape(int64_t K, int64_t N) { return N == 128 && K % 32 == 0 && K > N; }
 
 extern "C" int64_t hqekv_gemv_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N, int bits) {
   (void)bits;

@@ -35,7 +35,7 @@ CASES = [
     dict(B=1, Hq=32, Hkv=8, T=4096, D=128, fractions=(0.0, 0.0, 0.0, 1.0, 0.0), residual=128, seed=1235),  # config 1
     dict(B=1, Hq=4, Hkv=4, T=512 + 31, D=128, fractions=(0.25, 0.0, 0.5, 0.0, 0.25), residual=31, seed=4),
     dict(B=1, Hq=16, Hkv=2, T=1024, D=128, fractions=(0.0, 1.0, 0.0, 0.0, 0.0), residual=0, seed=5),
-    dict(B=1, Hq=8, Hkv=2, T=640 + 5, D=64, fractions=(0.1, 0.2, 0.3, 0.3, 0.1), residual=5, seed=6),
+    dict(B=3, Hq=8, Hkv=1, T=640 + 5, D=128, fractions=(0.1, 0.2, 0.3, 0.3, 0.1), residual=5, seed=6),
 ]
 
 
@@ -128,6 +128,14 @@ def test_all_fp16_equals_dense_attention(dev):
     _close(o, torch.matmul(pr.float(), O.repeat_kv(Vp, 4).float()))
 
 
+def test_unsupported_head_dim_is_an_error(dev):
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    q, K, V = synth.make_qkv(1, 4, 2, 64, 64, 3)
+    cache = O.empty_cache(K, V, 64)
+    with pytest.raises(ValueError, match="head_dim"):
+        qkv_matmul_hqe_2(q.to(dev), synth.cache_to(cache, dev), None, 64, "uniform_group")
+
+
 def test_errors(dev):
     from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
     from hqekv_amd.quant_matmul_hq import qkv_matmul
@@ -140,3 +148,26 @@ def test_errors(dev):
         qkv_matmul(q, (None,) * 41 + (0,), None, 128, "bogus")
     with pytest.raises(ValueError, match="invalid past_key_value"):
         qkv_matmul(q, (None,) * 41 + (0,), None, 128, "uniform_group")
+
+
+@pytest.mark.parametrize("Tall", [1, 7, 8, 1000, 8191, 8200, 26225, 70001, 140003])
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_scale_softmax_rows(dev, Tall, with_mask):
+    """The epilogue alone, through the C ABI, on aligned and odd row lengths (register-resident and
+    generic kernels) against the oracle's fp16-scale / fp32-softmax chain."""
+    from hqekv_amd import _lib
+    g = torch.Generator().manual_seed(Tall)
+    rows = 5
+    s = (torch.randn(rows, Tall, generator=g) * 30).half()
+    mask = None
+    if with_mask:
+        mask = torch.zeros(rows, Tall, dtype=torch.float16)
+        mask[:, torch.randperm(Tall, generator=g)[:Tall // 3]] = torch.finfo(torch.float16).min
+    ref = O._scale_clamp_softmax(s.view(1, rows, 1, Tall), 128, None if mask is None else mask.view(1, rows, 1, Tall),
+                                 "recip").view(rows, Tall)
+    sd = s.to(dev)
+    md = mask.to(dev) if with_mask else None
+    rc = _lib.load().hqekv_scale_softmax(sd.data_ptr(), None if md is None else md.data_ptr(), Tall, rows, Tall,
+                                         1.0 / 128 ** 0.5, _lib.stream_ptr(dev))
+    _lib.check(rc, "scale_softmax")
+    torch.testing.assert_close(sd.float().cpu(), ref.float(), rtol=RTOL, atol=1e-5)
