@@ -16,6 +16,7 @@ _PKG = Path(__file__).resolve().parent
 _LIB_PATH = Path(os.environ.get("HQEKV_LIB", _PKG / "libhqekv.so"))
 
 MAX_SEGS = 8
+FUSE_SOFTMAX = 1
 
 # every symbol include/hqekv.h declares
 EXPORTS = (
@@ -23,7 +24,7 @@ EXPORTS = (
     "hqekv_quant_pack_rows", "hqekv_quant_pack_k_tokenmajor", "hqekv_dequant_unpack_rows", "hqekv_pack_i32",
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
-    "hqekv_decode_attn",
+    "hqekv_decode_workspace_bytes", "hqekv_decode_attn",
 )
 
 
@@ -59,7 +60,8 @@ _PROTOS = {
     "hqekv_scale_softmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, C.c_float, _vp]),
     "hqekv_pv_workspace_bytes": (_i64, [_SEGP, _int, _i64, _i64, _i64, _i64]),
     "hqekv_pv_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
-    "hqekv_decode_attn": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "hqekv_decode_workspace_bytes": (_i64, [_SEGP, _int, _SEGP, _int, _i64, _i64, _i64, _i64]),
+    "hqekv_decode_attn": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _int, _vp]),
 }
 
 

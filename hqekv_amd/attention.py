@@ -9,6 +9,7 @@ Each populated class becomes one ``hqekv_seg``; the kernels read the tensors whe
 from __future__ import annotations
 
 import ctypes as C
+import os
 from typing import List, Optional, Tuple
 
 import torch
@@ -146,17 +147,32 @@ def _mask_arg(mask, B: int, Hq: int, Tall: int, dev, keep: list):
 
 
 def workspace_for(v_segs, n_v: int, B: int, Hq: int, Hkv: int, D: int, dev) -> torch.Tensor:
+    """Split-K workspace of a stand-alone p.V launch."""
     need = _lib.load().hqekv_pv_workspace_bytes(v_segs, n_v, B, Hq, Hkv, D)
     if need < 0:
         raise ValueError("invalid segment table")
     return torch.empty(max(need, 16) // 4, dtype=torch.float32, device=dev)
 
 
-def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool):
+def decode_workspace(k_segs, n_k: int, v_segs, n_v: int, B: int, Hq: int, Hkv: int, D: int, dev) -> torch.Tensor:
+    """Workspace of a whole decode-attention call (partials, softmax statistics, arrival counters)."""
+    need = _lib.load().hqekv_decode_workspace_bytes(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D)
+    if need < 0:
+        raise ValueError("invalid segment table")
+    return torch.empty(max(need, 256) // 4, dtype=torch.float32, device=dev)
+
+
+def default_flags() -> int:
+    """Fuse the softmax into the two GEMV launches unless HQEKV_UNFUSED=1 asks for the general path."""
+    return 0 if os.environ.get("HQEKV_UNFUSED", "0") == "1" else _lib.FUSE_SOFTMAX
+
+
+def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool, flags: Optional[int] = None):
     """q (B,Hq,1,D) fp16 -> (attn_weights (B,Hq,1,Tall) fp16 probabilities, attn_output (B,Hq,1,D) fp16).
 
-    One qk launch over all K classes, the scale/mask/clamp/softmax pass, one p.V launch over all
-    V classes plus the fixed-order combine, on torch's current stream.
+    One q.K^T launch over all K classes and one p.V launch over all V classes with the softmax fused
+    into them; or, with a mask / an incomplete cover of the positions / ``flags=0``, the general path
+    (q.K^T, scale+mask+clamp+softmax, p.V, fixed-order combine).  Runs on torch's current stream.
     """
     _lib.require_gpu(q, "q")
     if q.dtype != torch.float16:
@@ -180,11 +196,11 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     k_segs, v_segs = _lib.make_segs(k_items), _lib.make_segs(v_items)
     mptr, mstride = _mask_arg(mask, B, Hq, Tall, dev, keep)
     with torch.cuda.device(dev):
-        ws = workspace_for(v_segs, len(v_items), B, Hq, Hkv, D, dev)
+        ws = decode_workspace(k_segs, len(k_items), v_segs, len(v_items), B, Hq, Hkv, D, dev)
         rc = _lib.load().hqekv_decode_attn(
             k_segs, len(k_items), v_segs, len(v_items), qc.data_ptr(), mptr, mstride,
             weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4,
-            _lib.stream_ptr(dev))
+            default_flags() if flags is None else flags, _lib.stream_ptr(dev))
     _lib.check(rc, "decode_attention")
     return weights, out
 
@@ -195,7 +211,8 @@ class DecodePlan:
     combine) with no per-step Python work.  Holds references to every tensor it points into.
     """
 
-    def __init__(self, q_like: torch.Tensor, pkv: tuple, mask=None, Tall: Optional[int] = None):
+    def __init__(self, q_like: torch.Tensor, pkv: tuple, mask=None, Tall: Optional[int] = None,
+                 flags: Optional[int] = None):
         _lib.require_gpu(q_like, "q")
         B, Hq, _, D = q_like.shape
         self.dev = q_like.device
@@ -213,7 +230,8 @@ class DecodePlan:
         self.out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=self.dev)
         self.mask_ptr, self.mask_stride = _mask_arg(mask, B, Hq, self.Tall, self.dev, self._keep)
         with torch.cuda.device(self.dev):
-            self.ws = workspace_for(self.v_segs, self.n_v, B, Hq, self.Hkv, D, self.dev)
+            self.ws = decode_workspace(self.k_segs, self.n_k, self.v_segs, self.n_v, B, Hq, self.Hkv, D, self.dev)
+        self.flags = default_flags() if flags is None else flags
         self._lib = _lib.load()
         self.inv_sqrt_d = 1.0 / (D ** 0.5)
 
@@ -222,7 +240,7 @@ class DecodePlan:
         rc = self._lib.hqekv_decode_attn(
             self.k_segs, self.n_k, self.v_segs, self.n_v, q.data_ptr(), self.mask_ptr, self.mask_stride,
             self.weights.data_ptr(), self.out.data_ptr(), self.B, self.Hq, self.Hkv, self.D, self.Tall,
-            self.ws.data_ptr(), self.ws.numel() * 4, st)
+            self.ws.data_ptr(), self.ws.numel() * 4, self.flags, st)
         if rc:
             _lib.check(rc, "DecodePlan.run")
         return self.weights, self.out

@@ -47,6 +47,19 @@ struct SegTable {
   int32_t pad_;
 };
 
+// Optional fusion of the softmax into the two GEMV launches (valid when no mask is added and the K
+// classes as well as the V classes each cover every position exactly once):
+//   q.K^T stores the scaled fp16 logit instead of the raw score and one (max, sum exp) pair per tile and
+//   head; p.V turns a logit into its probability while staging it and writes it back for the caller.
+// The split-K partials are summed by a separate small launch: a "last workgroup sums" scheme needs
+// device-scope release/acquire fences, which write back and invalidate the whole L2 on this chip and cost
+// far more than the launch they would save.
+struct FuseArgs {
+  float2 *stats;       // (B*Hq, n_stat) pairs (m, l); nullptr = unfused
+  int32_t n_stat;      // tiles per row of stats = number of q.K^T tiles per (b, kv head)
+  float inv_sqrt_d;
+};
+
 // A workgroup learns its segment from blockIdx.z and its tile/chunk from blockIdx.x, so everything it
 // needs from the kernel arguments is fetched in one batch at the top of the kernel (a scalar load that
 // misses costs about a microsecond; a lookup through the table would chain several of them).
@@ -149,12 +162,21 @@ __host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
   return (bits == 16 && token_major) ? 64 : QK_TILE;
 }
 
-// uniform base + 32-bit byte offset: the address math stays in scalar registers
-__device__ __forceinline__ uint32_t ld_u32(const void *base, uint32_t byte_off) {
-  return *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(base) + byte_off);
+// Buffer addressing: a 128-bit descriptor per (b, head) slab in scalar registers, a per-lane byte offset
+// that never changes, and the row offset in a scalar register -- no vector ALU work per load, and reads
+// past the end of the slab return zero instead of faulting.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
-__device__ __forceinline__ half_t ld_f16(const void *base, uint32_t byte_off) {
-  return *reinterpret_cast<const half_t *>(reinterpret_cast<const char *>(base) + byte_off);
+__device__ __forceinline__ uint32_t buf_u32(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)row_off, 0);
+}
+__device__ __forceinline__ half_t buf_f16(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  const unsigned short u = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, (int)row_off, 0);
+  half_t h;
+  __builtin_memcpy(&h, &u, 2);
+  return h;
 }
 
 // Accumulate one quantised tile: 512 tokens x D channels.  A lane owns 8 consecutive tokens: half a
@@ -172,9 +194,9 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
   const uint32_t wofs = (ts / PF) * 4u;  // byte offset of this lane's first word inside a row
   const uint32_t gofs = (ts >> 5) * 2u;  // byte offset of this lane's group inside a scale/zero row
   const int sh2 = (BITS == 2) ? (int)((ts >> 3) & 1) * 16 : 0;  // which half of the 2-bit word
-  const uint32_t *code = (const uint32_t *)sg.data + (int64_t)bh * D * wpr;
-  const half_t *sc = sg.scale + (int64_t)bh * D * gpr;
-  const half_t *zr = sg.zero + (int64_t)bh * D * gpr;
+  const rsrc_t rc = make_rsrc((const uint32_t *)sg.data + (int64_t)bh * D * wpr, (uint32_t)D * wpr * 4u);
+  const rsrc_t rs = make_rsrc(sg.scale + (int64_t)bh * D * gpr, (uint32_t)D * gpr * 2u);
+  const rsrc_t rz = make_rsrc(sg.zero + (int64_t)bh * D * gpr, (uint32_t)D * gpr * 2u);
   const int DP = D >> 1;
 #pragma unroll 1
   for (int dp0 = wave; dp0 < DP; dp0 += QK_WAVES * QK_UNR) {
@@ -183,18 +205,17 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
 #pragma unroll
     for (int k = 0; k < QK_UNR; ++k) {
       const int dpk = dp0 + QK_WAVES * k;
-      const uint32_t d = 2u * (uint32_t)(dpk < DP ? dpk : dp0);    // uniform; past-the-end pairs reload dp0
-      const uint32_t *c0 = code + (size_t)d * wpr, *c1 = c0 + wpr;  // uniform row bases
-      const half_t *sa = sc + (size_t)d * gpr, *za = zr + (size_t)d * gpr;
+      const uint32_t d = 2u * (uint32_t)(dpk < DP ? dpk : dp0);  // uniform; past-the-end pairs reload dp0
+      const uint32_t crow = d * wpr * 4u, grow = d * gpr * 2u;   // scalar row offsets
 #pragma unroll
       for (int j = 0; j < NW; ++j) {
-        w0[k][j] = ld_u32(c0, wofs + 4 * j);
-        w1[k][j] = ld_u32(c1, wofs + 4 * j);
+        w0[k][j] = buf_u32(rc, wofs + 4 * j, crow);
+        w1[k][j] = buf_u32(rc, wofs + 4 * j, crow + wpr * 4u);
       }
-      s0[k] = ld_f16(sa, gofs);
-      s1[k] = ld_f16(sa + gpr, gofs);
-      z0[k] = ld_f16(za, gofs);
-      z1[k] = ld_f16(za + gpr, gofs);
+      s0[k] = buf_f16(rs, gofs, grow);
+      s1[k] = buf_f16(rs, gofs, grow + gpr * 2u);
+      z0[k] = buf_f16(rz, gofs, grow);
+      z1[k] = buf_f16(rz, gofs, grow + gpr * 2u);
     }
     HQ_LOADS_ABOVE();
 #pragma unroll
@@ -280,10 +301,16 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
 template <int NREP>
 __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int bh, int b, int hkv, int D,
                                                int Hq, int64_t Tall, int wave, int lane, const half2_t *q2s,
-                                               half_t *__restrict__ scores) {
+                                               half_t *__restrict__ scores, const FuseArgs &fz, float *red) {
   const int64_t n = sg.n_tokens;
   const half_t *kb = (const half_t *)sg.data + (int64_t)bh * n * D;
   const int DP = D >> 1;
+  float m_run[NREP], l_run[NREP];  // running softmax statistics of this wave's tokens (fused mode)
+#pragma unroll
+  for (int h = 0; h < NREP; ++h) {
+    m_run[h] = -INFINITY;
+    l_run[h] = 0.f;
+  }
 #pragma unroll 1
   for (int k = 0; k < 64 / QK_WAVES; ++k) {
     const int64_t t = (int64_t)tile * 64 + wave * (64 / QK_WAVES) + k;
@@ -296,13 +323,37 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
 #pragma unroll
       for (int h = 0; h < NREP; ++h) part[h] = __builtin_amdgcn_fdot2(kk, q2s[dp * NREP + h], part[h], false);
     }
+    const int64_t pos = sg.idx ? sg.idx[t] : sg.pos_base + t;
 #pragma unroll
-    for (int h = 0; h < NREP; ++h) part[h] = wave_sum(part[h]);
+    for (int h = 0; h < NREP; ++h) {
+      half_t r = (half_t)wave_sum(part[h]);
+      if (fz.stats) {
+        r = (half_t)((float)r * fz.inv_sqrt_d);
+        const float x = (float)r, mn = fmaxf(m_run[h], x);
+        l_run[h] = l_run[h] * __expf(m_run[h] - mn) + __expf(x - mn);
+        m_run[h] = mn;
+      }
+      if (lane == 0) scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = r;
+    }
+  }
+  if (fz.stats) {  // one (m, l) pair per head for the whole 64-token tile
     if (lane == 0) {
-      const int64_t pos = sg.idx ? sg.idx[t] : sg.pos_base + t;
 #pragma unroll
-      for (int h = 0; h < NREP; ++h)
-        scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = (half_t)part[h];
+      for (int h = 0; h < NREP; ++h) {
+        red[(wave * NREP + h) * 2 + 0] = m_run[h];
+        red[(wave * NREP + h) * 2 + 1] = l_run[h];
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < NREP) {
+      const int h = threadIdx.x;
+      float m = -INFINITY, l = 0.f;
+      for (int w = 0; w < QK_WAVES; ++w) m = fmaxf(m, red[(w * NREP + h) * 2]);
+      for (int w = 0; w < QK_WAVES; ++w) {
+        const float lw = red[(w * NREP + h) * 2 + 1];
+        if (lw > 0.f) l += lw * __expf(red[(w * NREP + h) * 2] - m);
+      }
+      fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
     }
   }
 }
@@ -312,7 +363,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
 template <int NREP>
 __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
                                                                half_t *__restrict__ scores, int Hq,
-                                                               int Hkv, int D, int64_t Tall) {
+                                                               int Hkv, int D, int64_t Tall, FuseArgs fz) {
   extern __shared__ float smem[];
   float *red = smem;                                                        // QK_WAVES * 2 * 8 * 64 floats
   half2_t *q2s = reinterpret_cast<half2_t *>(smem + QK_WAVES * 2 * QK_TPL * 64);  // D/2 x NREP pairs (q[d], q[d+1])
@@ -345,7 +396,7 @@ __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, cons
   }
   __syncthreads();
   if (tm) {
-    qk_f16_tm_tile<NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores);
+    qk_f16_tm_tile<NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
     return;
   }
 
@@ -375,27 +426,44 @@ __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, cons
 #pragma unroll
       for (int i = 0; i < QK_TPL; ++i) red[((wave * RH + j) * QK_TPL + i) * 64 + lane] = acc[h0 + j][i];
     __syncthreads();
-    if (wave < RH && t0 < n) {
+    if (wave < RH) {
       const int h = h0 + wave;
       half_t v[QK_TPL];
+      float m_lane = -INFINITY;
 #pragma unroll
       for (int i = 0; i < QK_TPL; ++i) {
         float a = 0.f;
 #pragma unroll
         for (int w = 0; w < QK_WAVES; ++w) a += red[((w * RH + wave) * QK_TPL + i) * 64 + lane];
         v[i] = (half_t)a;
+        if (fz.stats) {  // the fp16 steps of the reference epilogue: round the score, scale, round again
+          v[i] = (half_t)((float)v[i] * fz.inv_sqrt_d);
+          if (t0 + i < n) m_lane = fmaxf(m_lane, (float)v[i]);
+        }
       }
-      half_t *row = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
-      // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
-      // 128-bit store per head row; otherwise 2-byte scatters through idx
-      if (contig && (((uintptr_t)(row + pos[0])) & 15) == 0) {
-        uint4 raw;
-        __builtin_memcpy(&raw, v, 16);
-        *reinterpret_cast<uint4 *>(row + pos[0]) = raw;
-      } else {
+      if (fz.stats) {
+        const float m = wave_max(m_lane);
+        float l_lane = 0.f;
 #pragma unroll
         for (int i = 0; i < QK_TPL; ++i)
-          if (t0 + i < n) row[pos[i]] = v[i];
+          if (t0 + i < n) l_lane += __expf((float)v[i] - m);
+        const float l = wave_sum(l_lane);
+        if (lane == 0)
+          fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+      }
+      if (t0 < n) {
+        half_t *row = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+        // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
+        // 128-bit store per head row; otherwise 2-byte scatters through idx
+        if (contig && (((uintptr_t)(row + pos[0])) & 15) == 0) {
+          uint4 raw;
+          __builtin_memcpy(&raw, v, 16);
+          *reinterpret_cast<uint4 *>(row + pos[0]) = raw;
+        } else {
+#pragma unroll
+          for (int i = 0; i < QK_TPL; ++i)
+            if (t0 + i < n) row[pos[i]] = v[i];
+        }
       }
     }
   }
@@ -532,7 +600,8 @@ struct PvStage {
 // stage p (gathered through idx) and, for quantised classes, scale/zero of tokens [t0, t0+nt)
 template <int NREP, int NG, bool QUANT>
 __device__ __forceinline__ void pv_stage(const SegDev &sg, int64_t t0, int nt, int bh,
-                                         const half_t *const (&prow)[NREP], PvStage<NREP, NG> &st) {
+                                         half_t *const (&prow)[NREP], PvStage<NREP, NG> &st, bool fused,
+                                         const float *sm_ml) {
   const int ntp = (nt + 1) >> 1;
   const int64_t *ip = sg.idx;
   for (int tp = threadIdx.x; tp < ntp; tp += PV_THREADS) {
@@ -549,6 +618,18 @@ __device__ __forceinline__ void pv_stage(const SegDev &sg, int64_t t0, int nt, i
     for (int h = 0; h < NREP; ++h) {
       va[h] = prow[h][pa];
       vb[h] = prow[h][pb];
+    }
+    if (fused) {
+      // the row holds scaled logits: p = rnd16(exp(x - M) / L), written back for the caller.  Every
+      // position belongs to exactly one token of exactly one V class, so nobody else touches it.
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) {
+        const float M = sm_ml[2 * h], invL = sm_ml[2 * h + 1];
+        va[h] = (half_t)(__expf((float)va[h] - M) * invL);
+        vb[h] = (half_t)(__expf((float)vb[h] - M) * invL);
+        prow[h][pa] = va[h];
+        if (has_b) prow[h][pb] = vb[h];
+      }
     }
 #pragma unroll
     for (int h = 0; h < NREP; ++h) st.p2[tp][h] = pack_h2(va[h], has_b ? vb[h] : (half_t)0);
@@ -571,8 +652,8 @@ __device__ __forceinline__ void pv_stage(const SegDev &sg, int64_t t0, int nt, i
 // tokens needs only two butterfly steps across lanes.
 template <int BITS, int NREP, int D>
 __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh, int wave, int lane,
-                                         const half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
-                                         float (&acc)[NREP][PV_CPL]) {
+                                         half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
+                                         float (&acc)[NREP][PV_CPL], bool fused, const float *sm_ml) {
   static_assert(D == 128, "16 lanes x 8 channels cover one token row");
   constexpr int WPL = BITS == 16 ? 4 : (BITS == 8 ? 2 : 1);  // 32-bit words per lane per token
   constexpr int ROWW = D * BITS / 32;                         // 32-bit words per token row
@@ -587,8 +668,8 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
     const int ntp = (nt + 1) >> 1;
     const int nsteps = (ntp + 4 * PV_WAVES - 1) / (4 * PV_WAVES);
     __syncthreads();  // previous block fully consumed
-    if (BITS == 16) pv_stage<NREP, D / 32, false>(sg, t0, nt, bh, prow, st);
-    else pv_stage<NREP, D / 32, true>(sg, t0, nt, bh, prow, st);
+    if (BITS == 16) pv_stage<NREP, D / 32, false>(sg, t0, nt, bh, prow, st, fused, sm_ml);
+    else pv_stage<NREP, D / 32, true>(sg, t0, nt, bh, prow, st, fused, sm_ml);
     __syncthreads();
 #pragma unroll 1
     for (int s0 = 0; s0 < nsteps; s0 += PV_UNR) {
@@ -655,12 +736,13 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
 }
 
 template <int NREP, int D>
-__global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, const half_t *__restrict__ p,
+__global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half_t *__restrict__ p,
                                                                float *__restrict__ partial, int Hq, int Hkv,
                                                                int64_t Tall, int64_t chunk_tokens,
-                                                               int64_t n_bhq) {
+                                                               int64_t n_bhq, FuseArgs fz) {
   __shared__ float red[PV_WAVES * NREP * D];
   __shared__ PvStage<NREP, D / 32> st;
+  __shared__ float sm_ml[2 * NREP];  // fused mode: (max, 1 / sum exp) of each query head's row
   const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads
   if ((int)blockIdx.x >= sg.n_units) return;  // uniform: grid.x is the largest chunk count of any segment
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -669,19 +751,39 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, cons
   const int chunk_id = sg.unit_begin + (int)blockIdx.x;
   const int64_t c0 = (int64_t)blockIdx.x * chunk_tokens;
   const int64_t c1 = min(c0 + chunk_tokens, sg.n_tokens);
-  const half_t *prow[NREP];
+  const bool fused = fz.stats != nullptr;
+  half_t *prow[NREP];
 #pragma unroll
   for (int h = 0; h < NREP; ++h) prow[h] = p + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+  if (fused) {
+    // merge the per-tile (m, l) pairs of each head: wave w serves heads w, w+4, ...
+    for (int h = wave; h < NREP; h += PV_WAVES) {
+      const float2 *sp = fz.stats + ((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat;
+      float m = -INFINITY;
+      for (int e = lane; e < fz.n_stat; e += 64) m = fmaxf(m, sp[e].x);
+      m = wave_max(m);
+      float l = 0.f;
+      for (int e = lane; e < fz.n_stat; e += 64) {
+        const float2 v = sp[e];
+        l += v.y * __expf(v.x - m);
+      }
+      l = wave_sum(l);
+      if (lane == 0) {
+        sm_ml[2 * h] = m;
+        sm_ml[2 * h + 1] = 1.0f / l;
+      }
+    }
+  }
   float acc[NREP][PV_CPL];
 #pragma unroll
   for (int h = 0; h < NREP; ++h)
 #pragma unroll
     for (int i = 0; i < PV_CPL; ++i) acc[h][i] = 0.f;
-  switch (sg.bits) {
-    case 2: pv_chunk<2, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc); break;
-    case 4: pv_chunk<4, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc); break;
-    case 8: pv_chunk<8, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc); break;
-    default: pv_chunk<16, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc);
+  switch (sg.bits) {  // (the first barrier inside pv_chunk also publishes sm_ml)
+    case 2: pv_chunk<2, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
+    case 4: pv_chunk<4, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
+    case 8: pv_chunk<8, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
+    default: pv_chunk<16, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
   }
   // lanes 16 and 32 apart hold the same channels of other tokens
   const int cl = lane & 15;
@@ -792,14 +894,14 @@ static int check_heads(const char *who, int64_t B, int64_t Hq, int64_t Hkv, int6
 }
 
 static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
-                     int64_t D, int64_t Tall, hipStream_t st) {
+                     int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st) {
   if (tb.total_units == 0) return HQEKV_OK;
   const int nrep = (int)(Hq / Hkv);
   dim3 grid((unsigned)tb.max_units, (unsigned)(B * Hkv), (unsigned)tb.nseg), block(QK_THREADS);
   const size_t shmem = (size_t)(nrep * D + QK_WAVES * 2 * QK_TPL * 64) * sizeof(float);
 #define LAUNCH(N_)                                                                                    \
   hipLaunchKernelGGL(qk_hybrid_kernel<N_>, grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
-                     (int)Hq, (int)Hkv, (int)D, Tall)
+                     (int)Hq, (int)Hkv, (int)D, Tall, fz)
   switch (nrep) {
     case 1: LAUNCH(1); break;
     case 2: LAUNCH(2); break;
@@ -828,15 +930,15 @@ static int64_t seg_total_tokens(const hqekv_seg *segs, int nseg) {
   return n;
 }
 
-static int launch_pv(const SegTable &tb, int64_t chunk, const void *p, void *out, float *partial, int64_t B,
-                     int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, hipStream_t st) {
+static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, float *partial, int64_t B,
+                     int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st) {
   const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
   if (tb.total_units > 0) {
     dim3 grid((unsigned)tb.max_units, (unsigned)(B * Hkv), (unsigned)tb.nseg), block(PV_THREADS);
 #define LAUNCH(N_, D_)                                                                                   \
-  hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_>), grid, block, 0, st, tb, (const half_t *)p, partial, (int)Hq, \
-                     (int)Hkv, Tall, chunk, n_bhq)
+  hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
+                     (int)Hkv, Tall, chunk, n_bhq, fz)
 #define LAUNCH_D(N_) LAUNCH(N_, 128)
     switch (nrep) {
       case 1: LAUNCH_D(1); break;
@@ -867,7 +969,7 @@ extern "C" int hqekv_qk_hybrid(const hqekv_seg *segs, int nseg, const void *q, v
   SegTable tb{};
   rc = build_table(segs, nseg, true, D, 0, Tall, &tb, "qk_hybrid");
   if (rc) return rc;
-  return launch_qk(tb, q, scores, B, Hq, Hkv, D, Tall, (hipStream_t)stream);
+  return launch_qk(tb, q, scores, B, Hq, Hkv, D, Tall, FuseArgs{}, (hipStream_t)stream);
 }
 
 extern "C" int hqekv_scale_softmax(void *scores, const void *mask, int64_t mask_row_stride, int64_t n_rows,
@@ -918,20 +1020,87 @@ extern "C" int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, v
     return fail(HQEKV_E_WORKSPACE, "pv_hybrid: workspace %lld bytes < %lld needed", (long long)workspace_bytes,
                 (long long)need);
   if ((uintptr_t)workspace & 15) return fail(HQEKV_E_ALIGN, "pv_hybrid: workspace not 16-byte aligned");
-  return launch_pv(tb, chunk, p, out, (float *)workspace, B, Hq, Hkv, D, Tall, (hipStream_t)stream);
+  return launch_pv(tb, chunk, const_cast<void *>(p), out, (float *)workspace, B, Hq, Hkv, D, Tall, FuseArgs{},
+                   (hipStream_t)stream);
+}
+
+static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+struct DecodeLayout {  // carve-up of the caller's workspace
+  int64_t chunk, partial_bytes, stats_off, stats_bytes, total;
+  int64_t n_stat;
+};
+
+static int decode_layout(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v, int64_t B,
+                         int64_t Hq, int64_t Hkv, int64_t D, DecodeLayout *L) {
+  if (n_k < 0 || n_k > HQEKV_MAX_SEGS || n_v < 0 || n_v > HQEKV_MAX_SEGS || (n_k > 0 && !k_segs) ||
+      (n_v > 0 && !v_segs) || B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0)
+    return HQEKV_E_ARG;
+  L->chunk = pv_chunk_tokens(seg_total_tokens(v_segs, n_v), B * Hkv);
+  int64_t chunks = 0;
+  for (int k = 0; k < n_v; ++k)
+    if (v_segs[k].n_tokens > 0) chunks += (v_segs[k].n_tokens + L->chunk - 1) / L->chunk;
+  if (chunks == 0) chunks = 1;
+  int64_t tiles = 0;
+  for (int k = 0; k < n_k; ++k)
+    if (k_segs[k].n_tokens > 0) {
+      const int64_t per = qk_tile_tokens(k_segs[k].bits, k_segs[k].bits == 16 && k_segs[k].token_major);
+      tiles += (k_segs[k].n_tokens + per - 1) / per;
+    }
+  if (tiles == 0) tiles = 1;
+  L->n_stat = tiles;
+  L->partial_bytes = align_up(chunks * B * Hq * D * (int64_t)sizeof(float), 256);
+  L->stats_off = L->partial_bytes;
+  L->stats_bytes = align_up(B * Hq * tiles * (int64_t)sizeof(float2), 256);
+  L->total = L->stats_off + L->stats_bytes;
+  return HQEKV_OK;
+}
+
+extern "C" int64_t hqekv_decode_workspace_bytes(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs,
+                                                int n_v, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
+  DecodeLayout L;
+  if (decode_layout(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D, &L)) return -1;
+  return L.total;
 }
 
 extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
                                  const void *q, const void *mask, int64_t mask_row_stride, void *attn_weights,
                                  void *attn_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall,
-                                 void *workspace, int64_t workspace_bytes, void *stream) {
-  int rc = hqekv_qk_hybrid(k_segs, n_k, q, attn_weights, B, Hq, Hkv, D, Tall, stream);
+                                 void *workspace, int64_t workspace_bytes, int flags, void *stream) {
+  int rc = check_heads("decode_attn", B, Hq, Hkv, D);
   if (rc) return rc;
-  const float inv = 1.0f / (float)sqrt((double)D);
-  rc = hqekv_scale_softmax(attn_weights, mask, mask_row_stride, B * Hq, Tall, inv, stream);
+  if (D != 128) return fail(HQEKV_E_UNSUPPORTED, "decode_attn: head_dim %lld (supported: 128)", (long long)D);
+  if (!q || !attn_weights || !attn_out || Tall <= 0) return fail(HQEKV_E_ARG, "decode_attn: null pointer or Tall <= 0");
+  DecodeLayout L;
+  if (decode_layout(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D, &L)) return fail(HQEKV_E_ARG, "decode_attn: bad segment tables");
+  if (!workspace || workspace_bytes < L.total)
+    return fail(HQEKV_E_WORKSPACE, "decode_attn: workspace %lld bytes < %lld needed", (long long)workspace_bytes,
+                (long long)L.total);
+  if ((uintptr_t)workspace & 255) return fail(HQEKV_E_ALIGN, "decode_attn: workspace not 256-byte aligned");
+  SegTable kt{}, vt{};
+  rc = build_table(k_segs, n_k, true, D, 0, Tall, &kt, "decode_attn(K)");
   if (rc) return rc;
-  return hqekv_pv_hybrid(v_segs, n_v, attn_weights, attn_out, B, Hq, Hkv, D, Tall, workspace, workspace_bytes,
-                         stream);
+  rc = build_table(v_segs, n_v, false, D, L.chunk, Tall, &vt, "decode_attn(V)");
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char *ws = (char *)workspace;
+  // The softmax can ride inside the two GEMV launches when nothing is added to the logits and every
+  // position is produced by exactly one K token and consumed by exactly one V token.
+  const bool fuse = (flags & HQEKV_FUSE_SOFTMAX) && !mask && seg_total_tokens(k_segs, n_k) == Tall &&
+                    seg_total_tokens(v_segs, n_v) == Tall && kt.total_units > 0 && vt.total_units > 0;
+  FuseArgs fz{};
+  if (fuse) {
+    fz.stats = (float2 *)(ws + L.stats_off);
+    fz.n_stat = (int32_t)kt.total_units;
+    fz.inv_sqrt_d = 1.0f / (float)sqrt((double)D);
+  }
+  rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st);
+  if (rc) return rc;
+  if (!fuse) {
+    rc = hqekv_scale_softmax(attn_weights, mask, mask_row_stride, B * Hq, Tall, 1.0f / (float)sqrt((double)D), stream);
+    if (rc) return rc;
+  }
+  return launch_pv(vt, L.chunk, attn_weights, attn_out, (float *)ws, B, Hq, Hkv, D, Tall, fz, st);
 }
 
 // ------------------------------------------------------------------ per-class GEMV on the same kernels

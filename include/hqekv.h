@@ -144,15 +144,29 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
                     int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, void *workspace,
                     int64_t workspace_bytes, void *stream);
 
-/* The whole decode-attention layer-step: qk_hybrid -> scale_softmax -> pv_hybrid on one
- * stream.  Replaces qkv_matmul / qkv_matmul_hq (quant/quant_matmul_hq.py:23-174) and
- * qkv_matmul_hqe_2 (quant/hqe_matmul.py:354-451).  attn_weights (B,Hq,Tall) fp16 receives
- * the probabilities (the caller's importance tracker needs them, model/llama_hqe.py:200).
+/* The whole decode-attention layer-step on one stream.  Replaces qkv_matmul / qkv_matmul_hq
+ * (quant/quant_matmul_hq.py:23-174) and qkv_matmul_hqe_2 (quant/hqe_matmul.py:354-451).
+ * attn_weights (B,Hq,Tall) fp16 receives the probabilities (the caller's importance tracker needs
+ * them, model/llama_hqe.py:200); attn_out is (B,Hq,D) fp16.
+ *
+ * flags = 0: three launches plus the combine (qk_hybrid -> scale_softmax -> pv_hybrid), valid for any
+ *   idx arrays and any mask.
+ * flags & HQEKV_FUSE_SOFTMAX: no softmax launch.  The q.K^T launch stores scaled logits and per-tile softmax
+ *   statistics, the p.V launch normalises while it gathers; the fixed-order combine stays a third,
+ *   small launch.  REQUIRES that the idx arrays of the K segments, and those of the V segments, each cover
+ *   every position in [0, Tall) exactly once (true for every cache the reference's cache policy builds);
+ *   taken only when mask == NULL and both segment lists hold exactly Tall tokens, otherwise the call
+ *   silently runs the flags = 0 path.
+ * The workspace must hold hqekv_decode_workspace_bytes() bytes, 256-byte aligned; its contents need
+ * not be initialised and are not preserved.  Calls that share a workspace must not overlap in time.
  */
+#define HQEKV_FUSE_SOFTMAX 1
+int64_t hqekv_decode_workspace_bytes(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
+                                     int64_t B, int64_t Hq, int64_t Hkv, int64_t D);
 int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
                       const void *q, const void *mask, int64_t mask_row_stride,
                       void *attn_weights, void *attn_out, int64_t B, int64_t Hq, int64_t Hkv,
-                      int64_t D, int64_t Tall, void *workspace, int64_t workspace_bytes,
+                      int64_t D, int64_t Tall, void *workspace, int64_t workspace_bytes, int flags,
                       void *stream);
 
 #ifdef __cplusplus

@@ -41,8 +41,10 @@ CASES = [
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: f"B{c['B']}Hq{c['Hq']}T{c['T']}D{c['D']}s{c['seed']}")
 @pytest.mark.parametrize("permute", [False, True], ids=["blockidx", "randperm"])
-def test_hqe2_matches_oracle(dev, case, permute):
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "general"])
+def test_hqe2_matches_oracle(dev, case, permute, fused, monkeypatch):
     from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    monkeypatch.setenv("HQEKV_UNFUSED", "0" if fused else "1")
     q, cache = _case(permute=permute, **case)
     w_ref, o_ref = O.qkv_matmul(q, cache, None, case["D"], use_mask=False)
     _, o_ref32 = O.qkv_matmul(q, cache, None, case["D"], use_mask=False, round_per_class=False)
@@ -171,3 +173,20 @@ def test_scale_softmax_rows(dev, Tall, with_mask):
                                          1.0 / 128 ** 0.5, _lib.stream_ptr(dev))
     _lib.check(rc, "scale_softmax")
     torch.testing.assert_close(sd.float().cpu(), ref.float(), rtol=RTOL, atol=1e-5)
+
+
+def test_fused_path_is_deterministic_and_reusable(dev):
+    """Repeated calls on one plan (same workspace, uninitialised at first) give bit-identical results,
+    and the fused path matches the general path within the tolerance."""
+    from hqekv_amd.attention import DecodePlan
+    q, cache = _case(**CASES[1])
+    c = synth.cache_to(cache, dev)
+    plan = DecodePlan(q.to(dev), c, flags=1)
+    ref = DecodePlan(q.to(dev), c, flags=0)
+    w0, o0 = [x.clone() for x in plan.run(q.to(dev))]
+    for _ in range(5):
+        w, o = plan.run(q.to(dev))
+        assert torch.equal(w, w0) and torch.equal(o, o0)
+    wr, orr = ref.run(q.to(dev))
+    _close(w0, wr.cpu(), "fused vs general attn_weights")
+    _close(o0, orr.cpu(), "fused vs general attn_output")
