@@ -17,6 +17,9 @@ _LIB_PATH = Path(os.environ.get("HQEKV_LIB", _PKG / "libhqekv.so"))
 
 MAX_SEGS = 8
 FUSE_SOFTMAX = 1
+ONLY_QK = 0x100
+ONLY_PV = 0x200
+ONLY_COMBINE = 0x400
 
 # every symbol include/hqekv.h declares
 EXPORTS = (

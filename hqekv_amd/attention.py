@@ -235,12 +235,13 @@ class DecodePlan:
         self._lib = _lib.load()
         self.inv_sqrt_d = 1.0 / (D ** 0.5)
 
-    def run(self, q: torch.Tensor, stream: Optional[int] = None):
+    def run(self, q: torch.Tensor, stream: Optional[int] = None, only: int = 0):
+        """``only`` = _lib.ONLY_QK / ONLY_PV / ONLY_COMBINE runs one part of the step (per-kernel timing)."""
         st = _lib.stream_ptr(self.dev) if stream is None else stream
         rc = self._lib.hqekv_decode_attn(
             self.k_segs, self.n_k, self.v_segs, self.n_v, q.data_ptr(), self.mask_ptr, self.mask_stride,
             self.weights.data_ptr(), self.out.data_ptr(), self.B, self.Hq, self.Hkv, self.D, self.Tall,
-            self.ws.data_ptr(), self.ws.numel() * 4, self.flags, st)
+            self.ws.data_ptr(), self.ws.numel() * 4, self.flags | only, st)
         if rc:
             _lib.check(rc, "DecodePlan.run")
         return self.weights, self.out

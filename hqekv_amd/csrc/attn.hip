@@ -931,10 +931,11 @@ static int64_t seg_total_tokens(const hqekv_seg *segs, int nseg) {
 }
 
 static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, float *partial, int64_t B,
-                     int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st) {
+                     int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st,
+                     int stages = 3) {
   const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
-  if (tb.total_units > 0) {
+  if (tb.total_units > 0 && (stages & 1)) {
     dim3 grid((unsigned)tb.max_units, (unsigned)(B * Hkv), (unsigned)tb.nseg), block(PV_THREADS);
 #define LAUNCH(N_, D_)                                                                                   \
   hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
@@ -951,6 +952,7 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
     int rc = check_launch("pv_hybrid_kernel");
     if (rc) return rc;
   }
+  if (!(stages & 2)) return HQEKV_OK;
   hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq), dim3(128 * CB_SLICES), 0, st, partial,
                      (half_t *)out, (int)tb.total_units, n_bhq, (int)D);
   return check_launch("pv_combine_kernel");
@@ -1094,13 +1096,19 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
     fz.n_stat = (int32_t)kt.total_units;
     fz.inv_sqrt_d = 1.0f / (float)sqrt((double)D);
   }
-  rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st);
-  if (rc) return rc;
-  if (!fuse) {
-    rc = hqekv_scale_softmax(attn_weights, mask, mask_row_stride, B * Hq, Tall, 1.0f / (float)sqrt((double)D), stream);
+  const int only = flags & (HQEKV_ONLY_QK | HQEKV_ONLY_PV | HQEKV_ONLY_COMBINE);
+  const bool only_qk = only == HQEKV_ONLY_QK;
+  if (only == 0 || only_qk) {
+    rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st);
     if (rc) return rc;
+    if (!fuse) {
+      rc = hqekv_scale_softmax(attn_weights, mask, mask_row_stride, B * Hq, Tall, 1.0f / (float)sqrt((double)D), stream);
+      if (rc) return rc;
+    }
   }
-  return launch_pv(vt, L.chunk, attn_weights, attn_out, (float *)ws, B, Hq, Hkv, D, Tall, fz, st);
+  if (only_qk) return HQEKV_OK;
+  const int stages = only == HQEKV_ONLY_PV ? 1 : (only == HQEKV_ONLY_COMBINE ? 2 : 3);
+  return launch_pv(vt, L.chunk, attn_weights, attn_out, (float *)ws, B, Hq, Hkv, D, Tall, fz, st, stages);
 }
 
 // ------------------------------------------------------------------ per-class GEMV on the same kernels

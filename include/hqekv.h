@@ -159,8 +159,14 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
  *   silently runs the flags = 0 path.
  * The workspace must hold hqekv_decode_workspace_bytes() bytes, 256-byte aligned; its contents need
  * not be initialised and are not preserved.  Calls that share a workspace must not overlap in time.
+ * HQEKV_ONLY_QK / HQEKV_ONLY_PV / HQEKV_ONLY_COMBINE run one part of the call (q.K^T [+ softmax] / the p.V
+ * kernel / the combine) so that each can be timed on its own; the later parts expect the earlier ones to
+ * have run on the same buffers.
  */
 #define HQEKV_FUSE_SOFTMAX 1
+#define HQEKV_ONLY_QK 0x100
+#define HQEKV_ONLY_PV 0x200
+#define HQEKV_ONLY_COMBINE 0x400
 int64_t hqekv_decode_workspace_bytes(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
                                      int64_t B, int64_t Hq, int64_t Hkv, int64_t D);
 int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,

@@ -1,0 +1,240 @@
+"""Pins for the CPU oracle: known answers, closed forms, invariants and brute force chosen so that a
+dropped term, a wrong shift or a transposed operand fails at least one of them.  No GPU needed."""
+import json
+import math
+from pathlib import Path
+
+import pytest
+import torch
+
+from oracle import hqe_oracle as O
+
+GOLDEN = Path(__file__).parent / "golden"
+
+
+# ------------------------------------------------------------------ pack / unpack
+def test_pack_known_answer_lsb_first():
+    q = torch.tensor([0, 1, 2, 3] * 4, dtype=torch.int32).reshape(1, 1, 1, 16)
+    w = O.pack_along_last_dim(q, 2)
+    assert w.item() == -454761244 and (w.item() & 0xFFFFFFFF) == 0xE4E4E4E4
+    # one code in slot i sets exactly bits [i*b, i*b+b)
+    for bit in (2, 4, 8):
+        pf = 32 // bit
+        for i in range(pf):
+            q = torch.zeros(1, 1, 1, pf, dtype=torch.int32)
+            q[..., i] = 2 ** bit - 1
+            assert (O.pack_along_last_dim(q, bit).item() & 0xFFFFFFFF) == ((2 ** bit - 1) << (i * bit))
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_pack_unpack_round_trip_every_value_in_every_slot(bit):
+    pf = 32 // bit
+    vals = torch.arange(2 ** bit, dtype=torch.int32)
+    q = torch.stack([vals.roll(s) for s in range(pf)], dim=-1).reshape(1, 1, -1, pf)  # every value in every slot
+    code = O.pack_along_last_dim(q, bit)
+    assert code.shape == (1, 1, 2 ** bit, 1) and code.dtype == torch.int32
+    assert torch.equal(O.unpack_codes(code, bit), q)
+    assert torch.equal(O.unpack_along_last_dim(code, bit), q.to(torch.float16))
+
+
+def test_golden_pack_vectors():
+    g = json.loads((GOLDEN / "pack_vectors.json").read_text())
+    for case in g["cases"]:
+        q = torch.tensor(case["codes"], dtype=torch.int32).reshape(1, 1, 1, -1)
+        w = O.pack_along_last_dim(q, case["bit"]).flatten().tolist()
+        assert [x & 0xFFFFFFFF for x in w] == case["words_u32"], case["name"]
+
+
+# ------------------------------------------------------------------ quantise
+def test_quantise_known_answer_arange():
+    """The reference's own smoke input (quant/pack_unpack.py:382): arange(128), groups of 32, 2 bit.
+    mn = 32g, mx - mn = 31, scale = fp16(31/3) = 10.3359375; codes by hand: k/10.3359375 rounded half-even."""
+    x = torch.arange(0, 128, dtype=torch.float16).reshape(1, 1, 1, -1)
+    for mode in ("recip", "true"):
+        code, scale, mn = O.uniform_group_quantize_pack_last_dim(x, 32, 2, mode)
+        assert scale.flatten().tolist() == [10.3359375] * 4
+        assert mn.flatten().tolist() == [0.0, 32.0, 64.0, 96.0]
+        expect = [0] * 6 + [1] * 10 + [2] * 10 + [3] * 6
+        assert O.unpack_codes(code, 2).flatten().tolist() == expect * 4
+    g = json.loads((GOLDEN / "quant_arange128.json").read_text())
+    assert [w & 0xFFFFFFFF for w in code.flatten().tolist()] == g["words_u32_2bit"]
+
+
+def test_quantise_8bit_identity_on_integers():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randint(0, 256, (1, 2, 3, 64), generator=g).to(torch.float16)
+    x[..., 0], x[..., 31], x[..., 32], x[..., 63] = 0, 255, 0, 255  # every group spans exactly 0..255
+    code, scale, mn = O.uniform_group_quantize_pack_last_dim(x, 32, 8)
+    assert (scale == 1).all() and (mn == 0).all()
+    assert torch.equal(O.unpack_codes(code, 8), x.to(torch.int32))
+    assert torch.equal(O.uniform_group_dequantize_unpack_last_dim(code, scale, mn, 32, 8), x)
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+def test_quantise_invariants(bit):
+    g = torch.Generator().manual_seed(bit)
+    x = (torch.randn(2, 2, 16, 128, generator=g) * 3).half()
+    before = x.clone()
+    code, scale, mn = O.uniform_group_quantize_pack_last_dim(x, 32, bit)
+    assert torch.equal(x, before), "the oracle must not mutate its input"
+    c = O.unpack_codes(code, bit).reshape(2, 2, 16, 4, 32)
+    xg = x.reshape(2, 2, 16, 4, 32)
+    qmax = 2 ** bit - 1
+    assert c.min() >= 0 and c.max() <= qmax
+    assert torch.equal(mn, xg.min(-1)[0])                       # zero point is the group minimum
+    assert (c.gather(-1, xg.argmin(-1, keepdim=True)) == 0).all()   # the minimum maps to code 0
+    assert (c.gather(-1, xg.argmax(-1, keepdim=True)) == qmax).all()  # the maximum maps to the top code
+    dq = O.uniform_group_dequantize_unpack_last_dim(code, scale, mn, 32, bit).reshape(2, 2, 16, 4, 32)
+    err = (dq.float() - xg.float()).abs()
+    bound = scale.float().unsqueeze(-1) / 2 + 3 * 2.0 ** -11 * xg.float().abs().amax(-1, keepdim=True) + 1e-3
+    assert (err <= bound).all()
+    # monotone: a larger input never gets a smaller code within a group
+    order = xg.argsort(-1)
+    assert (c.gather(-1, order).diff(dim=-1) >= 0).all()
+
+
+def test_quantise_constant_group_and_scalar_division_modes():
+    x = torch.full((1, 1, 1, 32), 1.5, dtype=torch.float16)
+    code, scale, mn = O.uniform_group_quantize_pack_last_dim(x, 32, 4)
+    assert code.abs().sum() == 0 and scale.item() == 0 and mn.item() == 1.5
+    assert torch.equal(O.uniform_group_dequantize_unpack_last_dim(code, scale, mn, 32, 4), x)
+    # the two scalar-division rules differ by at most one fp16 ulp of the scale
+    g = torch.Generator().manual_seed(5)
+    y = torch.randn(1, 4, 64, 256, generator=g).half()
+    for bit in (2, 4, 8):
+        a = O.uniform_group_quantize_pack_last_dim(y, 32, bit, "recip")[1].float()
+        b = O.uniform_group_quantize_pack_last_dim(y, 32, bit, "true")[1].float()
+        assert ((a - b).abs() <= b.abs() * 2.0 ** -10).all()
+
+
+def test_dequantise_two_roundings_by_hand():
+    # code 3, scale 0.3333 (fp16 0.33325195), zero 100: fp16(3*0.33325195)=0.99951172, fp16(100.99951172)=101.0
+    code = O.pack_along_last_dim(torch.tensor([3] + [0] * 31, dtype=torch.int32).reshape(1, 1, 1, 32), 2)
+    s = torch.tensor(0.3333, dtype=torch.float16).reshape(1, 1, 1, 1)
+    z = torch.tensor(100.0, dtype=torch.float16).reshape(1, 1, 1, 1)
+    dq = O.uniform_group_dequantize_unpack_last_dim(code, s, z, 32, 2)
+    assert dq[0, 0, 0, 0].item() == 101.0 and dq[0, 0, 0, 1].item() == 100.0
+    # a case a single fused rounding gets wrong: 10 * fp16(0.1) = 0.999755859375 is a tie that rounds to
+    # 1.0; 2050 + 1.0 = 2051 is a tie (ulp 2) that rounds to the even 2052.  One rounding of the exact
+    # 2050.99976 would give 2050.
+    s2 = torch.tensor(0.0999755859375, dtype=torch.float16).reshape(1, 1, 1, 1)
+    z2 = torch.tensor(2050.0, dtype=torch.float16).reshape(1, 1, 1, 1)
+    code2 = O.pack_along_last_dim(torch.tensor([10] + [0] * 31, dtype=torch.int32).reshape(1, 1, 1, 32), 4)
+    dq2 = O.uniform_group_dequantize_unpack_last_dim(code2, s2, z2, 32, 4)
+    assert dq2[0, 0, 0, 0].item() == 2052.0
+
+
+# ------------------------------------------------------------------ GEMV
+def test_gemv_collapses_to_integer_matvec():
+    g = torch.Generator().manual_seed(1)
+    c = torch.randint(0, 8, (1, 2, 16, 64), generator=g, dtype=torch.int32)
+    q = torch.randint(-2, 3, (1, 4, 1, 16), generator=g).half()
+    code = O.pack_along_last_dim(c, 4)
+    s = torch.ones(1, 2, 16, 2, dtype=torch.float16)
+    z = torch.zeros_like(s)
+    out = O.gemv_uniform_group(32, q, code, s, z, 4)
+    exact = torch.matmul(q.long(), O.repeat_kv(c.long(), 2))
+    assert torch.equal(out.long(), exact)
+    # all codes zero: out = sum_k q_k * zero_k for every column of the group
+    z2 = torch.randn(1, 2, 16, 2, generator=g).half()
+    out0 = O.gemv_uniform_group(32, q, torch.zeros_like(code), s, z2, 4)
+    ref0 = torch.matmul(q.float(), O.repeat_kv(z2, 2).float()).half()
+    assert torch.equal(out0[..., 0:1], ref0[..., 0:1]) and torch.equal(out0[..., 63:64], ref0[..., 1:2])
+
+
+def test_repeat_kv_maps_query_head_to_kv_head():
+    x = torch.arange(3).reshape(1, 3, 1, 1).float()
+    assert O.repeat_kv(x, 2).flatten().tolist() == [0, 0, 1, 1, 2, 2]  # hq // n_rep
+
+
+# ------------------------------------------------------------------ hybrid attention
+def test_hybrid_all_fp16_equals_dense_attention_under_permutation():
+    g = torch.Generator().manual_seed(3)
+    B, Hq, Hkv, T, D = 1, 4, 2, 96, 32
+    q = torch.randn(B, Hq, 1, D, generator=g).half()
+    K = torch.randn(B, Hkv, T, D, generator=g).half()
+    V = torch.randn(B, Hkv, T, D, generator=g).half()
+    perm = torch.randperm(64, generator=g)
+    t = [None] * 42
+    t[0], t[1] = K[:, :, :64].transpose(2, 3).contiguous(), perm
+    t[2], t[3] = V[:, :, :64].contiguous(), perm.clone()
+    t[39], t[40], t[41] = K[:, :, 64:], V[:, :, 64:], T
+    w, o = O.qkv_matmul(q, tuple(t), None, D, use_mask=False, round_per_class=False)
+    Kp, Vp = K.clone(), V.clone()
+    Kp[:, :, perm], Vp[:, :, perm] = K[:, :, :64], V[:, :, :64]
+    s = torch.matmul(q.float(), O.repeat_kv(Kp, 2).transpose(2, 3).float()).half()
+    s = (s.float() * (torch.tensor(1.0) / torch.tensor(D ** 0.5))).half()
+    p = torch.softmax(s.float(), -1).half()
+    assert torch.equal(w, p)
+    torch.testing.assert_close(o.float(), torch.matmul(p.float(), O.repeat_kv(Vp, 2).float()), rtol=1e-3, atol=1e-3)
+    assert abs(float(w.float().sum(-1).mean()) - 1.0) < 2e-3
+
+
+def test_hybrid_single_class_equals_per_class_gemv():
+    g = torch.Generator().manual_seed(4)
+    B, Hq, Hkv, T, D = 1, 4, 1, 64, 32
+    q = torch.randn(B, Hq, 1, D, generator=g).half()
+    K = torch.randn(B, Hkv, T, D, generator=g).half()
+    V = torch.randn(B, Hkv, T, D, generator=g).half()
+    kc, ks, kz = O.uniform_group_quantize_pack_last_dim(K.transpose(2, 3).contiguous(), 32, 4)
+    vc, vs, vz = O.uniform_group_quantize_pack_last_dim(V, 32, 4)
+    idx = torch.arange(T)
+    t = [None] * 42
+    t[12], t[13], t[14], t[15] = kc, idx, ks, kz
+    t[16], t[17], t[18], t[19] = vc, idx.clone(), vs, vz
+    t[41] = T
+    w, o = O.qkv_matmul(q, tuple(t), None, D, use_mask=False)
+    s = O.gemv_uniform_group(32, q, kc, ks, kz, 4)
+    p = O._scale_clamp_softmax(s, D, None, "recip")
+    assert torch.equal(w, p)
+    assert torch.equal(o, O.gemv_uniform_group(32, p, vc, vs, vz, 4))
+
+
+def test_mask_and_errors():
+    q = torch.zeros(1, 2, 1, 32, dtype=torch.float16)
+    with pytest.raises(ValueError, match="invalid past_key_value"):
+        O.qkv_matmul(q, O.empty_cache(), None, 32)
+    with pytest.raises(ValueError, match="invalid quant_strategy"):
+        O.qkv_matmul(q, O.empty_cache(), None, 32, "bogus")
+    K = torch.randn(1, 1, 8, 32).half()
+    mask = torch.zeros(1, 1, 1, 8, dtype=torch.float16)
+    mask[..., :4] = torch.finfo(torch.float16).min
+    w, _ = O.qkv_matmul(q, O.empty_cache(K, K, 8), mask, 32)
+    assert (w[..., :4] == 0).all() and torch.allclose(w[..., 4:].float(), torch.full((1, 2, 1, 4), 0.25))
+
+
+# ------------------------------------------------------------------ policy helpers
+def test_make_sum_equal_closed_form():
+    a = torch.tensor([2, 0, 10, 10, 10, 5])
+    assert O.make_sum_equal(a, 35).tolist() == [2, 0, 10, 10, 8, 5]      # surplus 2 taken from index 4
+    assert O.make_sum_equal(a, 40).tolist() == [2, 0, 10, 10, 13, 5]     # deficit added to index 4
+    assert O.make_sum_equal(a, 25).tolist() == [2, 0, 10, 8, 0, 5]       # walks down when index 4 runs out
+    assert a.tolist() == [2, 0, 10, 10, 10, 5]
+
+
+def test_block_ranking_and_rerank_brute_force():
+    g = torch.Generator().manual_seed(9)
+    imp = torch.rand(8 * 32, generator=g)
+    idx = O.get_block_token_idx(32, 8, imp)
+    means = imp.reshape(8, 32).mean(-1)
+    assert idx.reshape(8, 32)[:, 0].div(32, rounding_mode="floor").tolist() == means.argsort(descending=True).tolist()
+    assert sorted(idx.tolist()) == list(range(256))
+    # survivors' ranks, brute force with Python sets
+    classes = [idx[:64], None, idx[64:160], idx[160:224]]   # idx[224:] evicted
+    out = O.rerank_after_eviction(classes)
+    alive = sorted(set(range(256)) - set(idx[224:].tolist()))
+    for c, o in zip(classes, out):
+        if c is None:
+            assert o is None
+        else:
+            assert o.tolist() == [alive.index(int(v)) for v in c.tolist()]
+    flat = sorted(v for o in out if o is not None for v in o.tolist())
+    assert flat == list(range(224))
+
+
+def test_token_range_closed_form():
+    v = torch.tensor([[[[1.0, -2.0, 3.0], [0.0, 0.5, 0.25]]]]).half()  # (1,1,2,3)
+    r = O.calculate_token_range(v, None)
+    assert r.tolist() == [5.0, 0.5]
+    assert O.calculate_token_range(v, r).tolist() == [5.0, 0.5, 5.0, 0.5]
+    assert O.calculate_token_range(None, r) is None
