@@ -1,0 +1,326 @@
+"""Class assignment and migration of the hybrid cache (host logic; the arithmetic runs in HIP kernels).
+
+One engine serves both generations of the reference's policy:
+  * ``KV_cache_hqe_2``      quant/hqe_2.py:456-843        (six targets: 16/8/4/2/1 bit + evict)
+  * ``KV_cache_compress``   quant/hybrid_quant.py:318-612  (five targets, no eviction)
+  * ``KV_cache_compress_1`` quant/hybrid_quant.py:614-730  (same, V range supplied by the caller)
+
+What is normative, because it fixes the order of tokens inside every class and therefore the packed
+bytes: targets are served from the lowest precision up (evict, 1, 2, 4, 8, 16); for each target the
+sources are visited as new tokens, then the 16, 8, 4, 2-bit classes, and only sources of HIGHER
+precision than the target move (a token is never promoted); moved tokens are appended to the target
+in source order; a quantised source is dequantised (two fp16 roundings) and re-quantised; K moves in
+whole 32-token groups.  After an eviction every surviving index is replaced by its rank among the
+survivors (quant/hqe_2.py:661-670).
+
+The reference re-copies whole class tensors with boolean masks; here a move gathers only the moved
+columns / rows with ``index_select`` and quantises them with one fused kernel (K straight from the
+token-major residual, no transpose copy).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from . import pack_unpack as PU
+from .public_func import calculate_token_range, get_block_token_idx
+
+BLOCK = 32
+CLASS_BITS = (16, 8, 4, 2, 1)
+K_SLOT = {16: 0, 8: 4, 4: 12, 2: 20, 1: 28}
+V_SLOT = {16: 2, 8: 8, 4: 16, 2: 24, 1: 32}
+_STRATEGIES = ("uniform", "normal", "uniform_group", "normal_group", "high_uniform_group_low_normal_group")
+
+
+class _Cls:
+    """One precision class of one side (K or V): data, positions, scale, zero."""
+    __slots__ = ("data", "idx", "scale", "zero")
+
+    def __init__(self, data=None, idx=None, scale=None, zero=None):
+        self.data, self.idx, self.scale, self.zero = data, idx, scale, zero
+
+    @property
+    def empty(self) -> bool:
+        return self.data is None
+
+
+def _read_side(pkv: tuple, slots: Dict[int, int]) -> Dict[int, _Cls]:
+    out = {}
+    for b in CLASS_BITS:
+        s = slots[b]
+        if b == 16:
+            out[b] = _Cls(pkv[s], pkv[s + 1])
+        else:
+            out[b] = _Cls(pkv[s], pkv[s + 1], pkv[s + 2], pkv[s + 3])
+    return out
+
+
+def _write_side(t: list, side: Dict[int, _Cls], slots: Dict[int, int]) -> None:
+    for b in CLASS_BITS:
+        s, c = slots[b], side[b]
+        t[s], t[s + 1] = c.data, c.idx
+        if b != 16:
+            t[s + 2], t[s + 3] = c.scale, c.zero
+
+
+def _cat(a: Optional[torch.Tensor], b: torch.Tensor, dim: int) -> torch.Tensor:
+    return b if a is None else torch.cat((a, b), dim=dim)
+
+
+def _none_if_empty(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return None if x is None or x.numel() == 0 else x
+
+
+def _check_low_bits(bits: int, strategy: str) -> None:
+    if bits == 1:
+        raise NotImplementedError(
+            "a populated 1-bit class needs the 1-bit quantisers (normal-quantile, or uniform with 32 codes per "
+            "word), which are not built; run with a zero 1-bit share")
+    if strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
+        raise NotImplementedError(f"quant_strategy '{strategy}' uses quantiser families that are not built")
+
+
+# ----------------------------------------------------------------------------------------------- K side
+# K classes are channel-major (B, H, D, X): X = tokens (fp16), tokens/pf (codes), tokens/32 (scale, zero).
+
+def _group_columns(groups: torch.Tensor, per_group: int) -> torch.Tensor:
+    return (groups[:, None] * per_group + torch.arange(per_group, device=groups.device)[None, :]).reshape(-1)
+
+
+def _k_split(c: _Cls, bits: int, mask: torch.Tensor):
+    """-> (moved class, kept class); ``mask`` marks tokens of ``c`` and must cover whole 32-token groups."""
+    gm = mask.view(-1, BLOCK)
+    if not bool((gm == gm[:, :1]).all()):
+        raise ValueError("K classes move in whole 32-token groups: the selection splits a group")
+    g_all = gm[:, 0]
+    sel, keep = g_all.nonzero().flatten(), (~g_all).nonzero().flatten()
+    per = BLOCK if bits == 16 else BLOCK // (32 // bits)
+
+    def part(groups: torch.Tensor, m: torch.Tensor) -> _Cls:
+        if groups.numel() == 0:
+            return _Cls()
+        data = c.data.index_select(3, _group_columns(groups, per))
+        if bits == 16:
+            return _Cls(data, c.idx[m])
+        return _Cls(data, c.idx[m], c.scale.index_select(3, groups), c.zero.index_select(3, groups))
+
+    return part(sel, mask), part(keep, ~mask)
+
+
+def _k_to_fp16(c: _Cls, bits: int) -> torch.Tensor:
+    if bits == 16:
+        return c.data
+    return PU.uniform_group_dequantize_unpack_last_dim(c.data, c.scale, c.zero, BLOCK, bits)
+
+
+def _k_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int) -> None:
+    """x is (B, H, D, n) fp16, possibly the transposed view of token-major memory."""
+    if bits == 16:
+        dst.data = _cat(dst.data, x, 3)
+    else:
+        code, scale, zero = PU.uniform_group_quantize_pack_last_dim(x, BLOCK, bits)
+        dst.data, dst.scale, dst.zero = _cat(dst.data, code, 3), _cat(dst.scale, scale, 3), _cat(dst.zero, zero, 3)
+    dst.idx = _cat(dst.idx, idx, 0)
+
+
+# ----------------------------------------------------------------------------------------------- V side
+# V classes are token-major (B, H, n, X): X = D (fp16), D/pf (codes), D/32 (scale, zero).
+
+def _v_split(c: _Cls, bits: int, mask: torch.Tensor):
+    sel, keep = mask.nonzero().flatten(), (~mask).nonzero().flatten()
+
+    def part(rows: torch.Tensor) -> _Cls:
+        if rows.numel() == 0:
+            return _Cls()
+        if bits == 16:
+            return _Cls(c.data.index_select(2, rows), c.idx[rows])
+        return _Cls(c.data.index_select(2, rows), c.idx[rows], c.scale.index_select(2, rows),
+                    c.zero.index_select(2, rows))
+
+    return part(sel), part(keep)
+
+
+def _v_to_fp16(c: _Cls, bits: int) -> torch.Tensor:
+    if bits == 16:
+        return c.data
+    return PU.uniform_group_dequantize_unpack_last_dim(c.data, c.scale, c.zero, BLOCK, bits)
+
+
+def _v_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int) -> None:
+    if bits == 16:
+        dst.data = _cat(dst.data, x, 2)
+    else:
+        code, scale, zero = PU.uniform_group_quantize_pack_last_dim(x, BLOCK, bits)
+        dst.data, dst.scale, dst.zero = _cat(dst.data, code, 2), _cat(dst.scale, scale, 2), _cat(dst.zero, zero, 2)
+    dst.idx = _cat(dst.idx, idx, 0)
+
+
+# ----------------------------------------------------------------------------------------------- engine
+
+def _targets(sorted_idx: torch.Tensor, bit_num: torch.Tensor) -> List[Optional[torch.Tensor]]:
+    """Slices of the ranked token list for (16, 8, 4, 2, 1[, evict]); None where a share is empty."""
+    cum = [0] + [int(v) for v in torch.cumsum(bit_num.to(torch.int64).cpu(), 0).tolist()]
+    return [sorted_idx[cum[i]:cum[i + 1]] if cum[i + 1] > cum[i] else None for i in range(len(cum) - 1)]
+
+
+def _rerank(side: Dict[int, _Cls]) -> None:
+    """Survivors keep their order; each index becomes its rank among all survivors."""
+    parts = [side[b].idx for b in CLASS_BITS if side[b].idx is not None]
+    if not parts:
+        return
+    allv = torch.cat(parts)
+    order = torch.argsort(allv)
+    rank = torch.empty_like(order)
+    rank[order] = torch.arange(order.numel(), device=order.device, dtype=order.dtype)
+    start = 0
+    for b in CLASS_BITS:
+        if side[b].idx is not None:
+            n = side[b].idx.numel()
+            side[b].idx = rank[start:start + n].to(side[b].idx.dtype)
+            start += n
+
+
+def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[torch.Tensor]], history: int,
+             is_k: bool, strategy: str, on_evict=None):
+    """Run one compression on one side.  ``new`` is (B, H, n_new, D) fp16 (token-major for K and V alike)."""
+    dev = new.device
+    new_idx = torch.arange(history, history + new.shape[2], device=dev, dtype=torch.int64)
+    split, to16, append = (_k_split, _k_to_fp16, _k_append) if is_k else (_v_split, _v_to_fp16, _v_append)
+    evict = targets[5] if len(targets) > 5 else None
+
+    def take_new(mask: torch.Tensor) -> torch.Tensor:
+        nonlocal new, new_idx
+        rows, keep = mask.nonzero().flatten(), (~mask).nonzero().flatten()
+        moved = new.index_select(2, rows)
+        new, new_idx = new.index_select(2, keep), new_idx[keep]
+        return moved
+
+    # 1. eviction: dropped tokens leave every tensor
+    if evict is not None:
+        m = torch.isin(new_idx, evict)
+        if bool(m.any()):
+            take_new(m)
+        for b in CLASS_BITS:
+            c = side[b]
+            if c.idx is None:
+                continue
+            m = torch.isin(c.idx, evict)
+            if bool(m.any()):
+                _, side[b] = split(c, b, m)
+        if on_evict is not None:
+            on_evict(side, new_idx)
+
+    # 2. demotions, lowest target first; sources: new tokens, then 16, 8, 4, 2 (only above the target)
+    for ti in (4, 3, 2, 1, 0):
+        tgt_bits, tgt_idx = CLASS_BITS[ti], targets[ti]
+        if tgt_idx is None:
+            continue
+        if new_idx.numel():
+            m = torch.isin(new_idx, tgt_idx)
+            if bool(m.any()):
+                if tgt_bits < 16:
+                    _check_low_bits(tgt_bits, strategy)
+                sel_idx = new_idx[m]
+                moved = take_new(m)  # (B, H, n, D)
+                append(side[tgt_bits], moved.transpose(2, 3) if is_k else moved, sel_idx, tgt_bits)
+        for src_bits in CLASS_BITS:
+            if src_bits <= tgt_bits:
+                break
+            c = side[src_bits]
+            if c.idx is None:
+                continue
+            m = torch.isin(c.idx, tgt_idx)
+            if not bool(m.any()):
+                continue
+            _check_low_bits(tgt_bits, strategy)
+            moved, side[src_bits] = split(c, src_bits, m)
+            append(side[tgt_bits], to16(moved, src_bits), moved.idx, tgt_bits)
+
+    if evict is not None:
+        _rerank(side)
+    return new, new_idx
+
+
+def compress(past_key_value: tuple, compress_length: int, history_length, K_sorted_idx: torch.Tensor,
+             K_bit_num: torch.Tensor, V_bit_num: torch.Tensor, token_importance: torch.Tensor,
+             quant_strategy: str, *, last_weights=None, block_size: int = 32, group_size: int = 32,
+             times_range: bool = True, n_targets: int = 6, V_token_range: Optional[torch.Tensor] = None) -> tuple:
+    if quant_strategy not in _STRATEGIES:
+        raise ValueError('invalid quant_strategy')
+    if block_size != BLOCK or group_size != BLOCK:
+        raise ValueError("block_size and group_size must be 32")
+    pkv = past_key_value
+    new_K, new_V = pkv[39], pkv[40]
+    if new_K is None or new_V is None:
+        raise ValueError('invalid past_key_value')
+    history = int(history_length)
+    if compress_length % BLOCK or history % BLOCK:
+        raise ValueError("compress_length and history_length must be multiples of 32")
+    if K_bit_num.numel() != n_targets or V_bit_num.numel() != n_targets:
+        raise ValueError(f"K_bit_num / V_bit_num must hold {n_targets} entries")
+    res_K = _none_if_empty(new_K[:, :, compress_length:, :].clone())
+    res_V = _none_if_empty(new_V[:, :, compress_length:, :].clone())
+    new_K, new_V = new_K[:, :, :compress_length, :], new_V[:, :, :compress_length, :]
+    total = history + compress_length
+    block_num = total // BLOCK
+
+    V_norm = V_token_range if V_token_range is not None else calculate_token_range(new_V, pkv[38])
+    V_score = token_importance * V_norm if times_range else token_importance.clone()
+    V_sorted_idx = get_block_token_idx(BLOCK, block_num, V_score)
+
+    k_side, v_side = _read_side(pkv, K_SLOT), _read_side(pkv, V_SLOT)
+    _migrate(k_side, new_K, _targets(K_sorted_idx, K_bit_num), history, True, quant_strategy)
+
+    def after_v_eviction(side, new_idx):
+        nonlocal V_norm
+        keep = [side[b].idx for b in CLASS_BITS if side[b].idx is not None] + [new_idx]
+        keep = torch.sort(torch.cat(keep))[0]
+        V_norm = V_norm[keep]
+        if last_weights is not None:
+            last_weights.eviction(keep)
+
+    _migrate(v_side, new_V, _targets(V_sorted_idx, V_bit_num), history, False, quant_strategy,
+             on_evict=after_v_eviction)
+
+    t = list(pkv)
+    _write_side(t, k_side, K_SLOT)
+    _write_side(t, v_side, V_SLOT)
+    t[38], t[39], t[40] = V_norm, res_K, res_V
+    return tuple(t)
+
+
+def reconstruct(past_key_value: tuple, quant_strategy: str, block_size: int = 32, group_size: int = 32):
+    """Dequantise every class back into dense (B, H, kv_seq_len, D) fp16 K and V
+    (quant/hybrid_quant.py:732-846, quant/hqe_2.py:967-1084).  Unlike the reference, the 4-bit V class
+    is restored whether or not an 8-bit class exists, and the result is fp16 for any class mix."""
+    if quant_strategy not in _STRATEGIES:
+        raise ValueError('invalid quant_strategy')
+    pkv = past_key_value
+    k_side, v_side = _read_side(pkv, K_SLOT), _read_side(pkv, V_SLOT)
+    new_K, new_V, T = pkv[39], pkv[40], int(pkv[41])
+    some = next((x for x in (v_side[16].data, v_side[8].data, v_side[4].data, v_side[2].data, new_V) if x is not None), None)
+    if some is None:
+        raise ValueError('invalid past_key_value')
+    B, H, dev = some.shape[0], some.shape[1], some.device
+    if new_V is not None:
+        D = new_V.shape[3]
+    elif v_side[16].data is not None:
+        D = v_side[16].data.shape[3]
+    else:
+        b = next(b for b in (8, 4, 2) if v_side[b].data is not None)
+        D = v_side[b].data.shape[3] * (32 // b)
+    K = torch.zeros(B, H, T, D, dtype=torch.float16, device=dev)
+    V = torch.zeros(B, H, T, D, dtype=torch.float16, device=dev)
+    for b in CLASS_BITS:
+        if b == 1 and (k_side[b].data is not None or v_side[b].data is not None):
+            _check_low_bits(1, quant_strategy)
+        if k_side[b].data is not None:
+            K[:, :, k_side[b].idx, :] = _k_to_fp16(k_side[b], b).transpose(2, 3)
+        if v_side[b].data is not None:
+            V[:, :, v_side[b].idx, :] = _v_to_fp16(v_side[b], b)
+    if new_K is not None:
+        K[:, :, T - new_K.shape[2]:, :] = new_K
+    if new_V is not None:
+        V[:, :, T - new_V.shape[2]:, :] = new_V
+    return K, V

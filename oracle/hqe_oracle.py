@@ -17,7 +17,7 @@ Pinned:
   gemv_uniform_group                            special cases that collapse to integer
                                                 mat-vec / torch.matmul
   qkv_matmul                                    permutation invariance against dense attention
-  compress_cache / rerank_after_eviction        brute force against Python sets
+  compress_cache / rerank_after_eviction        brute force against a per-block history model and Python sets
 
 Parity unpinned (no reference fixture exists and only a run of the original GPU stack
 could pin it): the last-bit behaviour of ``fp16_tensor / python_int`` on the GPU, which
@@ -315,3 +315,203 @@ def rerank_after_eviction(idx_per_class: Sequence[Optional[torch.Tensor]]) -> Li
     for t in idx_per_class:
         out.append(None if t is None else torch.tensor([rank[int(v)] for v in t.tolist()], dtype=torch.int64))
     return out
+
+
+# --------------------------------------------------------------------------- cache policy (unit lists)
+#
+# Restatement of KV_cache_hqe_2 (quant/hqe_2.py:456-843) and KV_cache_compress
+# (quant/hybrid_quant.py:318-612) on explicit lists of units instead of concatenated tensors:
+# a K unit is one 32-token group of one class (the granularity at which the reference moves K,
+# quant/hqe_2.py:102-117), a V unit is one token.  The quantiser is local to a group, so quantising
+# unit by unit equals the reference's batched calls; class tensors are the units concatenated in
+# list order, which is the reference's torch.cat order.  Slow by design (Python loops).
+
+_CLASS_BITS = (16, 8, 4, 2, 1)
+
+
+def _units_from_class(data, idx, scale, zero, bits, is_k):
+    units = []
+    if data is None:
+        return units
+    if is_k:
+        n = idx.numel()
+        assert n % 32 == 0
+        pf = 32 // bits if bits < 16 else 1
+        for g in range(n // 32):
+            u = dict(idx=idx[32 * g:32 * g + 32].clone(), bits=bits)
+            if bits == 16:
+                u["x"] = data[..., 32 * g:32 * g + 32].clone()
+            else:
+                w = 32 // pf
+                u["x"] = (data[..., w * g:w * g + w].clone(), scale[..., g:g + 1].clone(), zero[..., g:g + 1].clone())
+            units.append(u)
+    else:
+        for t in range(idx.numel()):
+            u = dict(idx=idx[t:t + 1].clone(), bits=bits)
+            if bits == 16:
+                u["x"] = data[:, :, t:t + 1, :].clone()
+            else:
+                u["x"] = (data[:, :, t:t + 1, :].clone(), scale[:, :, t:t + 1, :].clone(), zero[:, :, t:t + 1, :].clone())
+            units.append(u)
+    return units
+
+
+def _unit_fp16(u):
+    if u["bits"] == 16:
+        return u["x"]
+    c, s, z = u["x"]
+    return uniform_group_dequantize_unpack_last_dim(c, s, z, 32, u["bits"])
+
+
+def _unit_requant(u, bits, scalar_div):
+    x = _unit_fp16(u)
+    if bits == 16:
+        return dict(idx=u["idx"], bits=16, x=x)
+    return dict(idx=u["idx"], bits=bits, x=uniform_group_quantize_pack_last_dim(x, 32, bits, scalar_div))
+
+
+def _class_from_units(units, bits, is_k):
+    if not units:
+        return (None, None) if bits == 16 else (None, None, None, None)
+    idx = torch.cat([u["idx"] for u in units])
+    dim = 3 if is_k else 2
+    if bits == 16:
+        return torch.cat([u["x"] for u in units], dim=dim), idx
+    return (torch.cat([u["x"][0] for u in units], dim=dim), idx,
+            torch.cat([u["x"][1] for u in units], dim=dim), torch.cat([u["x"][2] for u in units], dim=dim))
+
+
+def _policy_side(pkv, new, history, sorted_idx, bit_num, is_k, scalar_div):
+    """-> ({bits: units}, surviving positions before re-ranking or None if nothing was to be evicted)."""
+    slots = K_BASE if is_k else V_BASE
+    cls = {}
+    for b in _CLASS_BITS:
+        if b == 16:
+            cls[b] = _units_from_class(pkv[K16 if is_k else V16], pkv[K16_IDX if is_k else V16_IDX], None, None, 16, is_k)
+        else:
+            s = slots[b]
+            cls[b] = _units_from_class(pkv[s], pkv[s + 1], pkv[s + 2], pkv[s + 3], b, is_k)
+    # new tokens as units (K: in 32-token groups that are formed at the moment they move)
+    n_new = new.shape[2]
+    new_tokens = [dict(idx=torch.tensor([history + t]), x=new[:, :, t:t + 1, :]) for t in range(n_new)]
+    cum = [0] + torch.cumsum(bit_num.to(torch.int64), 0).tolist()
+    target = [set(sorted_idx[cum[i]:cum[i + 1]].tolist()) for i in range(len(cum) - 1)]
+    has_evict = len(target) > 5 and len(target[5]) > 0
+    if has_evict:
+        new_tokens = [u for u in new_tokens if int(u["idx"][0]) not in target[5]]
+        for b in _CLASS_BITS:
+            kept = []
+            for u in cls[b]:
+                hit = [int(v) in target[5] for v in u["idx"].tolist()]
+                assert all(hit) or not any(hit), "a unit is evicted as a whole"
+                if not hit[0]:
+                    kept.append(u)
+            cls[b] = kept
+    survivors = None
+    if has_evict:
+        survivors = sorted([int(v) for b in _CLASS_BITS for u in cls[b] for v in u["idx"].tolist()]
+                           + [int(u["idx"][0]) for u in new_tokens])
+    for ti in (4, 3, 2, 1, 0):
+        tb, tset = _CLASS_BITS[ti], target[ti]
+        if not tset:
+            continue
+        moved = [u for u in new_tokens if int(u["idx"][0]) in tset]
+        if moved:
+            new_tokens = [u for u in new_tokens if int(u["idx"][0]) not in tset]
+            if is_k:
+                assert len(moved) % 32 == 0
+                for g in range(len(moved) // 32):
+                    grp = moved[32 * g:32 * g + 32]
+                    x = torch.cat([u["x"] for u in grp], dim=2).transpose(2, 3).contiguous()   # (B,H,D,32)
+                    cls[tb].append(_unit_requant(dict(idx=torch.cat([u["idx"] for u in grp]), bits=16, x=x), tb, scalar_div))
+            else:
+                for u in moved:
+                    cls[tb].append(_unit_requant(dict(idx=u["idx"], bits=16, x=u["x"]), tb, scalar_div))
+        for sb in _CLASS_BITS:
+            if sb <= tb:
+                break
+            stay = []
+            for u in cls[sb]:
+                hit = [int(v) in tset for v in u["idx"].tolist()]
+                assert all(hit) or not any(hit)
+                if hit[0]:
+                    cls[tb].append(_unit_requant(u, tb, scalar_div))
+                else:
+                    stay.append(u)
+            cls[sb] = stay
+    assert not new_tokens, "every new token is assigned to a class or evicted"
+    if len(target) > 5 and (cum[6] > cum[5]):
+        rank = {v: r for r, v in enumerate(sorted(int(v) for b in _CLASS_BITS for u in cls[b] for v in u["idx"].tolist()))}
+        for b in _CLASS_BITS:
+            for u in cls[b]:
+                u["idx"] = torch.tensor([rank[int(v)] for v in u["idx"].tolist()], dtype=torch.int64)
+    return cls, survivors
+
+
+def compress_cache(past_key_value: tuple, compress_length: int, history_length: int, K_sorted_idx, K_bit_num,
+                   V_bit_num, token_importance, *, times_range: bool = True, scalar_div: str = "recip",
+                   weights_ring: Optional[torch.Tensor] = None):
+    """One compression step; 6-entry bit_num = KV_cache_hqe_2, 5-entry = KV_cache_compress.
+    Returns (new 42-tuple, ring of recent attention rows after eviction or None).  1-bit shares must be 0."""
+    pkv = past_key_value
+    assert int(K_bit_num[4]) == 0 and int(V_bit_num[4]) == 0, "the 1-bit class is outside the oracle"
+    new_K, new_V = pkv[NEW_K], pkv[NEW_V]
+    res_K = new_K[:, :, compress_length:, :].clone()
+    res_V = new_V[:, :, compress_length:, :].clone()
+    new_K, new_V = new_K[:, :, :compress_length, :], new_V[:, :, :compress_length, :]
+    total = history_length + compress_length
+    V_norm = calculate_token_range(new_V, pkv[V_TOKEN_NORM])
+    V_score = token_importance * V_norm if times_range else token_importance.clone()
+    V_sorted_idx = get_block_token_idx(32, total // 32, V_score)
+    k_cls, _ = _policy_side(pkv, new_K, history_length, K_sorted_idx, K_bit_num, True, scalar_div)
+    v_cls, v_alive = _policy_side(pkv, new_V, history_length, V_sorted_idx, V_bit_num, False, scalar_div)
+    if v_alive is not None:
+        keep = torch.tensor(v_alive, dtype=torch.int64)
+        V_norm = V_norm[keep]
+        if weights_ring is not None:
+            weights_ring = weights_ring.clone()
+            kept = weights_ring[:, keep]
+            weights_ring[:, :kept.shape[1]] = kept
+    t = [None] * 42
+    t[K16], t[K16_IDX] = _class_from_units(k_cls[16], 16, True)
+    t[V16], t[V16_IDX] = _class_from_units(v_cls[16], 16, False)
+    for b in (8, 4, 2):
+        s = K_BASE[b]
+        t[s], t[s + 1], t[s + 2], t[s + 3] = _class_from_units(k_cls[b], b, True)
+        s = V_BASE[b]
+        t[s], t[s + 1], t[s + 2], t[s + 3] = _class_from_units(v_cls[b], b, False)
+    t[V_TOKEN_NORM] = V_norm
+    t[NEW_K] = res_K if res_K.numel() else None
+    t[NEW_V] = res_V if res_V.numel() else None
+    t[KV_SEQ_LEN] = pkv[KV_SEQ_LEN]
+    return tuple(t), weights_ring
+
+
+def reconstruct_cache(past_key_value: tuple):
+    """Dense fp16 (K, V) (B,H,kv_seq_len,D) from the tuple (quant/hybrid_quant.py:732-846, with the 4-bit V
+    class restored unconditionally)."""
+    pkv = past_key_value
+    T = int(pkv[KV_SEQ_LEN])
+    ref = next(x for x in (pkv[NEW_V], pkv[V16]) if x is not None) if (pkv[NEW_V] is not None or pkv[V16] is not None) else None
+    if ref is not None:
+        B, H, D = ref.shape[0], ref.shape[1], ref.shape[3]
+    else:
+        b = next(b for b in BITS if pkv[V_BASE[b]] is not None)
+        B, H, D = pkv[V_BASE[b]].shape[0], pkv[V_BASE[b]].shape[1], pkv[V_BASE[b]].shape[3] * (32 // b)
+    K = torch.zeros(B, H, T, D, dtype=torch.float16)
+    V = torch.zeros(B, H, T, D, dtype=torch.float16)
+    if pkv[K16] is not None:
+        K[:, :, pkv[K16_IDX]] = pkv[K16].transpose(2, 3)
+    if pkv[V16] is not None:
+        V[:, :, pkv[V16_IDX]] = pkv[V16]
+    for b in BITS:
+        s = K_BASE[b]
+        if pkv[s] is not None:
+            K[:, :, pkv[s + 1]] = uniform_group_dequantize_unpack_last_dim(pkv[s], pkv[s + 2], pkv[s + 3], 32, b).transpose(2, 3)
+        s = V_BASE[b]
+        if pkv[s] is not None:
+            V[:, :, pkv[s + 1]] = uniform_group_dequantize_unpack_last_dim(pkv[s], pkv[s + 2], pkv[s + 3], 32, b)
+    if pkv[NEW_K] is not None:
+        K[:, :, T - pkv[NEW_K].shape[2]:] = pkv[NEW_K]
+        V[:, :, T - pkv[NEW_V].shape[2]:] = pkv[NEW_V]
+    return K, V

@@ -48,3 +48,49 @@ def test_argument_validation_without_a_gpu():
         _lib.check(-1, "x")
     with pytest.raises(RuntimeError):
         _lib.check(700, "x")
+
+
+def test_reference_import_names_resolve():
+    """`from pack_unpack import ...`, `from quant.hqe_matmul import ...`, `from model.public_func import ...`"""
+    import importlib
+    import sys
+    from hqekv_amd import compat
+    saved = {k: sys.modules.get(k) for k in list(sys.modules) if k.split(".")[0] in ("quant", "model") or k in compat._MODULES}
+    try:
+        compat.install(force=True)
+        from pack_unpack import uniform_group_quantize_pack_last_dim  # noqa: F401
+        from matmul import cuda_bmm_fA_qB_uniform_group, cuda_bmm_forward_qk_group_hq  # noqa: F401
+        from quant.hqe_matmul import qkv_matmul_hqe_2  # noqa: F401
+        from quant.hqe_2 import KV_cache_hqe_2  # noqa: F401
+        from quant.quant_matmul_hq import qkv_matmul, qkv_matmul_hq  # noqa: F401
+        from quant.hybrid_quant import KV_cache_compress, KV_cache_reconstruct  # noqa: F401
+        from model.public_func import get_block_token_idx, last_attn_weights, make_sum_equal  # noqa: F401
+        assert importlib.import_module("quant.pack_unpack") is importlib.import_module("hqekv_amd.pack_unpack")
+    finally:
+        for k in list(sys.modules):
+            if (k.split(".")[0] in ("quant", "model") or k in compat._MODULES) and k not in saved:
+                del sys.modules[k]
+        for k, v in saved.items():
+            if v is not None:
+                sys.modules[k] = v
+
+
+def test_host_helpers_match_oracle():
+    import torch
+    from hqekv_amd import public_func as P
+    from oracle import hqe_oracle as O
+    g = torch.Generator().manual_seed(0)
+    imp = torch.rand(256, generator=g)
+    assert torch.equal(P.get_block_token_idx(32, 8, imp.clone()), O.get_block_token_idx(32, 8, imp))
+    v = torch.randn(2, 3, 16, 32, generator=g).half()
+    assert torch.equal(P.calculate_token_range(v, None), O.calculate_token_range(v, None))
+    a = torch.tensor([2, 0, 10, 10, 10, 5])
+    for target in (35, 40, 25):
+        assert P.make_sum_equal(a.clone(), target).tolist() == O.make_sum_equal(a, target).tolist()
+    lw = P.last_attn_weights(4)
+    lw.set_max_length(8)
+    for step in range(6):
+        lw.update(torch.full((1, 2, 1, 5 + (step > 2)), float(step + 1)))
+    # ring of the last 4 decode rows, each summed over 2 heads; columns seen by fewer rows divide by fewer
+    imp2 = lw.calculate_token_importance()
+    assert imp2.shape == (6,) and abs(float(imp2[0]) - 2 * (3 + 4 + 5 + 6) / 4) < 1e-6

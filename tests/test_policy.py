@@ -1,0 +1,109 @@
+"""The cache-policy oracle against an independent per-block history model (CPU only).
+
+The model knows nothing about tensors of classes: it tracks, for every original 32-token block, the
+sequence of precisions it went through and whether it survived, using only the published rules
+(targets served low to high, demotion only, whole blocks, survivors re-ranked).  The dense cache the
+oracle's tuple reconstructs to must equal the original data pushed through that chain of fake
+quantisations, at the position the model predicts."""
+import torch
+
+from oracle import hqe_oracle as O
+from tests import policy_cases as PC
+
+
+def _oracle_compress(pkv, cl, hist, ks, kb, vb, imp):
+    return O.compress_cache(pkv, cl, hist, ks, kb, vb, imp)[0]
+
+
+def _model(log, K, V):
+    """-> per side, the ordered list of (original block id, [precision chain]) of the survivors."""
+    sides = {}
+    for side in ("K", "V"):
+        order = []      # surviving original blocks in position order: (block id, chain)
+        n_seen = 0
+        for st in log:
+            n_new_blocks = st["compress_length"] // 32
+            order = order + [(n_seen + j, None) for j in range(n_new_blocks)]   # chain None = still new
+            total_blocks = len(order)
+            imp = st["importance"]
+            if side == "V":   # V ranks by importance x token range of the (dequantisation-free) originals
+                rng = torch.cat([(V[:, :, 32 * b:32 * b + 32].max(-1)[0] - V[:, :, 32 * b:32 * b + 32].min(-1)[0]).sum(0).sum(0)
+                                 for b, _ in order])
+                imp = imp * rng
+            blk = (imp.reshape(total_blocks, 32) / 32).sum(-1)
+            ranked = torch.sort(blk, descending=True, stable=True)[1].tolist()
+            counts = [c // 32 for c in st["counts"]]
+            tgt, pos = {}, 0
+            for bits, c in zip((16, 8, 4, 2, 1, 0), counts):
+                for p in ranked[pos:pos + c]:
+                    tgt[p] = bits
+                pos += c
+            nxt = []
+            for p, (bid, chain) in enumerate(order):
+                t = tgt[p]
+                if t == 0:
+                    continue
+                if chain is None:
+                    chain = [t]
+                elif t < chain[-1]:
+                    chain = chain + [t]
+                nxt.append((bid, chain))
+            order = nxt
+            n_seen += n_new_blocks
+        sides[side] = order
+    return sides
+
+
+def _expected_block(x_block, chain, is_k):
+    """x_block (B,H,32,D) original fp16 -> value after the chain of quantise/dequantise steps."""
+    x = x_block
+    for bits in chain:
+        if bits == 16:
+            continue
+        if is_k:
+            x = O.uniform_group_fake_quant(x.transpose(2, 3).contiguous(), 32, bits).transpose(2, 3)
+        else:
+            x = O.uniform_group_fake_quant(x.contiguous(), 32, bits)
+    return x
+
+
+def test_oracle_policy_matches_history_model():
+    caches, log, (K, V) = PC.run(_oracle_compress)
+    # the V ranking needs distinct block scores to be order-independent of sort stability; check that
+    final = caches[-1]
+    model = _model(log, K, V)
+    dK, dV = O.reconstruct_cache(final)
+    n_res = 0 if final[39] is None else final[39].shape[2]
+    for side, dense, src, is_k in (("K", dK, K, True), ("V", dV, V, False)):
+        order = model[side]
+        assert dense.shape[2] == 32 * len(order) + n_res
+        for p, (bid, chain) in enumerate(order):
+            exp = _expected_block(src[:, :, 32 * bid:32 * bid + 32], chain, is_k)
+            got = dense[:, :, 32 * p:32 * p + 32]
+            assert torch.equal(got, exp), (side, p, bid, chain)
+    # class membership: the number of tokens per class equals the model's count of final precisions
+    for side, slots in (("K", (0, 4, 12, 20)), ("V", (2, 8, 16, 24))):
+        for bits, s in zip((16, 8, 4, 2), slots):
+            want = 32 * sum(1 for _, ch in model[side] if ch[-1] == bits)
+            have = 0 if final[s + 1] is None else final[s + 1].numel()
+            assert have == want, (side, bits, have, want)
+
+
+def test_oracle_policy_invariants_every_step():
+    caches, log, _ = PC.run(_oracle_compress)
+    for pkv, st in zip(caches, log):
+        kept = st["history"] + st["compress_length"] - st["counts"][5]
+        for slots in ((1, 5, 13, 21), (3, 9, 17, 25)):
+            idx = torch.cat([pkv[s] for s in slots if pkv[s] is not None])
+            assert sorted(idx.tolist()) == list(range(kept)), "class positions partition the survivors"
+            for s in slots:
+                if pkv[s] is not None:
+                    assert pkv[s].numel() % 32 == 0 and pkv[s].dtype == torch.int64
+        assert pkv[38].numel() == kept
+        # shapes of a quantised class agree with its index
+        for b, s in ((8, 4), (4, 12), (2, 20)):
+            if pkv[s] is not None:
+                n = pkv[s + 1].numel()
+                assert pkv[s].shape == (PC.B, PC.H, PC.D, n * b // 32) and pkv[s + 2].shape == (PC.B, PC.H, PC.D, n // 32)
+            if pkv[s + 4] is not None:
+                assert pkv[s + 4].shape == (PC.B, PC.H, pkv[s + 5].numel(), PC.D * b // 32)
