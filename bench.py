@@ -128,6 +128,8 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="distinct layer caches cycled through")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one plain 256 MiB device copy, the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs the decode-attention path on ONE GPU; --gpus {args.gpus} is not "
@@ -141,6 +143,12 @@ def main():
     from hqekv_amd.attention import DecodePlan
 
     dev = torch.device("cuda:0")
+    if args.calibrate:  # a copy kernel of known size: reads 256 MiB, writes 256 MiB
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     n_layers = args.layers or {"c1": 64, "c2": 32, "c4": 4}[args.workload]
     layers = build_layers(args.workload, n_layers, dev)
     plans = [DecodePlan(q, cache) for q, cache in layers]

@@ -43,7 +43,7 @@ struct SegTable {
   SegDev seg[HQEKV_MAX_SEGS];
   int32_t nseg;
   int32_t total_units;
-  int32_t max_units;   // grid.x: the largest n_units of any segment
+  int32_t max_units;   // grid.y: the largest n_units of any segment
   int32_t pad_;
 };
 
@@ -60,9 +60,15 @@ struct FuseArgs {
   float inv_sqrt_d;
 };
 
-// A workgroup learns its segment from blockIdx.z and its tile/chunk from blockIdx.x, so everything it
+// A workgroup learns its segment and its tile/chunk from its (remapped) block id, so everything it
 // needs from the kernel arguments is fetched in one batch at the top of the kernel (a scalar load that
 // misses costs about a microsecond; a lookup through the table would chain several of them).
+
+// Workgroups are handed to the 8 XCDs round-robin in launch order, and each XCD has its own L2.
+// Neighbouring tiles of one (b, kv head) slab share cache lines (a tile's row segment is shorter than a
+// line, its scale/zero rows are a quarter of one), so the (b, kv head) index is the FASTEST grid
+// dimension: with B*Hkv a multiple of 8, every tile of a slab runs on the same XCD, neighbours meet in
+// one L2, and the eight XCDs get equal work.  (Tile-fastest order fetched every line 2x on average.)
 
 // keep every load issued above this point ahead of the arithmetic below it (the scheduler would
 // otherwise sink loads next to their uses to save registers, serialising the memory latency)
@@ -368,11 +374,10 @@ __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, cons
   float *red = smem;                                                        // QK_WAVES * 2 * 8 * 64 floats
   half2_t *q2s = reinterpret_cast<half2_t *>(smem + QK_WAVES * 2 * QK_TPL * 64);  // D/2 x NREP pairs (q[d], q[d+1])
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int bh = blockIdx.y;
+  const int bh = blockIdx.x, tile = blockIdx.y;
   const int b = bh / Hkv, hkv = bh % Hkv;
   const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads, no lazy re-reads
-  const int tile = blockIdx.x;
-  if (tile >= sg.n_units) return;  // uniform: grid.x is the largest tile count of any segment
+  if (tile >= sg.n_units) return;  // uniform: grid.y is the largest tile count of any segment
   const bool tm = sg.bits == 16 && sg.token_major;
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t t0 = (uint32_t)tile * QK_TILE + lane * QK_TPL;
@@ -743,13 +748,13 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
   __shared__ float red[PV_WAVES * NREP * D];
   __shared__ PvStage<NREP, D / 32> st;
   __shared__ float sm_ml[2 * NREP];  // fused mode: (max, 1 / sum exp) of each query head's row
+  const int bh = blockIdx.x, ux = blockIdx.y;
   const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads
-  if ((int)blockIdx.x >= sg.n_units) return;  // uniform: grid.x is the largest chunk count of any segment
+  if (ux >= sg.n_units) return;  // uniform: grid.y is the largest chunk count of any segment
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int bh = blockIdx.y;
   const int b = bh / Hkv, hkv = bh % Hkv;
-  const int chunk_id = sg.unit_begin + (int)blockIdx.x;
-  const int64_t c0 = (int64_t)blockIdx.x * chunk_tokens;
+  const int chunk_id = sg.unit_begin + ux;
+  const int64_t c0 = (int64_t)ux * chunk_tokens;
   const int64_t c1 = min(c0 + chunk_tokens, sg.n_tokens);
   const bool fused = fz.stats != nullptr;
   half_t *prow[NREP];
@@ -871,7 +876,7 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
     d.n_units = (int32_t)nu;
     if (nu > max_units) max_units = nu;
     units += nu;
-    if (units > 0x3fffffff) return fail(HQEKV_E_ARG, "%s: too many work units", who);
+    if (nu > 65535) return fail(HQEKV_E_ARG, "%s: segment %d needs %lld work units (limit 65535)", who, k, (long long)nu);
   }
   tb->nseg = m;
   tb->total_units = (int32_t)units;
@@ -888,7 +893,7 @@ static int check_heads(const char *who, int64_t B, int64_t Hq, int64_t Hkv, int6
   const int64_t nrep = Hq / Hkv;
   if (!(nrep == 1 || nrep == 2 || nrep == 4 || nrep == 8))
     return fail(HQEKV_E_UNSUPPORTED, "%s: Hq/Hkv=%lld (supported: 1, 2, 4, 8)", who, (long long)nrep);
-  if (B * Hkv > 65535) return fail(HQEKV_E_ARG, "%s: B*Hkv > 65535", who);
+  if (B * Hkv > 0x7fffffffLL) return fail(HQEKV_E_ARG, "%s: B*Hkv too large", who);
   if (D <= 0 || D % 32 != 0) return fail(HQEKV_E_ARG, "%s: D=%lld must be a positive multiple of 32", who, (long long)D);
   return HQEKV_OK;
 }
@@ -897,7 +902,7 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
                      int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st) {
   if (tb.total_units == 0) return HQEKV_OK;
   const int nrep = (int)(Hq / Hkv);
-  dim3 grid((unsigned)tb.max_units, (unsigned)(B * Hkv), (unsigned)tb.nseg), block(QK_THREADS);
+  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.max_units, (unsigned)tb.nseg), block(QK_THREADS);
   const size_t shmem = (size_t)(nrep * D + QK_WAVES * 2 * QK_TPL * 64) * sizeof(float);
 #define LAUNCH(N_)                                                                                    \
   hipLaunchKernelGGL(qk_hybrid_kernel<N_>, grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
@@ -936,7 +941,7 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
   const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
   if (tb.total_units > 0 && (stages & 1)) {
-    dim3 grid((unsigned)tb.max_units, (unsigned)(B * Hkv), (unsigned)tb.nseg), block(PV_THREADS);
+    dim3 grid((unsigned)(B * Hkv), (unsigned)tb.max_units, (unsigned)tb.nseg), block(PV_THREADS);
 #define LAUNCH(N_, D_)                                                                                   \
   hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
                      (int)Hkv, Tall, chunk, n_bhq, fz)
