@@ -592,7 +592,7 @@ constexpr int PV_THREADS = 256;
 constexpr int PV_WAVES = 4;
 constexpr int PV_CPL = 8;                        // channels per lane
 constexpr int PV_BLOCK = 512;                    // tokens staged in LDS at a time (256 token pairs)
-constexpr int PV_UNR = 4;                        // wave steps whose loads are in flight together
+constexpr int PV_UNR = 4;                        // word pairs per lane in flight together (steps = 4 / words per token)
 
 // LDS block, pair-interleaved: per token pair {s2, z2} for each of the D/32 groups and p2 for each
 // query head, so one 8-byte and one 4*NREP-byte LDS read feed a whole step of a lane.
@@ -602,51 +602,81 @@ struct PvStage {
   half2_t p2[PV_BLOCK / 2][NREP];
 };
 
-// stage p (gathered through idx) and, for quantised classes, scale/zero of tokens [t0, t0+nt)
+// What thread t fetches for token pair t of a 512-token block: positions, the two logits/probabilities
+// of every query head, and the pair's scale/zero rows.  Fetching and committing are separate so that the
+// requests of the next block (and of the first block, at kernel start) overlap with other work.
+template <int NREP, int NG>
+struct PvPair {
+  int64_t pa, pb;
+  half_t va[NREP], vb[NREP];
+  uint2 sa, sb, za, zb;  // 4 fp16 scales / zeros of token a and of token b (NG == 4)
+  bool valid, has_b;
+};
+
 template <int NREP, int NG, bool QUANT>
-__device__ __forceinline__ void pv_stage(const SegDev &sg, int64_t t0, int nt, int bh,
-                                         half_t *const (&prow)[NREP], PvStage<NREP, NG> &st, bool fused,
-                                         const float *sm_ml) {
-  const int ntp = (nt + 1) >> 1;
-  const int64_t *ip = sg.idx;
-  for (int tp = threadIdx.x; tp < ntp; tp += PV_THREADS) {
-    const int64_t ta = t0 + 2 * tp;
-    const bool has_b = 2 * tp + 1 < nt;
-    const int64_t tb2 = has_b ? ta + 1 : ta;
-    int64_t pa = sg.pos_base + ta, pb = sg.pos_base + tb2;
-    if (ip) {
-      pa = ip[ta];
-      pb = ip[tb2];
-    }
-    half_t va[NREP], vb[NREP];
-#pragma unroll
-    for (int h = 0; h < NREP; ++h) {
-      va[h] = prow[h][pa];
-      vb[h] = prow[h][pb];
-    }
-    if (fused) {
-      // the row holds scaled logits: p = rnd16(exp(x - M) / L), written back for the caller.  Every
-      // position belongs to exactly one token of exactly one V class, so nobody else touches it.
-#pragma unroll
-      for (int h = 0; h < NREP; ++h) {
-        const float M = sm_ml[2 * h], invL = sm_ml[2 * h + 1];
-        va[h] = (half_t)(__expf((float)va[h] - M) * invL);
-        vb[h] = (half_t)(__expf((float)vb[h] - M) * invL);
-        prow[h][pa] = va[h];
-        if (has_b) prow[h][pb] = vb[h];
-      }
-    }
-#pragma unroll
-    for (int h = 0; h < NREP; ++h) st.p2[tp][h] = pack_h2(va[h], has_b ? vb[h] : (half_t)0);
+__device__ __forceinline__ void pv_fetch(const SegDev &sg, int64_t t0, int nt, int bh, half_t *const (&prow)[NREP],
+                                         PvPair<NREP, NG> &pr) {
+  static_assert(NG == 4, "a token's scale row is read as one 8-byte load");
+  const int tp = threadIdx.x;
+  pr.valid = 2 * tp < nt;
+  pr.has_b = 2 * tp + 1 < nt;
+  const int64_t ta = t0 + (pr.valid ? 2 * tp : 0);
+  const int64_t tb2 = pr.has_b ? ta + 1 : ta;
+  pr.pa = sg.pos_base + ta;
+  pr.pb = sg.pos_base + tb2;
+  if (sg.idx) {
+    pr.pa = sg.idx[ta];
+    pr.pb = sg.idx[tb2];
   }
   if (QUANT) {  // n_tokens is a multiple of 32, so pairs are always complete
-    const half_t *sc = sg.scale + ((int64_t)bh * sg.n_tokens + t0) * NG;
-    const half_t *zr = sg.zero + ((int64_t)bh * sg.n_tokens + t0) * NG;
-    for (int k = threadIdx.x; k < ntp * NG; k += PV_THREADS) {
-      const int tp = k / NG, g = k % NG;
+    const uint2 *sc = reinterpret_cast<const uint2 *>(sg.scale + ((int64_t)bh * sg.n_tokens + ta) * NG);
+    const uint2 *zr = reinterpret_cast<const uint2 *>(sg.zero + ((int64_t)bh * sg.n_tokens + ta) * NG);
+    pr.sa = sc[0];
+    pr.sb = sc[1];
+    pr.za = zr[0];
+    pr.zb = zr[1];
+  }
+#pragma unroll
+  for (int h = 0; h < NREP; ++h) {
+    pr.va[h] = prow[h][pr.pa];
+    pr.vb[h] = prow[h][pr.pb];
+  }
+}
+
+template <int NREP, int NG, bool QUANT>
+__device__ __forceinline__ void pv_commit(const PvPair<NREP, NG> &pr, half_t *const (&prow)[NREP],
+                                          PvStage<NREP, NG> &st, bool fused, const float *sm_ml) {
+  if (!pr.valid) return;
+  const int tp = threadIdx.x;
+  half_t va[NREP], vb[NREP];
+#pragma unroll
+  for (int h = 0; h < NREP; ++h) {
+    va[h] = pr.va[h];
+    vb[h] = pr.vb[h];
+  }
+  if (fused) {
+    // the row holds scaled logits: p = rnd16(exp(x - M) / L), written back for the caller.  Every
+    // position belongs to exactly one token of exactly one V class, so nobody else touches it.
+#pragma unroll
+    for (int h = 0; h < NREP; ++h) {
+      const float M = sm_ml[2 * h], invL = sm_ml[2 * h + 1];
+      va[h] = (half_t)(__expf((float)va[h] - M) * invL);
+      vb[h] = (half_t)(__expf((float)vb[h] - M) * invL);
+      prow[h][pr.pa] = va[h];
+      if (pr.has_b) prow[h][pr.pb] = vb[h];
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < NREP; ++h) st.p2[tp][h] = pack_h2(va[h], pr.has_b ? vb[h] : (half_t)0);
+  if (QUANT) {
+    // (s_a[g], s_b[g]) pairs: halves 2g of the two rows
+    const uint32_t sa[2] = {pr.sa.x, pr.sa.y}, sb[2] = {pr.sb.x, pr.sb.y};
+    const uint32_t za[2] = {pr.za.x, pr.za.y}, zb[2] = {pr.zb.x, pr.zb.y};
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
       uint2 v;
-      v.x = as_u32(pack_h2(sc[(2 * tp) * NG + g], sc[(2 * tp + 1) * NG + g]));
-      v.y = as_u32(pack_h2(zr[(2 * tp) * NG + g], zr[(2 * tp + 1) * NG + g]));
+      v.x = (g & 1) ? as_u32(half_pair<1>(sa[g >> 1], sb[g >> 1])) : as_u32(half_pair<0>(sa[g >> 1], sb[g >> 1]));
+      v.y = (g & 1) ? as_u32(half_pair<1>(za[g >> 1], zb[g >> 1])) : as_u32(half_pair<0>(za[g >> 1], zb[g >> 1]));
       st.sz[tp][g] = v;
     }
   }
@@ -654,47 +684,68 @@ __device__ __forceinline__ void pv_stage(const SegDev &sg, int64_t t0, int nt, i
 
 // One class chunk.  16 lanes cover a token row (8 channels each: half a packed word at 2 bits, one word
 // at 4 bits, two words at 8 bits, 16 bytes of fp16), 4 token pairs per wave step, so the reduction over
-// tokens needs only two butterfly steps across lanes.
+// tokens needs only two butterfly steps across lanes.  Code words are requested one step-block ahead of
+// their use, and the staging requests of a block are issued before the previous block is consumed.
 template <int BITS, int NREP, int D>
 __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh, int wave, int lane,
                                          half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
                                          float (&acc)[NREP][PV_CPL], bool fused, const float *sm_ml) {
   static_assert(D == 128, "16 lanes x 8 channels cover one token row");
+  constexpr int NG = D / 32;
+  constexpr bool QUANT = BITS != 16;
   constexpr int WPL = BITS == 16 ? 4 : (BITS == 8 ? 2 : 1);  // 32-bit words per lane per token
-  constexpr int ROWW = D * BITS / 32;                         // 32-bit words per token row
+  constexpr int ROWB = D * BITS / 8;                          // bytes per token row
+  constexpr int UNR = PV_UNR / WPL;                           // wave steps per block: 8 words in flight per lane
   const int cl = lane & 15, tl = lane >> 4;
   const int g = cl >> 2;
   const int sh2 = (BITS == 2) ? (cl & 1) * 16 : 0;
   const uint32_t wofs = (BITS == 2 ? (cl >> 1) : cl * WPL) * 4u;  // byte offset inside a token row
-  const char *base = (const char *)sg.data + (int64_t)bh * sg.n_tokens * ROWW * 4;
+  const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * sg.n_tokens * ROWB, (uint32_t)(sg.n_tokens * ROWB));
+  const uint32_t lane_off = (uint32_t)(2 * tl) * ROWB + wofs;   // this lane's first token of a step + word
 
+  struct Words {
+    uint32_t w0[UNR][WPL], w1[UNR][WPL];
+  };
+  // the step-block starting at wave step s0 of the 512-token block at t0 (uniform offsets in scalars)
+  auto load_steps = [&](int64_t t0, int nt, int s0, Words &r) {
+#pragma unroll
+    for (int k = 0; k < UNR; ++k) {
+      const uint32_t tok = (uint32_t)(t0 + 8 * ((s0 + k) * PV_WAVES + wave));  // uniform: first token of the step
+      const bool odd_tail = (int)(8 * ((s0 + k) * PV_WAVES + wave) + 2 * tl + 1) >= nt;  // pair without a second token
+      const uint32_t row = tok * ROWB;
+#pragma unroll
+      for (int j = 0; j < WPL; ++j) {
+        r.w0[k][j] = buf_u32(rc, lane_off + 4 * j, row);
+        r.w1[k][j] = buf_u32(rc, lane_off + (odd_tail ? 0u : (uint32_t)ROWB) + 4 * j, row);
+      }
+    }
+  };
+
+  PvPair<NREP, NG> pr;
+  Words cur;
+  {
+    const int nt0 = (int)min((int64_t)PV_BLOCK, c1 - c0);
+    pv_fetch<NREP, NG, QUANT>(sg, c0, nt0, bh, prow, pr);
+    load_steps(c0, nt0, 0, cur);
+  }
   for (int64_t t0 = c0; t0 < c1; t0 += PV_BLOCK) {
     const int nt = (int)min((int64_t)PV_BLOCK, c1 - t0);
     const int ntp = (nt + 1) >> 1;
     const int nsteps = (ntp + 4 * PV_WAVES - 1) / (4 * PV_WAVES);
-    __syncthreads();  // previous block fully consumed
-    if (BITS == 16) pv_stage<NREP, D / 32, false>(sg, t0, nt, bh, prow, st, fused, sm_ml);
-    else pv_stage<NREP, D / 32, true>(sg, t0, nt, bh, prow, st, fused, sm_ml);
+    const bool more = t0 + PV_BLOCK < c1;
+    const int nt_next = more ? (int)min((int64_t)PV_BLOCK, c1 - t0 - PV_BLOCK) : 0;
+    __syncthreads();  // previous block fully consumed (and sm_ml published)
+    pv_commit<NREP, NG, QUANT>(pr, prow, st, fused, sm_ml);
+    if (more) pv_fetch<NREP, NG, QUANT>(sg, t0 + PV_BLOCK, nt_next, bh, prow, pr);
     __syncthreads();
 #pragma unroll 1
-    for (int s0 = 0; s0 < nsteps; s0 += PV_UNR) {
-      uint32_t w0[PV_UNR][WPL], w1[PV_UNR][WPL];
-#pragma unroll
-      for (int k = 0; k < PV_UNR; ++k) {
-        const int tp = 4 * ((s0 + k) * PV_WAVES + wave) + tl;
-        const int tpc = tp < ntp ? tp : 0;
-        const bool has_b = 2 * tpc + 1 < nt;
-        const char *ra = base + (t0 + 2 * tpc) * (int64_t)(ROWW * 4) + wofs;
-        const char *rb = has_b ? ra + ROWW * 4 : ra;
-#pragma unroll
-        for (int j = 0; j < WPL; ++j) {
-          w0[k][j] = *reinterpret_cast<const uint32_t *>(ra + 4 * j);
-          w1[k][j] = *reinterpret_cast<const uint32_t *>(rb + 4 * j);
-        }
-      }
+    for (int s0 = 0; s0 < nsteps; s0 += UNR) {
+      Words nxt;
+      if (s0 + UNR < nsteps) load_steps(t0, nt, s0 + UNR, nxt);
+      else if (more) load_steps(t0 + PV_BLOCK, nt_next, 0, nxt);
       HQ_LOADS_ABOVE();
 #pragma unroll
-      for (int k = 0; k < PV_UNR; ++k) {
+      for (int k = 0; k < UNR; ++k) {
         const int tp = 4 * ((s0 + k) * PV_WAVES + wave) + tl;
         if (tp < ntp) {
           half2_t p2[NREP];
@@ -704,8 +755,8 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
             // an odd tail pair has p = 0 for its second token, so the duplicated row adds nothing
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              const half2_t va = half_pair<0>(w0[k][j], w1[k][j]);  // channel 2j:   (v[t], v[t+1])
-              const half2_t vb = half_pair<1>(w0[k][j], w1[k][j]);  // channel 2j+1
+              const half2_t va = half_pair<0>(cur.w0[k][j], cur.w1[k][j]);  // channel 2j:   (v[t], v[t+1])
+              const half2_t vb = half_pair<1>(cur.w0[k][j], cur.w1[k][j]);  // channel 2j+1
 #pragma unroll
               for (int h = 0; h < NREP; ++h) {
                 acc[h][2 * j] = __builtin_amdgcn_fdot2(va, p2[h], acc[h][2 * j], false);
@@ -716,26 +767,27 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
             const uint2 sz = st.sz[tp][g];
             const half2_t s2 = as_h2(sz.x), z2 = as_h2(sz.y);
             if (BITS == 2) {
-              const uint32_t a0 = w0[k][0] >> sh2, a1 = w1[k][0] >> sh2;
+              const uint32_t a0 = cur.w0[k][0] >> sh2, a1 = cur.w1[k][0] >> sh2;
               consume_byte<2, NREP, PV_CPL>(byte_pair<0>(a0, a1), s2, z2, p2, acc, 0);
               consume_byte<2, NREP, PV_CPL>(byte_pair<1>(a0, a1), s2, z2, p2, acc, 4);
             } else if (BITS == 4) {
-              consume_byte<4, NREP, PV_CPL>(byte_pair<0>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 0);
-              consume_byte<4, NREP, PV_CPL>(byte_pair<1>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 2);
-              consume_byte<4, NREP, PV_CPL>(byte_pair<2>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 4);
-              consume_byte<4, NREP, PV_CPL>(byte_pair<3>(w0[k][0], w1[k][0]), s2, z2, p2, acc, 6);
+              consume_byte<4, NREP, PV_CPL>(byte_pair<0>(cur.w0[k][0], cur.w1[k][0]), s2, z2, p2, acc, 0);
+              consume_byte<4, NREP, PV_CPL>(byte_pair<1>(cur.w0[k][0], cur.w1[k][0]), s2, z2, p2, acc, 2);
+              consume_byte<4, NREP, PV_CPL>(byte_pair<2>(cur.w0[k][0], cur.w1[k][0]), s2, z2, p2, acc, 4);
+              consume_byte<4, NREP, PV_CPL>(byte_pair<3>(cur.w0[k][0], cur.w1[k][0]), s2, z2, p2, acc, 6);
             } else {
 #pragma unroll
               for (int j = 0; j < (BITS == 8 ? 2 : 0); ++j) {
-                consume_byte<8, NREP, PV_CPL>(byte_pair<0>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 0);
-                consume_byte<8, NREP, PV_CPL>(byte_pair<1>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 1);
-                consume_byte<8, NREP, PV_CPL>(byte_pair<2>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 2);
-                consume_byte<8, NREP, PV_CPL>(byte_pair<3>(w0[k][j], w1[k][j]), s2, z2, p2, acc, 4 * j + 3);
+                consume_byte<8, NREP, PV_CPL>(byte_pair<0>(cur.w0[k][j], cur.w1[k][j]), s2, z2, p2, acc, 4 * j + 0);
+                consume_byte<8, NREP, PV_CPL>(byte_pair<1>(cur.w0[k][j], cur.w1[k][j]), s2, z2, p2, acc, 4 * j + 1);
+                consume_byte<8, NREP, PV_CPL>(byte_pair<2>(cur.w0[k][j], cur.w1[k][j]), s2, z2, p2, acc, 4 * j + 2);
+                consume_byte<8, NREP, PV_CPL>(byte_pair<3>(cur.w0[k][j], cur.w1[k][j]), s2, z2, p2, acc, 4 * j + 3);
               }
             }
           }
         }
       }
+      cur = nxt;
     }
   }
 }
@@ -859,6 +911,10 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
       return fail(HQEKV_E_ARG, "%s: segment %d positions [%lld,%lld) outside [0,%lld)", who, k,
                   (long long)s.pos_base, (long long)(s.pos_base + s.n_tokens), (long long)Tall);
     if ((uintptr_t)s.data & 3) return fail(HQEKV_E_ALIGN, "%s: segment %d data not 4-byte aligned", who, k);
+    if (!is_k && s.bits != 16 && ((((uintptr_t)s.scale) | ((uintptr_t)s.zero)) & 7))
+      return fail(HQEKV_E_ALIGN, "%s: segment %d scale/zero rows must be 8-byte aligned", who, k);
+    if (s.bits == 16 && ((uintptr_t)s.data & 15))
+      return fail(HQEKV_E_ALIGN, "%s: segment %d fp16 data must be 16-byte aligned", who, k);
     if (s.n_tokens * D >= (1LL << 31))
       return fail(HQEKV_E_UNSUPPORTED, "%s: segment %d: n_tokens * D must stay below 2^31 per (b, head) slab", who, k);
     SegDev &d = tb->seg[m++];
