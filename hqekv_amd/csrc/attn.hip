@@ -20,6 +20,8 @@
 //            scale/zero and the gathered probabilities of a 512-token block are staged in LDS in
 //            pair-interleaved order; lanes are reduced by butterflies, waves through LDS, workgroups
 //            through fp32 partials summed in a fixed order.
+#include <stdlib.h>
+
 #include "common.h"
 
 #pragma clang fp contract(off)  // the two fp16 roundings of the dequantiser must stay separate
@@ -862,8 +864,9 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
 }
 
 // fixed-order sum over chunks: deterministic replacement for the reference's half atomics
-// (quant/csrc/gemv_cuda_wv_uniform.cu:110).  One workgroup per (b, hq) row; CB_SLICES slices of the
-// chunk list are summed in parallel (strided, ascending within a slice), then the slices in order.
+// (quant/csrc/gemv_cuda_wv_uniform.cu:110).  One workgroup per (b, hq) row and 128 channels; CB_SLICES
+// slices of the chunk list are summed in parallel (strided, ascending within a slice, eight requests in
+// flight per thread), then the slices in order.
 constexpr int CB_SLICES = 8;
 __global__ __launch_bounds__(1024) void pv_combine_kernel(const float *__restrict__ partial,
                                                           half_t *__restrict__ out, int n_chunks,
@@ -871,19 +874,28 @@ __global__ __launch_bounds__(1024) void pv_combine_kernel(const float *__restric
   __shared__ float sh[CB_SLICES][128];
   const int64_t r = blockIdx.x;
   const int d = threadIdx.x % 128, sl = threadIdx.x / 128;
-  for (int d0 = 0; d0 < D; d0 += 128) {
-    float v = 0.f;
-    if (d0 + d < D)
-      for (int c = sl; c < n_chunks; c += CB_SLICES) v += partial[((int64_t)c * n_bhq + r) * D + d0 + d];
-    sh[sl][d] = v;
-    __syncthreads();
-    if (sl == 0 && d0 + d < D) {
-      float t = sh[0][d];
+  const int d0 = blockIdx.y * 128;
+  const bool in = d0 + d < D;
+  const float *src = partial + r * D + d0 + (in ? d : 0);
+  const int64_t cstride = n_bhq * D;
+  float v = 0.f;
+  for (int c0 = sl; c0 < n_chunks; c0 += CB_SLICES * 8) {
+    float t[8];
 #pragma unroll
-      for (int k = 1; k < CB_SLICES; ++k) t += sh[k][d];
-      out[r * D + d0 + d] = (half_t)t;
+    for (int k = 0; k < 8; ++k) {
+      const int c = c0 + k * CB_SLICES;
+      t[k] = c < n_chunks ? src[(int64_t)c * cstride] : 0.f;
     }
-    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v += t[k];
+  }
+  sh[sl][d] = v;
+  __syncthreads();
+  if (sl == 0 && in) {
+    float t = sh[0][d];
+#pragma unroll
+    for (int k = 1; k < CB_SLICES; ++k) t += sh[k][d];
+    out[r * D + d0 + d] = (half_t)t;
   }
 }
 
@@ -975,7 +987,7 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
 
 // chunk length for the p.V split-K: aim for a few workgroups per CU, never below 64 tokens
 static int64_t pv_chunk_tokens(int64_t total_tokens, int64_t BHkv) {
-  const int64_t target_wgs = 256 * 4;
+  static const int64_t target_wgs = getenv("HQEKV_PV_TARGET_WGS") ? atoll(getenv("HQEKV_PV_TARGET_WGS")) : 256 * 4;
   int64_t chunks_per_bh = (target_wgs + BHkv - 1) / BHkv;
   if (chunks_per_bh < 1) chunks_per_bh = 1;
   int64_t c = (total_tokens + chunks_per_bh - 1) / chunks_per_bh;
@@ -1014,7 +1026,7 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
     if (rc) return rc;
   }
   if (!(stages & 2)) return HQEKV_OK;
-  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq), dim3(128 * CB_SLICES), 0, st, partial,
+  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq, (unsigned)((D + 127) / 128)), dim3(128 * CB_SLICES), 0, st, partial,
                      (half_t *)out, (int)tb.total_units, n_bhq, (int)D);
   return check_launch("pv_combine_kernel");
 }
