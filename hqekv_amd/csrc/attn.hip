@@ -160,8 +160,9 @@ __device__ __forceinline__ void consume_words(uint32_t w0, uint32_t w1, half2_t 
 }
 
 // =============================================================================== q.K^T
-constexpr int QK_THREADS = 512;
-constexpr int QK_WAVES = 8;
+// A tile is worked on by W = 8 waves (small launches: shortest critical path per tile) or W = 4 waves
+// (large launches: more independent workgroups per CU, so one tile's load and reduce phases overlap
+// another's arithmetic).
 constexpr int QK_TPL = 8;               // tokens per lane in every channel-major class
 constexpr int QK_TILE = 64 * QK_TPL;    // tokens per workgroup tile
 constexpr int QK_UNR = 8;               // row pairs whose loads are in flight together, per wave
@@ -191,7 +192,7 @@ __device__ __forceinline__ half_t buf_f16(rsrc_t r, uint32_t lane_off, uint32_t 
 // packed word at 2 bits (two lanes read the same word), one word at 4 bits, two words at 8 bits.
 // QK_UNR row pairs at a time: every load of a block is issued before its first use, and the rolled outer
 // loop keeps the code small enough to stay in the instruction cache from one launch to the next.
-template <int BITS, int NREP>
+template <int BITS, int NREP, int QK_WAVES>
 __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int D, int wave,
                                                     const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
   constexpr int PF = 32 / BITS;
@@ -257,7 +258,7 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
 }
 
 // fp16 class stored channel-major (B,Hkv,D,T): a lane owns 8 adjacent tokens of each row
-template <int NREP>
+template <int NREP, int QK_WAVES>
 __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t t0, int bh, int D, int wave,
                                                      const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
   const uint32_t n = (uint32_t)sg.n_tokens;
@@ -306,7 +307,7 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
 }
 
 // fp16 residual stored token-major (B,Hkv,T,D): a wave walks tokens, lanes split the channels
-template <int NREP>
+template <int NREP, int QK_WAVES>
 __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int bh, int b, int hkv, int D,
                                                int Hq, int64_t Tall, int wave, int lane, const half2_t *q2s,
                                                half_t *__restrict__ scores, const FuseArgs &fz, float *red) {
@@ -368,8 +369,8 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
 
 // One workgroup = one tile of one class for one (b, kv head).  The class-specific code is only the
 // accumulation; the cross-wave reduction and the (scattered) store are shared by every class.
-template <int NREP>
-__global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
+template <int NREP, int QK_WAVES>
+__global__ __launch_bounds__(QK_WAVES * 64) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
                                                                half_t *__restrict__ scores, int Hq,
                                                                int Hkv, int D, int64_t Tall, FuseArgs fz) {
   extern __shared__ float smem[];
@@ -397,13 +398,13 @@ __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, cons
     }
   }
   const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * D);
-  for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_THREADS) {
+  for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_WAVES * 64) {
     const int h = k / (D >> 1), dp = k % (D >> 1);
     q2s[dp * NREP + h] = as_h2(qsrc[k]);  // [dp][h]: one 16-byte LDS read fetches a row pair for 4 heads
   }
   __syncthreads();
   if (tm) {
-    qk_f16_tm_tile<NREP>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
+    qk_f16_tm_tile<NREP, QK_WAVES>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
     return;
   }
 
@@ -413,10 +414,10 @@ __global__ __launch_bounds__(QK_THREADS) void qk_hybrid_kernel(SegTable tb, cons
 #pragma unroll
     for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {
-    case 2: qk_quant_accumulate<2, NREP>(sg, ts, bh, D, wave, q2s, acc); break;
-    case 4: qk_quant_accumulate<4, NREP>(sg, ts, bh, D, wave, q2s, acc); break;
-    case 8: qk_quant_accumulate<8, NREP>(sg, ts, bh, D, wave, q2s, acc); break;
-    default: qk_f16_cm_accumulate<NREP>(sg, t0, bh, D, wave, q2s, acc);
+    case 2: qk_quant_accumulate<2, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
+    case 4: qk_quant_accumulate<4, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
+    case 8: qk_quant_accumulate<8, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
+    default: qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, q2s, acc);
   }
 
   // cross-wave reduction, RH heads per pass (bounds LDS at QK_WAVES*RH*8*64*4 bytes): every wave parks
@@ -970,17 +971,23 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
                      int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st) {
   if (tb.total_units == 0) return HQEKV_OK;
   const int nrep = (int)(Hq / Hkv);
-  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.max_units, (unsigned)tb.nseg), block(QK_THREADS);
-  const size_t shmem = (size_t)(nrep * D + QK_WAVES * 2 * QK_TPL * 64) * sizeof(float);
-#define LAUNCH(N_)                                                                                    \
-  hipLaunchKernelGGL(qk_hybrid_kernel<N_>, grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
+  // few tiles: 8 waves per tile; many tiles (several workgroups queue up per CU): 4 waves per tile
+  static const char *force = getenv("HQEKV_QK_WAVES");
+  const int waves = force ? atoi(force) : ((int64_t)tb.total_units * B * Hkv <= 1024 ? 8 : 4);
+  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.max_units, (unsigned)tb.nseg), block((unsigned)waves * 64);
+  const size_t shmem = (size_t)(nrep * D + waves * 2 * QK_TPL * 64) * sizeof(float);
+#define LAUNCH(N_, W_)                                                                                        \
+  hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
                      (int)Hq, (int)Hkv, (int)D, Tall, fz)
+#define LAUNCH_W(N_) \
+  if (waves == 8) LAUNCH(N_, 8); else LAUNCH(N_, 4)
   switch (nrep) {
-    case 1: LAUNCH(1); break;
-    case 2: LAUNCH(2); break;
-    case 4: LAUNCH(4); break;
-    default: LAUNCH(8);
+    case 1: LAUNCH_W(1); break;
+    case 2: LAUNCH_W(2); break;
+    case 4: LAUNCH_W(4); break;
+    default: LAUNCH_W(8);
   }
+#undef LAUNCH_W
 #undef LAUNCH
   return check_launch("qk_hybrid_kernel");
 }
