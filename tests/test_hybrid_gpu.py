@@ -190,3 +190,51 @@ def test_fused_path_is_deterministic_and_reusable(dev):
     wr, orr = ref.run(q.to(dev))
     _close(w0, wr.cpu(), "fused vs general attn_weights")
     _close(o0, orr.cpu(), "fused vs general attn_output")
+
+
+def test_config2_full_size_against_oracle(dev):
+    """BASELINE config 2 at its full size (B=1, 32 query heads, 8 KV heads, context 32768, hybrid split with
+    20 % evicted): caches built by the HIP quantiser are bit-identical to the oracle's, attention within
+    tolerance, and the probabilities of every head sum to one."""
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    from hqekv_amd.pack_unpack import uniform_group_quantize_pack_last_dim as hip_quant
+    cfg = synth.CONFIGS["c2"]
+    q, K, V = synth.make_qkv(cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["T"], cfg["D"], cfg["seed"])
+    classes = synth.split_blocks(cfg["T"], cfg["fractions"], cfg["seed"])
+    assert [classes[b].numel() for b in (16, 8, 4, 2, 0)] == [1632, 4928, 9824, 9824, 6560]
+    cache_cpu = synth.build_cache(K, V, classes, 0, O.uniform_group_quantize_pack_last_dim)
+    cache_gpu = synth.build_cache(K.to(dev), V.to(dev), classes, 0, hip_quant)
+    for i, (a, b) in enumerate(zip(cache_cpu[:41], cache_gpu[:41])):
+        if torch.is_tensor(a):
+            assert torch.equal(a, b.cpu()), f"cache slot {i}"
+    w_ref, o_ref = O.qkv_matmul(q, cache_cpu, None, 128, use_mask=False)
+    w, o = qkv_matmul_hqe_2(q.to(dev), cache_gpu, None, 128, "uniform_group")
+    assert w.shape == (1, 32, 1, 26208)
+    _close(w, w_ref, "attn_weights")
+    _close(o, o_ref, "attn_output")
+    torch.testing.assert_close(w.float().sum(-1).cpu(), torch.ones(1, 32, 1), rtol=0, atol=5e-3)
+
+
+def test_linearity_in_v_at_scale(dev):
+    """Size-independent property: with q = 0 every probability is 1/T, so the output is the mean of the
+    dequantised V rows -- checked against the HIP dequantiser at 16k tokens, batch 2."""
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    from hqekv_amd import pack_unpack as P
+    g = torch.Generator().manual_seed(8)
+    B, Hkv, T, D = 2, 2, 16384, 128
+    V = torch.randn(B, Hkv, T, D, generator=g).half().to(dev)
+    K = torch.randn(B, Hkv, T, D, generator=g).half().to(dev)
+    kc, ks, kz = P.uniform_group_quantize_pack_last_dim(K.transpose(2, 3), 32, 2)
+    vc, vs, vz = P.uniform_group_quantize_pack_last_dim(V, 32, 4)
+    idx = torch.arange(T, device=dev)
+    t = [None] * 42
+    t[20], t[21], t[22], t[23] = kc, idx, ks, kz
+    t[16], t[17], t[18], t[19] = vc, idx.clone(), vs, vz
+    t[41] = T
+    q = torch.zeros(B, 8, 1, D, dtype=torch.float16, device=dev)
+    w, o = qkv_matmul_hqe_2(q, tuple(t), None, D, "uniform_group")
+    assert torch.allclose(w.float(), torch.full_like(w, 1.0 / T, dtype=torch.float32), rtol=2e-3, atol=0)
+    dq = P.uniform_group_dequantize_unpack_last_dim(vc, vs, vz, 32, 4).float()
+    expect = (dq * w[0, 0, 0, 0].float()).sum(2, keepdim=True)                     # (B,Hkv,1,D)
+    expect = expect[:, :, None].expand(B, Hkv, 4, 1, D).reshape(B, 8, 1, D)
+    torch.testing.assert_close(o.float(), expect, rtol=2e-3, atol=2e-3)

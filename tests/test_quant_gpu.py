@@ -148,3 +148,22 @@ def test_argument_errors(dev):
         P.uniform_group_quantize_pack_last_dim(x.float(), 32, 2)
     with pytest.raises(RuntimeError):
         P.uniform_group_quantize_pack_last_dim(x.cpu(), 32, 2)
+
+
+def test_dequant_keeps_the_two_fp16_roundings(dev):
+    """10 * fp16(0.1) is a tie that rounds to 1.0 and 2050 + 1.0 is a tie that rounds to 2052; a fused
+    multiply-add (one rounding) would give 2050.  The same values must come out of the attention kernels."""
+    from hqekv_amd import pack_unpack as P
+    from hqekv_amd.matmul import cuda_bmm_fA_qB_uniform_group
+    codes = torch.zeros(1, 1, 128, 32, dtype=torch.int32)
+    codes[..., 0] = 10
+    code = O.pack_along_last_dim(codes, 4)
+    s = torch.full((1, 1, 128, 1), 0.0999755859375, dtype=torch.float16)
+    z = torch.full((1, 1, 128, 1), 2050.0, dtype=torch.float16)
+    dq = P.uniform_group_dequantize_unpack_last_dim(code.to(dev), s.to(dev), z.to(dev), 32, 4)
+    assert (dq[..., 0] == 2052.0).all() and (dq[..., 1] == 2050.0).all()
+    # q = e_0 picks K[d=0][t]: the GEMV must see 2052 for token 0 (exactly representable in the fp16 output)
+    q = torch.zeros(1, 1, 1, 128, dtype=torch.float16)
+    q[..., 0] = 1.0
+    out = cuda_bmm_fA_qB_uniform_group(32, q.to(dev), code.to(dev), s.to(dev), z.to(dev), 4)
+    assert out[0, 0, 0, 0].item() == 2052.0 and out[0, 0, 0, 1].item() == 2050.0
