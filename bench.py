@@ -32,6 +32,7 @@ WORKLOADS = {
     "c1": "Llama-3.1-8B shape, B=1, ctx 4096: 3968 tokens 2-bit + 128 fp16 residual",
     "c2": "Llama-3.1-8B shape, B=1, ctx 32768 hybrid: fp16 5% / 8-bit 15% / 4-bit 30% / 2-bit 30% / evicted 20%",
     "c4": "Qwen3-8B shape, B=8, ctx 65536 hybrid: fp16 10% / 4-bit 20% / 2-bit 50% / evicted 20%",
+    "c3": "quantize-and-pack: 8 KV heads x 128 x 8192 new fp16 tokens appended at token 24576 of a 32768-token cache",
 }
 
 
@@ -119,6 +120,104 @@ def cpu_baseline(name: str, n_iter: int = 5):
                 sample=f"{sample}; median of {n_iter} after 1 warm-up; torch {torch.__version__} CPU ops"), (q, cache, ref)
 
 
+def bench_quantize(args):
+    """Config 3: K (per channel, read in place from token-major memory) and V (per token) of 8192 new
+    tokens quantised at 2/4/8 bit straight into windows of capacity-sized cache buffers."""
+    from hqekv_amd import synth
+    from hqekv_amd.pack_unpack import quantize_pack_into
+    dev = torch.device("cuda:0")
+    B, H, D, Tn, off, cap = 1, 8, 128, 8192, 24576, 32768
+    n_copies = 8  # distinct inputs so no step finds its input in cache
+    ins = []
+    for c in range(n_copies):
+        _, K, V = synth.make_qkv(B, 32, H, Tn, D, 1237 + 1000 * c) if c == 0 else (None, None, None)
+        if c:
+            g = torch.Generator(device=dev).manual_seed(1237 + 1000 * c)
+            K = torch.randn(B, H, Tn, D, generator=g, device=dev)
+            for ch in synth.OUTLIER_CHANNELS:
+                K[..., ch] *= 10.0
+            K = K.half()
+            V = torch.randn(B, H, Tn, D, generator=g, device=dev).half()
+        ins.append((K.to(dev), V.to(dev)))
+    bufs = {}
+    for bit in (2, 4, 8):
+        pf = 32 // bit
+        bufs[bit] = dict(
+            kc=torch.zeros(B, H, D, cap // pf, dtype=torch.int32, device=dev),
+            ks=torch.zeros(B, H, D, cap // 32, dtype=torch.float16, device=dev),
+            kz=torch.zeros(B, H, D, cap // 32, dtype=torch.float16, device=dev),
+            vc=torch.zeros(B, H, cap, D // pf, dtype=torch.int32, device=dev),
+            vs=torch.zeros(B, H, cap, D // 32, dtype=torch.float16, device=dev),
+            vz=torch.zeros(B, H, cap, D // 32, dtype=torch.float16, device=dev))
+
+    def step(i, bit):
+        K, V = ins[i % n_copies]
+        b = bufs[bit]
+        pf = 32 // bit
+        quantize_pack_into(K.transpose(2, 3), bit, b["kc"][..., off // pf:], b["ks"][..., off // 32:], b["kz"][..., off // 32:])
+        quantize_pack_into(V, bit, b["vc"][:, :, off:], b["vs"][:, :, off:], b["vz"][:, :, off:])
+
+    def k_call(i, bit):
+        b = bufs[bit]
+        quantize_pack_into(ins[i][0].transpose(2, 3), bit, b["kc"][..., off // (32 // bit):], b["ks"][..., off // 32:], b["kz"][..., off // 32:])
+
+    def v_call(i, bit):
+        b = bufs[bit]
+        quantize_pack_into(ins[i][1], bit, b["vc"][:, :, off:], b["vs"][:, :, off:], b["vz"][:, :, off:])
+
+    def graph_of(fn):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        g.replay()
+        torch.cuda.synchronize()
+        return g
+
+    res = {}
+    for bit in (2, 4, 8):
+        for i in range(args.warmup):
+            step(i, bit)
+        torch.cuda.synchronize()
+        # launches replayed from a HIP graph, so the figures are the kernels' and not the host's
+        g_both = graph_of(lambda: [step(i, bit) for i in range(n_copies)])
+        g_k = graph_of(lambda: [k_call(i, bit) for i in range(n_copies)])
+        g_v = graph_of(lambda: [v_call(i, bit) for i in range(n_copies)])
+        reps = max(1, args.steps // n_copies)
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            g_both.replay()
+        torch.cuda.synchronize()
+        us = (time.perf_counter() - t0) / (reps * n_copies) * 1e6
+        k_us = event_avg_us(g_k.replay, n_copies, 9)
+        v_us = event_avg_us(g_v.replay, n_copies, 9)
+        elems = B * H * D * Tn
+        nbytes = elems * 2 + elems * bit // 8 + elems // 32 * 4     # per tensor: read fp16, write codes + scale + zero
+        res[bit] = dict(us_k_plus_v=round(us, 2), k_us=round(k_us, 2), v_us=round(v_us, 2), bytes_per_tensor=nbytes,
+                        k_GBps=round(nbytes / k_us / 1e3, 1), v_GBps=round(nbytes / v_us / 1e3, 1))
+    # bit-exactness of what was appended (2-bit, first input) against the oracle on the CPU
+    from oracle import hqe_oracle as O
+    step(0, 2)
+    torch.cuda.synchronize()
+    K0, V0 = ins[0][0].cpu(), ins[0][1].cpu()
+    okc, oks, okz = O.uniform_group_quantize_pack_last_dim(K0.transpose(2, 3).contiguous(), 32, 2)
+    ovc, ovs, ovz = O.uniform_group_quantize_pack_last_dim(V0, 32, 2)
+    b = bufs[2]
+    exact = bool(torch.equal(b["kc"][..., off // 16:].cpu(), okc) and torch.equal(b["ks"][..., off // 32:].cpu(), oks)
+                 and torch.equal(b["kz"][..., off // 32:].cpu(), okz) and torch.equal(b["vc"][:, :, off:].cpu(), ovc)
+                 and torch.equal(b["vs"][:, :, off:].cpu(), ovs) and torch.equal(b["vz"][:, :, off:].cpu(), ovz))
+    dom = max(res[2]["k_us"], res[2]["v_us"])
+    out = {"metric": "us per quantize-and-pack of 8192 new tokens (K + V, 2-bit) & GB/s", "value": res[2]["us_k_plus_v"],
+           "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(res[2]["us_k_plus_v"] / 1e3, 6), "higher_is_better": False, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+           "config": {"workload": f"c3: {WORKLOADS['c3']}", "launch": "hip-graph replay"},
+           "per_bit": res, "bit_exact_vs_oracle_2bit": exact,
+           "roofline": {"bound": "hbm", "kernel": "quant_k_tokenmajor_kernel<2>" if res[2]["k_us"] >= res[2]["v_us"] else "quant_rows_kernel<2>",
+                        "achieved": round(res[2]["bytes_per_tensor"] / dom / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": round(res[2]["bytes_per_tensor"] / dom / 1e3 / HBM_PEAK_GBPS, 4), "traffic": None}}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -138,6 +237,10 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
+
+    if args.workload == "c3":
+        bench_quantize(args)
+        return
 
     from hqekv_amd import synth
     from hqekv_amd.attention import DecodePlan

@@ -25,6 +25,7 @@ ONLY_COMBINE = 0x400
 EXPORTS = (
     "hqekv_version", "hqekv_last_error",
     "hqekv_quant_pack_rows", "hqekv_quant_pack_k_tokenmajor", "hqekv_dequant_unpack_rows", "hqekv_pack_i32",
+    "hqekv_selftest_quant_division",
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
     "hqekv_decode_workspace_bytes", "hqekv_decode_attn",
@@ -57,6 +58,7 @@ _PROTOS = {
     "hqekv_quant_pack_k_tokenmajor": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "hqekv_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "hqekv_pack_i32": (C.c_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "hqekv_selftest_quant_division": (C.c_int, [_vp, _vp]),
     "hqekv_gemv_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64, _int]),
     "hqekv_gemv_uniform_group": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
     "hqekv_qk_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),

@@ -171,23 +171,6 @@ __host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
   return (bits == 16 && token_major) ? 64 : QK_TILE;
 }
 
-// Buffer addressing: a 128-bit descriptor per (b, head) slab in scalar registers, a per-lane byte offset
-// that never changes, and the row offset in a scalar register -- no vector ALU work per load, and reads
-// past the end of the slab return zero instead of faulting.
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ uint32_t buf_u32(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
-  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)row_off, 0);
-}
-__device__ __forceinline__ half_t buf_f16(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
-  const unsigned short u = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, (int)row_off, 0);
-  half_t h;
-  __builtin_memcpy(&h, &u, 2);
-  return h;
-}
-
 // Accumulate one quantised tile: 512 tokens x D channels.  A lane owns 8 consecutive tokens: half a
 // packed word at 2 bits (two lanes read the same word), one word at 4 bits, two words at 8 bits.
 // QK_UNR row pairs at a time: every load of a block is issued before its first use, and the rolled outer

@@ -43,4 +43,21 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Buffer addressing: a 128-bit descriptor per (b, head) slab in scalar registers, a per-lane byte offset
+// that never changes, and the row offset in a scalar register -- no vector ALU work per load, and reads
+// past the end of the slab return zero instead of faulting.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint32_t buf_u32(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)row_off, 0);
+}
+__device__ __forceinline__ half_t buf_f16(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  const unsigned short u = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, (int)row_off, 0);
+  half_t h;
+  __builtin_memcpy(&h, &u, 2);
+  return h;
+}
+
 }  // namespace hq

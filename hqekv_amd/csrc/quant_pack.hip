@@ -13,122 +13,269 @@
 // contract or reassociate across it.
 #include "common.h"
 
+#pragma clang fp contract(off)
+
 namespace hq {
 
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t h2_bits(half2_t h) {
+  uint32_t u;
+  __builtin_memcpy(&u, &h, 4);
+  return u;
+}
+__device__ __forceinline__ half2_t bits_h2(uint32_t u) {
+  half2_t h;
+  __builtin_memcpy(&h, &u, 4);
+  return h;
+}
+
+// How the element-wise part of the chain is evaluated (results are those of the chain above, bit for bit):
+//  * u = rnd16(x - mn) is one packed fp16 subtraction.  Rounding an fp16 sum first to fp32 (24-bit
+//    significand >= 2*11+2) and then to fp16 gives the directly rounded fp16 sum, so there is nothing
+//    to gain from the detour through fp32 that the op-by-op evaluation takes.
+//  * v = rnd16(f32(u) / f32(scale)) is rnd16(f32(u) * r) with r the fp32 reciprocal of the group's
+//    scale after one Newton step.  A quotient of two 11-bit significands is never closer than
+//    1/(2047*4095) (relative) to a midpoint of the fp16 grid, which is more than the error of the
+//    rounded product; hqekv_selftest_quant_division compares the two over all 2^32 operand pairs.
+//    scale == 0 (constant group, or a range that underflows) and a non-finite scale keep the hardware
+//    reciprocal (inf / 0 / NaN), which reproduces x/0 = inf, 0/0 = NaN and x/inf = 0.
+//  * rne(clamp(v, 0, qmax)) is read from the significand of rnd16(clamp(v) + 1024): the fp16 grid has
+//    spacing 1 on [1024, 2048) and 1024 is even, so the sum is 1024 + rne(v) exactly.  max() drops a
+//    NaN operand, which turns the 0/0 of a constant group into code 0.
+__device__ __forceinline__ float group_recip(float s) {
+  const float r0 = __builtin_amdgcn_rcpf(s);
+  const float e = __builtin_fmaf(-s, r0, 1.0f);
+  const float r = __builtin_fmaf(e, r0, r0);
+  // +-normal or +-denormal: classes 3, 4, 7, 8
+  return __builtin_amdgcn_classf(s, 0x198) ? r : r0;
+}
+
+// fp16 bit patterns of 1024 + code for the pair (a, b) of already centred (x - mn) fp32 values
 template <int BITS>
-__device__ __forceinline__ uint32_t quant_one(half_t x, float mn, float scale_f) {
-  constexpr float QMAX = (float)((1 << BITS) - 1);
-  const float u = (float)(half_t)((float)x - mn);
-  float v = (float)(half_t)(u / scale_f);
-  // fmaxf/fminf drop a NaN operand: NaN -> 0, which is what the float->int conversion of the
-  // reference path yields for a constant group.
-  v = fminf(fmaxf(v, 0.0f), QMAX);
-  return (uint32_t)(int)__builtin_rintf(v);
+__device__ __forceinline__ uint32_t code_pair_biased(float ua, float ra, float ub, float rb) {
+  constexpr _Float16 QMAX = (_Float16)((1 << BITS) - 1);
+  const float2_t q = {ua * ra, ub * rb};
+  half2_t v = __builtin_convertvector(q, half2_t);
+  v = __builtin_elementwise_max(v, (half2_t){(_Float16)0, (_Float16)0});
+  v = __builtin_elementwise_min(v, (half2_t){QMAX, QMAX});
+  v = v + (half2_t){(_Float16)1024, (_Float16)1024};
+  return h2_bits(v);
+}
+
+// z[i] holds (1024 + code[i], 1024 + code[i + N]) for i < N, N * BITS <= 16:
+// returns code[i] at bit i*BITS and code[i + N] at bit 16 + i*BITS.
+template <int BITS, int N>
+__device__ __forceinline__ uint32_t horner_pack(const uint32_t *z) {
+  constexpr uint32_t MASK = ((1u << BITS) - 1u) * 0x00010001u;
+  uint32_t w = z[N - 1] & MASK;
+#pragma unroll
+  for (int i = N - 2; i >= 0; --i) w = (z[i] & MASK) | (w << BITS);
+  return w;
 }
 
 // ---------------------------------------------------------------- rows: groups along a contiguous axis
-// 4 lanes per 32-element group, 8 contiguous fp16 (one 128-bit load) per lane.
+// 4 lanes per 32-element group, 8 contiguous fp16 (one 128-bit load) per lane.  grid.x enumerates
+// (outer slab, block of 64 groups); a slab's groups are numbered row-major over (row, group in row).
 template <int BITS>
 __global__ __launch_bounds__(256) void quant_rows_kernel(
     const half_t *__restrict__ x, int64_t xo, int64_t xr, uint32_t *__restrict__ code, int64_t co,
     int64_t cr, half_t *__restrict__ scale, half_t *__restrict__ zero, int64_t so, int64_t sr,
-    int64_t n_rows, int64_t groups_per_row, int64_t n_groups) {
+    uint32_t groups_per_row, int gpr_shift, uint32_t groups_per_slab, uint32_t blocks_per_slab) {
   constexpr int PF = 32 / BITS;
   constexpr float INV_QMAX = 1.0f / (float)((1 << BITS) - 1);
-  const int64_t gid = (int64_t)blockIdx.x * 64 + (threadIdx.x >> 2);
-  const int sub = threadIdx.x & 3;
-  if (gid >= n_groups) return;  // the four lanes of a group leave together
-  const int64_t g = gid % groups_per_row;
-  const int64_t rr = gid / groups_per_row;
-  const int64_t r = rr % n_rows;
-  const int64_t o = rr / n_rows;
-
-  const uint4 raw = *reinterpret_cast<const uint4 *>(x + o * xo + r * xr + g * 32 + sub * 8);
-  half_t v[8];
-  __builtin_memcpy(v, &raw, 16);
-
-  float mn = (float)v[0], mx = (float)v[0];
-#pragma unroll
-  for (int i = 1; i < 8; ++i) {
-    mn = fminf(mn, (float)v[i]);
-    mx = fmaxf(mx, (float)v[i]);
+  const uint32_t o = blockIdx.x / blocks_per_slab;
+  const uint32_t blk = blockIdx.x - o * blocks_per_slab;
+  const uint32_t gin = blk * 64u + (threadIdx.x >> 2);
+  const uint32_t sub = threadIdx.x & 3;
+  if (gin >= groups_per_slab) return;  // the four lanes of a group leave together
+  uint32_t r, g;
+  if (gpr_shift >= 0) {
+    r = gin >> gpr_shift;
+    g = gin & (groups_per_row - 1u);
+  } else {
+    r = gin / groups_per_row;
+    g = gin - r * groups_per_row;
   }
-  mn = fminf(mn, xor_f(mn, 1));
-  mx = fmaxf(mx, xor_f(mx, 1));
-  mn = fminf(mn, xor_f(mn, 2));
-  mx = fmaxf(mx, xor_f(mx, 2));
+
+  const uint4 raw = *reinterpret_cast<const uint4 *>(x + (int64_t)o * xo + (int64_t)r * xr + g * 32u + sub * 8u);
+  const half2_t p[4] = {bits_h2(raw.x), bits_h2(raw.y), bits_h2(raw.z), bits_h2(raw.w)};
+
+  half2_t lo2 = __builtin_elementwise_min(__builtin_elementwise_min(p[0], p[1]), __builtin_elementwise_min(p[2], p[3]));
+  half2_t hi2 = __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]), __builtin_elementwise_max(p[2], p[3]));
+  // (min, -max) in one register: one packed min per butterfly step serves both
+  half2_t mm = {(half_t)__builtin_fminf((float)lo2[0], (float)lo2[1]), (half_t)(-__builtin_fmaxf((float)hi2[0], (float)hi2[1]))};
+  mm = __builtin_elementwise_min(mm, bits_h2(xor_u(h2_bits(mm), 1)));
+  mm = __builtin_elementwise_min(mm, bits_h2(xor_u(h2_bits(mm), 2)));
+  const half_t mn_h = mm[0];
+  const float mn = (float)mn_h, mx = -(float)mm[1];
 
   const half_t d = (half_t)(mx - mn);
   const half_t sc = (half_t)((float)d * INV_QMAX);
-  const float sc_f = (float)sc;
+  const float rcp = group_recip((float)sc);
 
-  uint32_t c[8];
+  const half2_t mn2 = {mn_h, mn_h};
+  float u[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) c[i] = quant_one<BITS>(v[i], mn, sc_f);
+  for (int i = 0; i < 4; ++i) {
+    const half2_t c = p[i] - mn2;
+    u[2 * i] = (float)c[0];
+    u[2 * i + 1] = (float)c[1];
+  }
 
-  uint32_t *crow = code + o * co + r * cr + g * (32 / PF);
-  if (BITS == 2) {
-    uint32_t h = 0;
+  uint32_t *crow = code + (int64_t)o * co + (int64_t)r * cr + g * (32 / PF);
+  if (BITS == 8) {
+    uint32_t z[2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h |= c[i] << (2 * i);
-    const uint32_t other = xor_u(h, 1);
-    if ((sub & 1) == 0) crow[sub >> 1] = h | (other << 16);
-  } else if (BITS == 4) {
-    uint32_t w = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) w |= c[i] << (4 * i);
-    crow[sub] = w;
+    for (int h = 0; h < 2; ++h) {
+      z[0] = code_pair_biased<8>(u[4 * h + 0], rcp, u[4 * h + 2], rcp);
+      z[1] = code_pair_biased<8>(u[4 * h + 1], rcp, u[4 * h + 3], rcp);
+      crow[sub * 2 + h] = horner_pack<8, 2>(z);
+    }
   } else {
-    crow[sub * 2 + 0] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
-    crow[sub * 2 + 1] = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+    uint32_t z[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) z[i] = code_pair_biased<BITS>(u[i], rcp, u[i + 4], rcp);
+    if (BITS == 4) {
+      crow[sub] = horner_pack<4, 4>(z);
+    } else {
+      const uint32_t w = horner_pack<2, 4>(z);             // codes 0-3 in byte 0, codes 4-7 in byte 2
+      const uint32_t h = __builtin_amdgcn_perm(0u, w, 0x0c0c0200u);   // 16 bits: this lane's 8 codes
+      const uint32_t other = xor_u(h, 1);
+      if ((sub & 1) == 0) crow[sub >> 1] = h | (other << 16);
+    }
   }
   if (sub == 0) {
-    scale[o * so + r * sr + g] = sc;
-    zero[o * so + r * sr + g] = (half_t)mn;
+    scale[(int64_t)o * so + (int64_t)r * sr + g] = sc;
+    zero[(int64_t)o * so + (int64_t)r * sr + g] = mn_h;
   }
 }
 
 // ---------------------------------------------------------------- K handed over token-major
-// One wavefront per (32-token group, outer slab); a lane owns two adjacent channels and keeps the
-// 32 x 2 fp16 tile in registers, so a token row (D fp16) is read as one coalesced 4-byte-per-lane load.
+// A workgroup of 8 wavefronts takes 256 tokens (8 groups of 32) of one slab.  Within a wavefront a lane
+// owns two adjacent channels (lane & 7) of one token group (lane >> 3) and keeps that 32 x 2 fp16 tile in
+// registers; the 8 wavefronts cover 128 channels per pass.  The eight lanes that share a channel pair hold
+// eight consecutive token groups, so each channel row of the code / scale / zero planes is written in runs
+// of 8 groups (64 to 256 bytes of codes) instead of one group at a time.
+constexpr int QK_GROUPS_PER_BLOCK = 8;
+
 template <int BITS>
-__global__ __launch_bounds__(64) void quant_k_tokenmajor_kernel(
+__global__ __launch_bounds__(512) void quant_k_tokenmajor_kernel(
     const half_t *__restrict__ x, int64_t xo, int64_t xt, uint32_t *__restrict__ code, int64_t co,
     int64_t cr, half_t *__restrict__ scale, half_t *__restrict__ zero, int64_t so, int64_t sr,
-    int64_t D) {
+    uint32_t D, uint32_t n_groups) {
   constexpr int PF = 32 / BITS;
   constexpr int WPG = 32 / PF;  // words per group
+  constexpr int HALF = PF / 2;
   constexpr float INV_QMAX = 1.0f / (float)((1 << BITS) - 1);
-  const int64_t g = blockIdx.x;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t cp = lane & 7u, tg = lane >> 3;
+  const uint32_t G0 = blockIdx.x * QK_GROUPS_PER_BLOCK;
+  const uint32_t G = G0 + tg;
   const int64_t o = blockIdx.y;
-  const half_t *xb = x + o * xo + g * 32 * xt;
-  for (int64_t cp = threadIdx.x; cp * 2 < D; cp += 64) {
+  const uint32_t row_b = (uint32_t)xt * 2u;  // bytes between token rows
+  const uint32_t groups_here = min((uint32_t)QK_GROUPS_PER_BLOCK, n_groups - G0);
+  const rsrc_t rx = make_rsrc(x + o * xo + (int64_t)G0 * 32 * xt, (groups_here * 32u - 1u) * row_b + D * 2u);
+
+  for (uint32_t c0 = wv * 16u; c0 < D; c0 += 128u) {
+    const uint32_t c = c0 + cp * 2u;
+    const bool live = (G < n_groups) && (c < D);
+    const uint32_t voff = live ? tg * 32u * row_b + c * 2u : 0u;  // idle lanes re-read the first element
     half2_t t[32];
 #pragma unroll
-    for (int k = 0; k < 32; ++k) t[k] = *reinterpret_cast<const half2_t *>(xb + k * xt + cp * 2);
+    for (int k = 0; k < 32; ++k) t[k] = bits_h2(buf_u32(rx, voff, (uint32_t)k * row_b));
+
+    half2_t lo2 = t[0], hi2 = t[0];
+#pragma unroll
+    for (int k = 1; k < 32; ++k) {
+      lo2 = __builtin_elementwise_min(lo2, t[k]);
+      hi2 = __builtin_elementwise_max(hi2, t[k]);
+    }
+    half_t sc[2];
+    float rcp[2];
 #pragma unroll
     for (int ch = 0; ch < 2; ++ch) {
-      float mn = (float)t[0][ch], mx = (float)t[0][ch];
-#pragma unroll
-      for (int k = 1; k < 32; ++k) {
-        mn = fminf(mn, (float)t[k][ch]);
-        mx = fmaxf(mx, (float)t[k][ch]);
-      }
-      const half_t d = (half_t)(mx - mn);
-      const half_t sc = (half_t)((float)d * INV_QMAX);
-      const float sc_f = (float)sc;
-      const int64_t c_idx = cp * 2 + ch;
-      uint32_t *crow = code + o * co + c_idx * cr + g * WPG;
-#pragma unroll
-      for (int wj = 0; wj < WPG; ++wj) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int i = 0; i < PF; ++i) w |= quant_one<BITS>(t[wj * PF + i][ch], mn, sc_f) << (i * BITS);
-        crow[wj] = w;
-      }
-      scale[o * so + c_idx * sr + g] = sc;
-      zero[o * so + c_idx * sr + g] = (half_t)mn;
+      const half_t d = (half_t)((float)hi2[ch] - (float)lo2[ch]);
+      sc[ch] = (half_t)((float)d * INV_QMAX);
+      rcp[ch] = group_recip((float)sc[ch]);
     }
+    float u[2][32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      const half2_t cpair = t[k] - lo2;
+      u[0][k] = (float)cpair[0];
+      u[1][k] = (float)cpair[1];
+    }
+    if (live) {
+#pragma unroll
+      for (int ch = 0; ch < 2; ++ch) {
+        uint32_t *crow = code + o * co + (int64_t)(c + ch) * cr + (int64_t)G * WPG;
+#pragma unroll
+        for (int wj = 0; wj < WPG; ++wj) {
+          uint32_t z[HALF];
+#pragma unroll
+          for (int i = 0; i < HALF; ++i)
+            z[i] = code_pair_biased<BITS>(u[ch][wj * PF + i], rcp[ch], u[ch][wj * PF + i + HALF], rcp[ch]);
+          crow[wj] = horner_pack<BITS, HALF>(z);
+        }
+        scale[o * so + (int64_t)(c + ch) * sr + G] = sc[ch];
+        zero[o * so + (int64_t)(c + ch) * sr + G] = lo2[ch];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- exhaustive check of the division
+// Every pair of fp16 bit patterns (u, s): v' = rnd16(f32(u) * group_recip(f32(s))) against the correctly
+// rounded v = rnd16(f32(u) / f32(s)), and the 8-bit codes rne(clamp(., 0, 255)) of both (the 4- and 2-bit
+// codes are min(code8, qmax)).  The two quotients can differ only where v is an fp16 denormal: there the
+// fp16 grid is coarse enough for u/s to fall exactly on a midpoint, and the product's last-place error
+// decides the tie -- some 30000 times below the 0.5 at which a code changes.
+// counts[0]: code mismatches over all 2^32 pairs; counts[1]: code mismatches with both sign bits clear
+// (the quantiser's domain: u = x - min >= 0, s = range / qmax >= 0, or NaN); counts[2]: pairs with
+// v' != v (two NaNs count as equal); counts[3]: the largest |v| (as fp16 bits) among those.
+__device__ __forceinline__ int code8_of(half_t v) {
+  const float c = __builtin_fminf(__builtin_fmaxf((float)v, 0.0f), 255.0f);
+  return (int)__builtin_rintf(c);
+}
+
+__global__ __launch_bounds__(256) void selftest_division_kernel(unsigned long long *counts) {
+  const uint32_t sbits = blockIdx.x;  // 65536 blocks: one scale pattern each
+  half_t s;
+  {
+    const unsigned short b = (unsigned short)sbits;
+    __builtin_memcpy(&s, &b, 2);
+  }
+  const float sf = (float)s;
+  const float rcp = group_recip(sf);
+  unsigned long long bad_all = 0, bad_dom = 0, bad_v = 0, max_v = 0;
+  for (uint32_t ub = threadIdx.x; ub < 65536u; ub += 256u) {
+    half_t u;
+    const unsigned short b = (unsigned short)ub;
+    __builtin_memcpy(&u, &b, 2);
+    const float uf = (float)u;
+    const half_t fast = (half_t)(uf * rcp);
+    const half_t ref = (half_t)(uf / sf);
+    unsigned short fb, rb;
+    __builtin_memcpy(&fb, &fast, 2);
+    __builtin_memcpy(&rb, &ref, 2);
+    const bool both_nan = (fast != fast) && (ref != ref);
+    if (fb != rb && !both_nan) {
+      ++bad_v;
+      const unsigned long long mag = rb & 0x7fffu;
+      max_v = mag > max_v ? mag : max_v;
+    }
+    if (code8_of(fast) != code8_of(ref)) {
+      ++bad_all;
+      if (((ub | sbits) & 0x8000u) == 0) ++bad_dom;
+    }
+  }
+  if (bad_all) atomicAdd(&counts[0], bad_all);
+  if (bad_dom) atomicAdd(&counts[1], bad_dom);
+  if (bad_v) {
+    atomicAdd(&counts[2], bad_v);
+    atomicMax(&counts[3], max_v);
   }
 }
 
@@ -204,14 +351,18 @@ extern "C" int hqekv_quant_pack_rows(const void *x, int64_t xo, int64_t xr, void
   if (!x || !code || !scale || !zero) return fail(HQEKV_E_ARG, "quant_pack_rows: null pointer");
   if (((uintptr_t)x & 15) || (xo % 8) || (xr % 8))
     return fail(HQEKV_E_ALIGN, "quant_pack_rows: x rows must be 16-byte aligned");
-  const int64_t blocks = (n_groups + 63) / 64;
-  if (blocks > 0x7fffffffLL) return fail(HQEKV_E_ARG, "quant_pack_rows: too many groups");
+  const int64_t gpr = L / 32, gps = n_rows * gpr;
+  const int64_t bps = (gps + 63) / 64;
+  if (gps > 0x7fffffffLL || bps * n_outer > 0x7fffffffLL)
+    return fail(HQEKV_E_ARG, "quant_pack_rows: too many groups");
+  int shift = -1;
+  if ((gpr & (gpr - 1)) == 0) for (shift = 0; (1LL << shift) < gpr; ++shift) {}
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)blocks), block(256);
+  dim3 grid((unsigned)(bps * n_outer)), block(256);
 #define LAUNCH(B_)                                                                              \
   hipLaunchKernelGGL(quant_rows_kernel<B_>, grid, block, 0, st, (const half_t *)x, xo, xr,     \
-                     (uint32_t *)code, co, cr, (half_t *)scale, (half_t *)zero, so, sr, n_rows, \
-                     L / 32, n_groups)
+                     (uint32_t *)code, co, cr, (half_t *)scale, (half_t *)zero, so, sr,         \
+                     (uint32_t)gpr, shift, (uint32_t)gps, (uint32_t)bps)
   if (bits == 2) LAUNCH(2); else if (bits == 4) LAUNCH(4); else LAUNCH(8);
 #undef LAUNCH
   return check_launch("quant_rows_kernel");
@@ -230,14 +381,27 @@ extern "C" int hqekv_quant_pack_k_tokenmajor(const void *x, int64_t xo, int64_t 
   if (((uintptr_t)x & 3) || (xo % 2) || (xt % 2))
     return fail(HQEKV_E_ALIGN, "quant_pack_k_tokenmajor: x rows must be 4-byte aligned");
   if (n_outer > 65535) return fail(HQEKV_E_ARG, "quant_pack_k_tokenmajor: n_outer > 65535");
+  // 32-bit byte offsets inside one block of 256 token rows
+  if (xt < D || xt > (1LL << 22) || D > (1LL << 22) || T / 32 > 0x7fffffffLL)
+    return fail(HQEKV_E_ARG, "quant_pack_k_tokenmajor: need D <= xt <= 2^22 (xt=%lld D=%lld)", (long long)xt, (long long)D);
+  const int64_t n_groups = T / 32;
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)(T / 32), (unsigned)n_outer), block(64);
+  dim3 grid((unsigned)((n_groups + QK_GROUPS_PER_BLOCK - 1) / QK_GROUPS_PER_BLOCK), (unsigned)n_outer), block(512);
 #define LAUNCH(B_)                                                                                  \
   hipLaunchKernelGGL(quant_k_tokenmajor_kernel<B_>, grid, block, 0, st, (const half_t *)x, xo, xt, \
-                     (uint32_t *)code, co, cr, (half_t *)scale, (half_t *)zero, so, sr, D)
+                     (uint32_t *)code, co, cr, (half_t *)scale, (half_t *)zero, so, sr,             \
+                     (uint32_t)D, (uint32_t)n_groups)
   if (bits == 2) LAUNCH(2); else if (bits == 4) LAUNCH(4); else LAUNCH(8);
 #undef LAUNCH
   return check_launch("quant_k_tokenmajor_kernel");
+}
+
+extern "C" int hqekv_selftest_quant_division(void *counts, void *stream) {
+  if (!counts) return fail(HQEKV_E_ARG, "selftest_quant_division: null pointer");
+  if ((uintptr_t)counts & 7) return fail(HQEKV_E_ALIGN, "selftest_quant_division: counts must be 8-byte aligned");
+  hipLaunchKernelGGL(selftest_division_kernel, dim3(65536), dim3(256), 0, (hipStream_t)stream,
+                     (unsigned long long *)counts);
+  return check_launch("selftest_division_kernel");
 }
 
 extern "C" int hqekv_dequant_unpack_rows(const void *code, int64_t co, int64_t cr, const void *scale,

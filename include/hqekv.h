@@ -77,6 +77,17 @@ int hqekv_dequant_unpack_rows(const void *code, int64_t code_outer_stride, int64
                               int64_t out_row_stride, int64_t n_outer, int64_t n_rows, int64_t L,
                               int bits, void *stream);
 
+/* No counterpart in the reference: a device-side proof obligation of the quantiser above.  The kernels
+ * evaluate the reference's v = u / scale (quant/pack_unpack.py:173, fp16 operands, fp32 divide, fp16
+ * result) as u * (1/scale); this call compares the two over all 2^32 pairs of fp16 bit patterns.
+ * counts: 4 x uint64 on the device, zeroed by the caller.  [0] pairs whose 8-bit code
+ * rne(clamp(v, 0, 255)) differs (the 4- and 2-bit codes are min(code8, qmax)), [1] the same with both sign
+ * bits clear (the quantiser's domain), [2] pairs whose fp16 quotient differs at all, [3] the largest |v|
+ * (fp16 bit pattern) among those: below 0x0400, i.e. only ties among fp16 denormals, which all round to
+ * code 0.
+ */
+int hqekv_selftest_quant_division(void *counts, void *stream);
+
 /* Replaces pack_along_last_dim (quant/pack_unpack.py:16-70): q is (n_rows, L) int32 codes,
  * code is (n_rows, L/pf) int32, both contiguous. */
 int hqekv_pack_i32(const void *q, void *code, int64_t n_rows, int64_t L, int bits, void *stream);

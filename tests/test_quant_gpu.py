@@ -167,3 +167,35 @@ def test_dequant_keeps_the_two_fp16_roundings(dev):
     q[..., 0] = 1.0
     out = cuda_bmm_fA_qB_uniform_group(32, q.to(dev), code.to(dev), s.to(dev), z.to(dev), 4)
     assert out[0, 0, 0, 0].item() == 2052.0 and out[0, 0, 0, 1].item() == 2050.0
+
+
+@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("magnitude", [2.0 ** -21, 2.0 ** -14, 9000.0])
+def test_quant_denormal_and_near_overflow_ranges_both_layouts(dev, bit, magnitude):
+    """Scales that are fp16 denormals, underflow to zero, or sit next to overflow; constant and one-hot groups."""
+    from hqekv_amd import pack_unpack as P
+    g = torch.Generator().manual_seed(int(magnitude * 2 ** 22) % 9973 + bit)
+    x = (torch.randn(1, 2, 64, 128, generator=g) * magnitude).half()
+    x[0, 0, :8] = x[0, 0, :8, :1]                      # constant rows
+    x[0, 1, :, 5] = x[0, 1, :1, 5]                     # constant column
+    x[0, 1, 7, 40] += torch.tensor(magnitude * 2 ** -3).half()
+    for data in (x, x.transpose(2, 3)):                # rows kernel, token-major K kernel
+        code, scale, mn = P.uniform_group_quantize_pack_last_dim(data.to(dev), 32, bit)
+        oc, os_, om = O.uniform_group_quantize_pack_last_dim(data.contiguous(), 32, bit)
+        assert torch.equal(code.cpu(), oc)
+        assert torch.equal(scale.cpu().view(torch.int16), os_.view(torch.int16))
+        assert torch.equal(mn.cpu().view(torch.int16), om.view(torch.int16))
+
+
+def test_reciprocal_division_matches_true_division_for_every_fp16_pair(dev):
+    """The quantiser's u * (1/scale) against the correctly rounded u / scale, all 2^32 operand pairs."""
+    from hqekv_amd import _lib
+    counts = torch.zeros(4, dtype=torch.int64, device=dev)
+    _lib.check(_lib.load().hqekv_selftest_quant_division(counts.data_ptr(), _lib.stream_ptr(counts.device)),
+               "selftest_quant_division")
+    torch.cuda.synchronize()
+    c = counts.cpu().tolist()
+    assert c[1] == 0, f"{c[1]} code mismatches in the quantiser's domain"
+    assert c[0] == 0, f"{c[0]} code mismatches over all pairs"
+    # the quotients themselves may differ only on exact ties among fp16 denormals (|v| < 2^-14)
+    assert c[3] < 0x0400, f"quotients differ at |v| bits {c[3]:#06x} ({c[2]} pairs)"
