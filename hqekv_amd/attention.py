@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 
-BITS = (8, 4, 2)
+BITS = (8, 4, 2, 1)   # 1: the uniform 1-bit class of the 'uniform_group' strategy (32 codes per word)
 K_BASE = {8: 4, 4: 12, 2: 20, 1: 28}
 V_BASE = {8: 8, 4: 16, 2: 24, 1: 32}
 K16, K16_IDX, V16, V16_IDX = 0, 1, 2, 3
@@ -49,7 +49,15 @@ def _f16_k_item(k16: torch.Tensor, idx, keep: list) -> dict:
     return dict(bits=16, n_tokens=T, data=data, idx=idx, token_major=tm)
 
 
-def key_segments(pkv: tuple, dev, Tall: int, keep: list) -> Tuple[List[dict], int, int]:
+def _check_one_bit(pkv: tuple, base: int, low_uniform: bool) -> None:
+    if pkv[base] is not None and not low_uniform:
+        raise NotImplementedError(
+            "under 'high_uniform_group_low_normal_group' the 1-bit class is the normal-quantile one, which is "
+            "not built (the uniform 1-bit class of 'uniform_group' is)")
+
+
+def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True) -> Tuple[List[dict], int, int]:
+    _check_one_bit(pkv, K_BASE[1], low_uniform)
     items = []
     nh_kv = D = None
     if pkv[K16] is not None:
@@ -66,8 +74,6 @@ def key_segments(pkv: tuple, dev, Tall: int, keep: list) -> Tuple[List[dict], in
             idx = _idx(pkv[base + 1], n, dev)
             keep += [code, sc, zr, idx]
             items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx))
-    if pkv[K_BASE[1]] is not None:
-        raise NotImplementedError("the 1-bit normal-quantile class is not built")
     new_K = pkv[NEW_K]
     if new_K is not None and new_K.shape[2] > 0:
         nk = new_K.contiguous()
@@ -78,7 +84,8 @@ def key_segments(pkv: tuple, dev, Tall: int, keep: list) -> Tuple[List[dict], in
     return items, nh_kv, D
 
 
-def value_segments(pkv: tuple, dev, Tall: int, keep: list) -> Tuple[List[dict], int, int]:
+def value_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True) -> Tuple[List[dict], int, int]:
+    _check_one_bit(pkv, V_BASE[1], low_uniform)
     items = []
     nh_kv = D = None
     if pkv[V16] is not None:
@@ -97,8 +104,6 @@ def value_segments(pkv: tuple, dev, Tall: int, keep: list) -> Tuple[List[dict], 
             idx = _idx(pkv[base + 1], n, dev)
             keep += [code, sc, zr, idx]
             items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx))
-    if pkv[V_BASE[1]] is not None:
-        raise NotImplementedError("the 1-bit normal-quantile class is not built")
     new_V = pkv[NEW_V]
     if new_V is not None and new_V.shape[2] > 0:
         nv = new_V.contiguous()
@@ -167,7 +172,8 @@ def default_flags() -> int:
     return 0 if os.environ.get("HQEKV_UNFUSED", "0") == "1" else _lib.FUSE_SOFTMAX
 
 
-def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool, flags: Optional[int] = None):
+def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool, flags: Optional[int] = None,
+                     low_uniform: bool = True):
     """q (B,Hq,1,D) fp16 -> (attn_weights (B,Hq,1,Tall) fp16 probabilities, attn_output (B,Hq,1,D) fp16).
 
     One q.K^T launch over all K classes and one p.V launch over all V classes with the softmax fused
@@ -182,8 +188,8 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     B, Hq, _, D = q.shape
     dev = q.device
     keep: list = []
-    k_items, hk, dk = key_segments(pkv, dev, Tall, keep)
-    v_items, hv, dv = value_segments(pkv, dev, Tall, keep)
+    k_items, hk, dk = key_segments(pkv, dev, Tall, keep, low_uniform)
+    v_items, hv, dv = value_segments(pkv, dev, Tall, keep, low_uniform)
     Hkv = hk if hk is not None else hv
     if Hkv is None:
         raise ValueError("invalid past_key_value")

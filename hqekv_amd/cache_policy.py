@@ -73,10 +73,10 @@ def _none_if_empty(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
 
 
 def _check_low_bits(bits: int, strategy: str) -> None:
-    if bits == 1:
+    if bits == 1 and strategy != "uniform_group":
         raise NotImplementedError(
-            "a populated 1-bit class needs the 1-bit quantisers (normal-quantile, or uniform with 32 codes per "
-            "word), which are not built; run with a zero 1-bit share")
+            "under 'high_uniform_group_low_normal_group' a populated 1-bit class needs the normal-quantile "
+            "quantisers, which are not built; use 'uniform_group' (uniform 1-bit class) or a zero 1-bit share")
     if strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
         raise NotImplementedError(f"quant_strategy '{strategy}' uses quantiser families that are not built")
 

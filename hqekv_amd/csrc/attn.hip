@@ -146,6 +146,10 @@ __device__ __forceinline__ void consume_byte(uint32_t u, half2_t s2, half2_t z2,
   HQ_FIELD(1)
   HQ_FIELD(2)
   HQ_FIELD(3)
+  HQ_FIELD(4)
+  HQ_FIELD(5)
+  HQ_FIELD(6)
+  HQ_FIELD(7)
 #undef HQ_FIELD
 }
 
@@ -171,8 +175,9 @@ __host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
   return (bits == 16 && token_major) ? 64 : QK_TILE;
 }
 
-// Accumulate one quantised tile: 512 tokens x D channels.  A lane owns 8 consecutive tokens: half a
-// packed word at 2 bits (two lanes read the same word), one word at 4 bits, two words at 8 bits.
+// Accumulate one quantised tile: 512 tokens x D channels.  A lane owns 8 consecutive tokens: a byte of a
+// packed word at 1 bit (four lanes read the same word), half a word at 2 bits, one word at 4 bits, two
+// words at 8 bits.
 // QK_UNR row pairs at a time: every load of a block is issued before its first use, and the rolled outer
 // loop keeps the code small enough to stay in the instruction cache from one launch to the next.
 template <int BITS, int NREP, int QK_WAVES>
@@ -185,7 +190,9 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
   const uint32_t gpr = n >> 5;   // groups per row
   const uint32_t wofs = (ts / PF) * 4u;  // byte offset of this lane's first word inside a row
   const uint32_t gofs = (ts >> 5) * 2u;  // byte offset of this lane's group inside a scale/zero row
-  const int sh2 = (BITS == 2) ? (int)((ts >> 3) & 1) * 16 : 0;  // which half of the 2-bit word
+  const int sh2 = (BITS == 2) ? (int)((ts >> 3) & 1) * 16      // which half of the 2-bit word
+                  : (BITS == 1) ? (int)((ts >> 3) & 3) * 8     // which byte of the 1-bit word
+                                : 0;
   const rsrc_t rc = make_rsrc((const uint32_t *)sg.data + (int64_t)bh * D * wpr, (uint32_t)D * wpr * 4u);
   const rsrc_t rs = make_rsrc(sg.scale + (int64_t)bh * D * gpr, (uint32_t)D * gpr * 2u);
   const rsrc_t rz = make_rsrc(sg.zero + (int64_t)bh * D * gpr, (uint32_t)D * gpr * 2u);
@@ -218,7 +225,10 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
 #pragma unroll
       for (int h = 0; h < NREP; ++h) q2[h] = q2s[dp * NREP + h];
       const half2_t s2 = pack_h2(s0[k], s1[k]), z2 = pack_h2(z0[k], z1[k]);
-      if (BITS == 2) {
+      if (BITS == 1) {
+        const uint32_t a0 = w0[k][0] >> sh2, a1 = w1[k][0] >> sh2;
+        consume_byte<1, NREP, QK_TPL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
+      } else if (BITS == 2) {
         const uint32_t a0 = w0[k][0] >> sh2, a1 = w1[k][0] >> sh2;
         consume_byte<2, NREP, QK_TPL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
         consume_byte<2, NREP, QK_TPL>(byte_pair<1>(a0, a1), s2, z2, q2, acc, 4);
@@ -397,6 +407,7 @@ __global__ __launch_bounds__(QK_WAVES * 64) void qk_hybrid_kernel(SegTable tb, c
 #pragma unroll
     for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {
+    case 1: qk_quant_accumulate<1, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
     case 2: qk_quant_accumulate<2, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
     case 4: qk_quant_accumulate<4, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
     case 8: qk_quant_accumulate<8, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
@@ -668,8 +679,8 @@ __device__ __forceinline__ void pv_commit(const PvPair<NREP, NG> &pr, half_t *co
   }
 }
 
-// One class chunk.  16 lanes cover a token row (8 channels each: half a packed word at 2 bits, one word
-// at 4 bits, two words at 8 bits, 16 bytes of fp16), 4 token pairs per wave step, so the reduction over
+// One class chunk.  16 lanes cover a token row (8 channels each: a byte of a packed word at 1 bit, half a
+// word at 2 bits, one word at 4 bits, two words at 8 bits, 16 bytes of fp16), 4 token pairs per wave step, so the reduction over
 // tokens needs only two butterfly steps across lanes.  Code words are requested one step-block ahead of
 // their use, and the staging requests of a block are issued before the previous block is consumed.
 template <int BITS, int NREP, int D>
@@ -684,8 +695,8 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
   constexpr int UNR = PV_UNR / WPL;                           // wave steps per block: 8 words in flight per lane
   const int cl = lane & 15, tl = lane >> 4;
   const int g = cl >> 2;
-  const int sh2 = (BITS == 2) ? (cl & 1) * 16 : 0;
-  const uint32_t wofs = (BITS == 2 ? (cl >> 1) : cl * WPL) * 4u;  // byte offset inside a token row
+  const int sh2 = (BITS == 2) ? (cl & 1) * 16 : (BITS == 1) ? (cl & 3) * 8 : 0;
+  const uint32_t wofs = (BITS == 1 ? (cl >> 2) : BITS == 2 ? (cl >> 1) : cl * WPL) * 4u;  // byte offset inside a token row
   const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * sg.n_tokens * ROWB, (uint32_t)(sg.n_tokens * ROWB));
   const uint32_t lane_off = (uint32_t)(2 * tl) * ROWB + wofs;   // this lane's first token of a step + word
 
@@ -752,7 +763,10 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
           } else {
             const uint2 sz = st.sz[tp][g];
             const half2_t s2 = as_h2(sz.x), z2 = as_h2(sz.y);
-            if (BITS == 2) {
+            if (BITS == 1) {
+              const uint32_t a0 = cur.w0[k][0] >> sh2, a1 = cur.w1[k][0] >> sh2;
+              consume_byte<1, NREP, PV_CPL>(byte_pair<0>(a0, a1), s2, z2, p2, acc, 0);
+            } else if (BITS == 2) {
               const uint32_t a0 = cur.w0[k][0] >> sh2, a1 = cur.w1[k][0] >> sh2;
               consume_byte<2, NREP, PV_CPL>(byte_pair<0>(a0, a1), s2, z2, p2, acc, 0);
               consume_byte<2, NREP, PV_CPL>(byte_pair<1>(a0, a1), s2, z2, p2, acc, 4);
@@ -823,6 +837,7 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
 #pragma unroll
     for (int i = 0; i < PV_CPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {  // (the first barrier inside pv_chunk also publishes sm_ml)
+    case 1: pv_chunk<1, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
     case 2: pv_chunk<2, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
     case 4: pv_chunk<4, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
     case 8: pv_chunk<8, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
@@ -895,8 +910,8 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
     const hqekv_seg &s = segs[k];
     if (s.n_tokens < 0) return fail(HQEKV_E_ARG, "%s: segment %d has negative n_tokens", who, k);
     if (s.n_tokens == 0) continue;
-    if (!(s.bits == 16 || s.bits == 8 || s.bits == 4 || s.bits == 2))
-      return fail(HQEKV_E_ARG, "%s: segment %d bits=%d (must be 16, 8, 4 or 2)", who, k, s.bits);
+    if (!(s.bits == 16 || s.bits == 8 || s.bits == 4 || s.bits == 2 || s.bits == 1))
+      return fail(HQEKV_E_ARG, "%s: segment %d bits=%d (must be 16, 8, 4, 2 or 1)", who, k, s.bits);
     if (!s.data) return fail(HQEKV_E_ARG, "%s: segment %d has null data", who, k);
     if (s.bits != 16) {
       if (!s.scale || !s.zero) return fail(HQEKV_E_ARG, "%s: segment %d lacks scale/zero", who, k);
@@ -1189,7 +1204,7 @@ extern "C" int64_t hqekv_gemv_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv
 extern "C" int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale, const void *zero,
                                         void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N,
                                         int bits, void *workspace, int64_t workspace_bytes, void *stream) {
-  if (!(bits == 2 || bits == 4 || bits == 8)) return fail(HQEKV_E_ARG, "gemv_uniform_group: bits=%d", bits);
+  if (!(bits == 1 || bits == 2 || bits == 4 || bits == 8)) return fail(HQEKV_E_ARG, "gemv_uniform_group: bits=%d", bits);
   if (K <= 0 || N <= 0 || N % 32 != 0) return fail(HQEKV_E_ARG, "gemv_uniform_group: need N %% 32 == 0, K > 0");
   hqekv_seg s{};
   s.bits = bits;

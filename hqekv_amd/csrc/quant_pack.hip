@@ -138,6 +138,12 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(
     for (int i = 0; i < 4; ++i) z[i] = code_pair_biased<BITS>(u[i], rcp, u[i + 4], rcp);
     if (BITS == 4) {
       crow[sub] = horner_pack<4, 4>(z);
+    } else if (BITS == 1) {
+      const uint32_t w = horner_pack<1, 4>(z);             // codes 0-3 in bits 0-3, codes 4-7 in bits 16-19
+      const uint32_t b8 = (w & 0xfu) | ((w >> 12) & 0xf0u);  // this lane's 8 codes
+      const uint32_t b16 = b8 | (xor_u(b8, 1) << 8);        // even lanes: two lanes' codes in order
+      const uint32_t other = xor_u(b16, 2);
+      if (sub == 0) crow[0] = b16 | (other << 16);
     } else {
       const uint32_t w = horner_pack<2, 4>(z);             // codes 0-3 in byte 0, codes 4-7 in byte 2
       const uint32_t h = __builtin_amdgcn_perm(0u, w, 0x0c0c0200u);   // 16 bits: this lane's 8 codes
@@ -333,7 +339,7 @@ __global__ __launch_bounds__(256) void pack_i32_kernel(const int32_t *__restrict
   code[wid] = w;
 }
 
-static inline bool bits_ok(int bits) { return bits == 2 || bits == 4 || bits == 8; }
+static inline bool bits_ok(int bits) { return bits == 1 || bits == 2 || bits == 4 || bits == 8; }
 
 }  // namespace hq
 
@@ -343,7 +349,7 @@ extern "C" int hqekv_quant_pack_rows(const void *x, int64_t xo, int64_t xr, void
                                      int64_t cr, void *scale, void *zero, int64_t so, int64_t sr,
                                      int64_t n_outer, int64_t n_rows, int64_t L, int bits,
                                      void *stream) {
-  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "quant_pack_rows: bits must be 2, 4 or 8 (got %d)", bits);
+  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "quant_pack_rows: bits must be 1, 2, 4 or 8 (got %d)", bits);
   if (n_outer < 0 || n_rows < 0 || L < 0 || L % 32 != 0)
     return fail(HQEKV_E_ARG, "quant_pack_rows: L=%lld must be a non-negative multiple of 32", (long long)L);
   const int64_t n_groups = n_outer * n_rows * (L / 32);
@@ -363,7 +369,7 @@ extern "C" int hqekv_quant_pack_rows(const void *x, int64_t xo, int64_t xr, void
   hipLaunchKernelGGL(quant_rows_kernel<B_>, grid, block, 0, st, (const half_t *)x, xo, xr,     \
                      (uint32_t *)code, co, cr, (half_t *)scale, (half_t *)zero, so, sr,         \
                      (uint32_t)gpr, shift, (uint32_t)gps, (uint32_t)bps)
-  if (bits == 2) LAUNCH(2); else if (bits == 4) LAUNCH(4); else LAUNCH(8);
+  if (bits == 1) LAUNCH(1); else if (bits == 2) LAUNCH(2); else if (bits == 4) LAUNCH(4); else LAUNCH(8);
 #undef LAUNCH
   return check_launch("quant_rows_kernel");
 }
@@ -372,7 +378,7 @@ extern "C" int hqekv_quant_pack_k_tokenmajor(const void *x, int64_t xo, int64_t 
                                              int64_t co, int64_t cr, void *scale, void *zero,
                                              int64_t so, int64_t sr, int64_t n_outer, int64_t T,
                                              int64_t D, int bits, void *stream) {
-  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "quant_pack_k_tokenmajor: bits must be 2, 4 or 8 (got %d)", bits);
+  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "quant_pack_k_tokenmajor: bits must be 1, 2, 4 or 8 (got %d)", bits);
   if (n_outer < 0 || T < 0 || T % 32 != 0 || D <= 0 || D % 2 != 0)
     return fail(HQEKV_E_ARG, "quant_pack_k_tokenmajor: need T %% 32 == 0 and even D (T=%lld D=%lld)",
                 (long long)T, (long long)D);
@@ -391,7 +397,7 @@ extern "C" int hqekv_quant_pack_k_tokenmajor(const void *x, int64_t xo, int64_t 
   hipLaunchKernelGGL(quant_k_tokenmajor_kernel<B_>, grid, block, 0, st, (const half_t *)x, xo, xt, \
                      (uint32_t *)code, co, cr, (half_t *)scale, (half_t *)zero, so, sr,             \
                      (uint32_t)D, (uint32_t)n_groups)
-  if (bits == 2) LAUNCH(2); else if (bits == 4) LAUNCH(4); else LAUNCH(8);
+  if (bits == 1) LAUNCH(1); else if (bits == 2) LAUNCH(2); else if (bits == 4) LAUNCH(4); else LAUNCH(8);
 #undef LAUNCH
   return check_launch("quant_k_tokenmajor_kernel");
 }
@@ -408,7 +414,7 @@ extern "C" int hqekv_dequant_unpack_rows(const void *code, int64_t co, int64_t c
                                          const void *zero, int64_t so, int64_t sr, void *out,
                                          int64_t oo, int64_t orow, int64_t n_outer, int64_t n_rows,
                                          int64_t L, int bits, void *stream) {
-  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "dequant_unpack_rows: bits must be 2, 4 or 8 (got %d)", bits);
+  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "dequant_unpack_rows: bits must be 1, 2, 4 or 8 (got %d)", bits);
   const int pf = 32 / bits;
   if (n_outer < 0 || n_rows < 0 || L < 0 || L % pf != 0 || (scale && L % 32 != 0))
     return fail(HQEKV_E_ARG, "dequant_unpack_rows: bad L=%lld", (long long)L);
@@ -426,9 +432,9 @@ extern "C" int hqekv_dequant_unpack_rows(const void *code, int64_t co, int64_t c
                      co, cr, (const half_t *)scale, (const half_t *)zero, so, sr, (half_t *)out, \
                      oo, orow, n_rows, L / pf, n_words)
   if (scale) {
-    if (bits == 2) LAUNCH(2, true); else if (bits == 4) LAUNCH(4, true); else LAUNCH(8, true);
+    if (bits == 1) LAUNCH(1, true); else if (bits == 2) LAUNCH(2, true); else if (bits == 4) LAUNCH(4, true); else LAUNCH(8, true);
   } else {
-    if (bits == 2) LAUNCH(2, false); else if (bits == 4) LAUNCH(4, false); else LAUNCH(8, false);
+    if (bits == 1) LAUNCH(1, false); else if (bits == 2) LAUNCH(2, false); else if (bits == 4) LAUNCH(4, false); else LAUNCH(8, false);
   }
 #undef LAUNCH
   return check_launch("dequant_rows_kernel");
@@ -436,7 +442,7 @@ extern "C" int hqekv_dequant_unpack_rows(const void *code, int64_t co, int64_t c
 
 extern "C" int hqekv_pack_i32(const void *q, void *code, int64_t n_rows, int64_t L, int bits,
                               void *stream) {
-  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "pack_i32: bits must be 2, 4 or 8 (got %d)", bits);
+  if (!bits_ok(bits)) return fail(HQEKV_E_ARG, "pack_i32: bits must be 1, 2, 4 or 8 (got %d)", bits);
   const int pf = 32 / bits;
   if (n_rows < 0 || L < 0 || L % pf != 0) return fail(HQEKV_E_ARG, "pack_i32: L %% pf != 0");
   const int64_t n_words = n_rows * (L / pf);
@@ -446,7 +452,8 @@ extern "C" int hqekv_pack_i32(const void *q, void *code, int64_t n_rows, int64_t
   if (blocks > 0x7fffffffLL) return fail(HQEKV_E_ARG, "pack_i32: too many words");
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)blocks), block(256);
-  if (bits == 2) hipLaunchKernelGGL(pack_i32_kernel<2>, grid, block, 0, st, (const int32_t *)q, (uint32_t *)code, n_words);
+  if (bits == 1) hipLaunchKernelGGL(pack_i32_kernel<1>, grid, block, 0, st, (const int32_t *)q, (uint32_t *)code, n_words);
+  else if (bits == 2) hipLaunchKernelGGL(pack_i32_kernel<2>, grid, block, 0, st, (const int32_t *)q, (uint32_t *)code, n_words);
   else if (bits == 4) hipLaunchKernelGGL(pack_i32_kernel<4>, grid, block, 0, st, (const int32_t *)q, (uint32_t *)code, n_words);
   else hipLaunchKernelGGL(pack_i32_kernel<8>, grid, block, 0, st, (const int32_t *)q, (uint32_t *)code, n_words);
   return check_launch("pack_i32_kernel");

@@ -1,0 +1,143 @@
+"""The caller of the decode path: the cache-side state machine of the reference's attention layer
+(``LlamaAttention_hqe.forward``, model/llama_hqe.py:55-251; ``Qwen3Attention_hqe`` has the same cache
+logic) without what surrounds it -- projections, rotary embedding, ``o_proj``.
+
+Per call (model/llama_hqe.py, line numbers in brackets):
+  prefill   attention over the prompt; cache = ``(None,)*39 + (K, V, len)`` [186]
+  decode    ``new_K/new_V = cat(residual, k/v)`` [131-133] -> hybrid attention over the 42-field tuple [136]
+  always    the probabilities feed the ring of the last 20 rows [199]; with >= 32 un-quantised tokens:
+            class sizes from the ratios [216-224] (or layer 0's, handed down as ``auxiliary_parameters``
+            [211-214]), block ranking [228], ``KV_cache_hqe_2`` [230-231], bookkeeping and the ratio
+            update for the next 32-token increment [233-239].
+
+Decode attention, quantisation, demotion and eviction run on the HIP kernels of this package.  The prompt
+attention (outside the quantised path) uses torch: ``scaled_dot_product_attention`` for the output and a
+matmul for the last 20 rows of probabilities, the only rows the ring keeps [146-170].
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .hqe_2 import KV_cache_hqe_2
+from .hqe_matmul import qkv_matmul_hqe_2
+from .public_func import get_block_token_idx, last_attn_weights, make_sum_equal
+
+LAST_TOKEN_NUM = 20
+BLOCK = 32
+
+
+def _repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    if n_rep == 1:
+        return x
+    B, H, T, D = x.shape
+    return x[:, :, None, :, :].expand(B, H, n_rep, T, D).reshape(B, H * n_rep, T, D)
+
+
+class HqeAttentionLayer:
+    """State of one layer: un-quantised length, kept history length, eviction / quantisation ratios and the
+    importance ring.  ``bit_0`` is the evicted share, ``bit_4``/``bit_2``/``bit_1`` the 4-, 2- and 1-bit
+    shares of what is kept (config.bit_* of the reference); two blocks always stay fp16 and the 8-bit
+    share is 0 [216]."""
+
+    def __init__(self, head_dim: int, bit_0: float, bit_4: float, bit_2: float, bit_1: float = 0.0,
+                 quant_strategy: str = "uniform_group", times_range: bool = True,
+                 last_length: int = LAST_TOKEN_NUM):
+        self.head_dim = head_dim
+        self.scaling = head_dim ** -0.5
+        self.quant_strategy = quant_strategy
+        self.times_range = times_range
+        self.ratio_e_0 = torch.tensor([bit_0], dtype=torch.float32)
+        self.ratio_e = self.ratio_e_0.clone()
+        self.ratio_q = torch.tensor([bit_4, bit_2, bit_1], dtype=torch.float32)
+        self.current_length = 0
+        self.history_reserve_length = 0
+        self.token_num = 0
+        self.last_weights = last_attn_weights(last_length=last_length)
+
+    def reset(self) -> None:
+        """What the reference's ``generate`` does per layer before a new prompt [555-557]."""
+        self.current_length = 0
+        self.history_reserve_length = 0
+        self.token_num = 0
+        self.ratio_e = self.ratio_e_0.clone()
+        self.last_weights.reset()
+
+    def set_max_length(self, max_length: int) -> None:
+        """Prompt length + new tokens: the width of the importance ring [691-695]."""
+        self.last_weights.set_max_length(max_length)
+
+    # ------------------------------------------------------------------ prompt
+    def _prefill(self, q, k, v, attention_mask):
+        n_rep = q.shape[1] // k.shape[1]
+        T = k.shape[-2]
+        rows = min(T, LAST_TOKEN_NUM)
+        kr = _repeat_kv(k, n_rep)
+        w = torch.matmul(q[:, :, -rows:, :], kr.transpose(2, 3)) * self.scaling
+        if attention_mask is not None:
+            w = w + attention_mask[:, :, -rows:, :]
+            w = torch.max(w, torch.tensor(torch.finfo(w.dtype).min, dtype=w.dtype, device=w.device))
+        attn_weights = torch.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
+        attn_output = torch.nn.functional.scaled_dot_product_attention(
+            q, kr, _repeat_kv(v, n_rep), attn_mask=attention_mask, is_causal=attention_mask is None and T > 1,
+            scale=self.scaling)
+        return attn_weights, attn_output
+
+    # ------------------------------------------------------------------ one call
+    def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
+                attention_mask: Optional[torch.Tensor] = None, past_key_value: Optional[tuple] = None,
+                auxiliary_parameters: Optional[Tuple[torch.Tensor, ...]] = None):
+        """query (B,Hq,L,D), key/value (B,Hkv,L,D), rotary already applied.
+        -> (attn_output (B,Hq,L,D), attn_weights (the last <= 20 rows for a prompt), tuple, auxiliary_parameters)."""
+        L = key_states.shape[-2]
+        self.current_length += L
+        kv_seq_len = L + (past_key_value[-1] if past_key_value is not None else 0)
+        if past_key_value is not None:
+            new_K = torch.cat((past_key_value[-3], key_states), dim=2) if past_key_value[-3] is not None else key_states
+            new_V = torch.cat((past_key_value[-2], value_states), dim=2) if past_key_value[-2] is not None else value_states
+            past_key_value = past_key_value[:-3] + (new_K, new_V, kv_seq_len)
+            attn_weights, attn_output = qkv_matmul_hqe_2(query_states, past_key_value, attention_mask,
+                                                         self.head_dim, self.quant_strategy)
+        else:
+            attn_weights, attn_output = self._prefill(query_states, key_states, value_states, attention_mask)
+            past_key_value = (None,) * 39 + (key_states, value_states, kv_seq_len)
+
+        self.last_weights.update(attn_weights)
+        if self.current_length >= BLOCK:
+            residual_length = self.current_length % BLOCK
+            compress_length = self.current_length - residual_length
+            total_length = self.history_reserve_length + compress_length
+            block_num = total_length // BLOCK
+            token_importance = self.last_weights.calculate_token_importance()
+            if auxiliary_parameters is not None:
+                compress_ratio, K_bit_num, V_bit_num = auxiliary_parameters
+            else:
+                ratio_168 = torch.tensor([64 / total_length, 0], dtype=torch.float32)
+                compress_ratio = torch.cat((ratio_168, self.ratio_q, self.ratio_e))
+                compress_ratio[2:] = (1 - compress_ratio[0]) * compress_ratio[2:]
+                K_bit_num = torch.round(block_num * compress_ratio).to(torch.int)
+                K_bit_num = make_sum_equal(K_bit_num, block_num)
+                K_bit_num *= BLOCK
+                V_bit_num = K_bit_num.clone()
+            eviction_len = int(K_bit_num[-1])
+            sort_importance = token_importance[:total_length].clone()
+            # ranks the blocks AND divides sort_importance by 32 in place, as the reference does
+            K_token_idx = get_block_token_idx(BLOCK, block_num, sort_importance)
+            past_key_value = KV_cache_hqe_2(past_key_value, compress_length, self.history_reserve_length,
+                                            K_token_idx, K_bit_num, V_bit_num, sort_importance,
+                                            self.quant_strategy, self.last_weights, BLOCK, BLOCK, self.times_range)
+            self.history_reserve_length += compress_length - eviction_len
+            self.current_length -= compress_length
+            if auxiliary_parameters is None:
+                next_total_length = (self.history_reserve_length + BLOCK) // BLOCK * BLOCK
+                add_length = next_total_length - self.history_reserve_length
+                self.ratio_e = (add_length * self.ratio_e_0) / (self.history_reserve_length + add_length)
+                self.ratio_q = (1 - self.ratio_e) * self.ratio_q / self.ratio_q.sum()
+            auxiliary_parameters = (compress_ratio, K_bit_num, V_bit_num)
+        else:
+            auxiliary_parameters = None
+        self.token_num += 1
+        return attn_output, attn_weights, past_key_value, auxiliary_parameters
+
+    __call__ = forward

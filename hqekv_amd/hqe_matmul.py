@@ -24,4 +24,5 @@ def qkv_matmul_hqe_2(q: torch.Tensor, past_key_value: Tuple, attention_mask, hea
     real_len = value_length(past_key_value)
     if real_len == 0:
         raise ValueError('invalid past_key_value')
-    return decode_attention(q, past_key_value, None, real_len, zero_init=False)
+    return decode_attention(q, past_key_value, None, real_len, zero_init=False,
+                            low_uniform=quant_strategy == "uniform_group")

@@ -31,8 +31,8 @@ def cuda_bmm_fA_qB_uniform_group(group_size: int, fA: torch.Tensor, qB: torch.Te
     """
     if group_size != 32:
         raise ValueError("group_size must be 32")
-    if bits not in (2, 4, 8):
-        raise ValueError("bits must be 2, 4 or 8")
+    if bits not in (1, 2, 4, 8):
+        raise ValueError("bits must be 1, 2, 4 or 8")
     fA = _need_f16(fA, "fA")
     B, nh_q, M, K = fA.shape
     if M != 1:
@@ -67,14 +67,16 @@ cuda_bmm_fA_qB_wv_uniform_group = cuda_bmm_fA_qB_uniform_group
 def _hq_tuple(m16, m16_idx, m8, m8_idx, s8, z8, m4, m4_idx, s4, z4, m2, m2_idx, s2, z2,
               m1, m1_idx, s1, z1, new, is_k: bool) -> tuple:
     """Lay the positional arguments of the *_group_hq wrappers into the slots of a 42-tuple."""
-    if m1 is not None:
-        raise NotImplementedError("the 1-bit normal-quantile class is not built")
+    # m1/s1/z1: the uniform 1-bit class ('uniform_group'); the normal-quantile class of the other strategy
+    # would arrive here with (std, mean) in place of (scale, zero) and cannot be told apart, so callers
+    # of these wrappers own that distinction, as upstream
     t = [None] * 42
     kb, vb = _att.K_BASE, _att.V_BASE
     base = kb if is_k else vb
     t[_att.K16 if is_k else _att.V16] = m16
     t[_att.K16_IDX if is_k else _att.V16_IDX] = m16_idx
-    for b, (m, i, s, z) in zip((8, 4, 2), ((m8, m8_idx, s8, z8), (m4, m4_idx, s4, z4), (m2, m2_idx, s2, z2))):
+    for b, (m, i, s, z) in zip((8, 4, 2, 1), ((m8, m8_idx, s8, z8), (m4, m4_idx, s4, z4), (m2, m2_idx, s2, z2),
+                                              (m1, m1_idx, s1, z1))):
         t[base[b]], t[base[b] + 1], t[base[b] + 2], t[base[b] + 3] = m, i, s, z
     t[_att.NEW_K if is_k else _att.NEW_V] = new
     return tuple(t)

@@ -44,8 +44,8 @@ def __getattr__(name):
 
 
 def _check_bits(bit: int) -> int:
-    if bit not in (2, 4, 8):
-        raise ValueError(f"bit must be 2, 4 or 8 (got {bit})")
+    if bit not in (1, 2, 4, 8):
+        raise ValueError(f"bit must be 1, 2, 4 or 8 (got {bit})")
     return 32 // bit
 
 

@@ -34,15 +34,21 @@ def calculate_token_range(new_cache: Optional[torch.Tensor], token_range: Option
 
 
 def get_block_importance(block_size: int, block_num: int, importance: torch.Tensor) -> torch.Tensor:
-    """Mean importance of each block (the caller's tensor is left untouched)."""
+    """Mean importance of each block.  Like the reference (model/public_func.py:85-90) this divides
+    ``importance`` by the block length IN PLACE when it is contiguous (the reshape is then a view): the
+    decode layer relies on that side effect -- the importance it hands to the cache policy afterwards is
+    the divided one (model/llama_hqe.py:226-231)."""
     b = importance.reshape(block_num, -1)
-    return torch.sum(b / b.shape[1], dim=-1)
+    b /= b.shape[1]
+    return torch.sum(b, dim=-1)
 
 
 def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tensor) -> torch.Tensor:
-    """Token indices of the blocks ordered by descending mean importance: the block order comes from
-    ``torch.sort(descending=True)``, tokens inside a block stay in order."""
-    _, order = torch.sort(get_block_importance(block_size, block_num, importance), descending=True)
+    """Token indices of the blocks ordered by descending mean importance, tokens inside a block in order
+    (model/public_func.py:92-106, including the in-place divide of ``importance``).  The sort is stable --
+    equal block scores keep their original order -- where the reference leaves the order of ties to the
+    device sort."""
+    _, order = torch.sort(get_block_importance(block_size, block_num, importance), descending=True, stable=True)
     ar = torch.arange(block_size, dtype=order.dtype, device=order.device)
     return (order.reshape(-1, 1) * block_size + ar.reshape(1, -1)).flatten()
 

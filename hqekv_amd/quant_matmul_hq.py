@@ -36,7 +36,8 @@ def qkv_matmul(q: torch.Tensor, past_key_value: Tuple, attention_mask, head_dim:
     if head_dim != q.shape[-1]:
         raise ValueError("head_dim does not match q")
     Tall = int(past_key_value[KV_SEQ_LEN])
-    return decode_attention(q, past_key_value, attention_mask, Tall, zero_init=True)
+    return decode_attention(q, past_key_value, attention_mask, Tall, zero_init=True,
+                            low_uniform=quant_strategy == "uniform_group")
 
 
 qkv_matmul_hq = qkv_matmul

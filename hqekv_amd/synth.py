@@ -17,6 +17,7 @@ import torch
 
 OUTLIER_CHANNELS = (3, 35, 67, 99)
 CLASS_ORDER = (16, 8, 4, 2, 0)  # 0 = evicted
+CLASS_ORDER_1BIT = (16, 8, 4, 2, 1, 0)  # six fractions: with the uniform 1-bit class
 
 
 def make_qkv(B: int, Hq: int, Hkv: int, T: int, D: int, seed: int, device="cpu"):
@@ -51,7 +52,9 @@ def split_blocks(T: int, fractions: Sequence[float], seed: int, block: int = 32)
     counts = block_counts(n_blocks, fractions)
     out, start = {}, 0
     ar = torch.arange(block)
-    for bits, c in zip(CLASS_ORDER, counts):
+    order_of = CLASS_ORDER if len(fractions) == len(CLASS_ORDER) else CLASS_ORDER_1BIT
+    assert len(fractions) == len(order_of)
+    for bits, c in zip(order_of, counts):
         blocks = torch.sort(order[start:start + c])[0]
         out[bits] = (blocks[:, None] * block + ar[None, :]).reshape(-1)
         start += c
@@ -93,7 +96,7 @@ def build_cache(K: torch.Tensor, V: torch.Tensor, classes: Dict[int, torch.Tenso
         if bits == 16:
             t[0], t[1], t[2], t[3] = k.transpose(2, 3).contiguous(), p, v.contiguous(), p.clone()
         else:
-            kb = {8: 4, 4: 12, 2: 20}[bits]
+            kb = {8: 4, 4: 12, 2: 20, 1: 28}[bits]
             vb = kb + 4
             kc, ks, kz = quantize(k.transpose(2, 3).contiguous(), 32, bits)
             vc, vs, vz = quantize(v.contiguous(), 32, bits)
@@ -118,7 +121,7 @@ def algorithmic_bytes(pkv: tuple, Hq: int) -> int:
     for i, x in enumerate(pkv[:41]):
         if torch.is_tensor(x) and i not in (36, 37, 38):
             n += x.numel() * x.element_size()
-    some = next(x for x in (pkv[2], pkv[8], pkv[16], pkv[24], pkv[40]) if x is not None)
+    some = next(x for x in (pkv[2], pkv[8], pkv[16], pkv[24], pkv[32], pkv[40]) if x is not None)
     B, D = some.shape[0], (pkv[40].shape[3] if pkv[40] is not None else pkv[2].shape[3] if pkv[2] is not None else 128)
     n += 2 * B * Hq * D * 2
     return n

@@ -16,6 +16,9 @@
  *   fp16 K class    : (B,Hkv,D,T) fp16 (channel-major);  fp16 V class: (B,Hkv,T,D)
  *   residual new_K / new_V : (B,Hkv,T,D) fp16 (token-major)
  * Codes are packed LSB first: word j holds elements j*pf .. j*pf+pf-1 of the last axis.
+ * b is 8, 4, 2 or 1: the 1-bit class is the uniform one of the reference's 'uniform_group' strategy
+ * (quant/hqe_matmul.py:375-377, quant/hqe_2.py:482-484; 32 codes per word, qmax 1), which the decode
+ * layer's count repair feeds even with a zero 1-bit share (model/public_func.py:259-268, start_idx 4).
  *
  * Each entry point names the reference interface it replaces (paths relative to the
  * reference checkout).
@@ -49,7 +52,7 @@ const char *hqekv_last_error(void);
  * x is (n_outer, n_rows, L) fp16 with a contiguous last axis; groups of 32 along L.
  * Strides are in ELEMENTS of the respective array (fp16 for x/scale/zero, int32 words for
  * code), so the outputs may be windows of larger, capacity-sized cache buffers (append).
- * Requires L % 32 == 0, x 16-byte aligned rows (x strides % 8 == 0).
+ * Requires L % 32 == 0, x 16-byte aligned rows (x strides % 8 == 0), bits in {1, 2, 4, 8}.
  */
 int hqekv_quant_pack_rows(const void *x, int64_t x_outer_stride, int64_t x_row_stride,
                           void *code, int64_t code_outer_stride, int64_t code_row_stride,
@@ -117,7 +120,7 @@ int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale
  * the fp16 residual at the tail).  Evicted tokens are simply absent from every segment.
  */
 typedef struct hqekv_seg {
-  int32_t bits;          /* 16, 8, 4 or 2                                              */
+  int32_t bits;          /* 16, 8, 4, 2 or 1                                           */
   int32_t token_major;   /* K segments with bits == 16 only: 1 = (B,Hkv,T,D) residual   */
   int64_t n_tokens;      /* multiple of 32 unless bits == 16                           */
   int64_t pos_base;      /* used when idx == NULL                                      */

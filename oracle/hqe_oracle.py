@@ -32,7 +32,7 @@ from typing import List, Optional, Sequence, Tuple
 
 import torch
 
-BITS = (8, 4, 2)
+BITS = (8, 4, 2, 1)   # 1 = the uniform 1-bit class of the 'uniform_group' strategy (qmax 1, 32 codes per word)
 
 # --------------------------------------------------------------------------- pack / unpack
 
@@ -210,12 +210,14 @@ def qkv_matmul(
 
     ``round_per_class=True`` keeps the reference's ``attn_output +=`` in fp16 after every
     class; ``False`` accumulates every class in fp32 and rounds once (what a fused kernel does).
-    Only the uniform classes (16/8/4/2) are restated; a populated 1-bit class raises.
+    Under 'uniform_group' the 1-bit class is a uniform class like the others (quant/hqe_matmul.py:375-377);
+    under 'high_uniform_group_low_normal_group' it is the normal-quantile class, which is not restated:
+    a populated 1-bit class raises there.
     """
     if quant_strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
         raise ValueError("invalid quant_strategy")
     pkv = past_key_value
-    if pkv[K_BASE[1]] is not None or pkv[V_BASE[1]] is not None:
+    if quant_strategy != "uniform_group" and (pkv[K_BASE[1]] is not None or pkv[V_BASE[1]] is not None):
         raise NotImplementedError("1-bit normal-quantile class is outside the oracle")
     new_K, new_V = pkv[NEW_K], pkv[NEW_V]
     B, Hq, _, D = q.shape
@@ -452,9 +454,9 @@ def compress_cache(past_key_value: tuple, compress_length: int, history_length: 
                    V_bit_num, token_importance, *, times_range: bool = True, scalar_div: str = "recip",
                    weights_ring: Optional[torch.Tensor] = None):
     """One compression step; 6-entry bit_num = KV_cache_hqe_2, 5-entry = KV_cache_compress.
-    Returns (new 42-tuple, ring of recent attention rows after eviction or None).  1-bit shares must be 0."""
+    Returns (new 42-tuple, ring of recent attention rows after eviction or None).  The 1-bit class is the
+    uniform one of the 'uniform_group' strategy (quant/hqe_2.py:482-484)."""
     pkv = past_key_value
-    assert int(K_bit_num[4]) == 0 and int(V_bit_num[4]) == 0, "the 1-bit class is outside the oracle"
     new_K, new_V = pkv[NEW_K], pkv[NEW_V]
     res_K = new_K[:, :, compress_length:, :].clone()
     res_V = new_V[:, :, compress_length:, :].clone()
@@ -475,7 +477,7 @@ def compress_cache(past_key_value: tuple, compress_length: int, history_length: 
     t = [None] * 42
     t[K16], t[K16_IDX] = _class_from_units(k_cls[16], 16, True)
     t[V16], t[V16_IDX] = _class_from_units(v_cls[16], 16, False)
-    for b in (8, 4, 2):
+    for b in BITS:
         s = K_BASE[b]
         t[s], t[s + 1], t[s + 2], t[s + 3] = _class_from_units(k_cls[b], b, True)
         s = V_BASE[b]
@@ -515,3 +517,119 @@ def reconstruct_cache(past_key_value: tuple):
         K[:, :, T - pkv[NEW_K].shape[2]:] = pkv[NEW_K]
         V[:, :, T - pkv[NEW_V].shape[2]:] = pkv[NEW_V]
     return K, V
+
+
+# --------------------------------------------------------------------------- the layer that calls the path
+class ImportanceRing:
+    """model/public_func.py:208-257: ring of the last ``last_length`` attention rows, summed over batch and
+    heads in the rows' own dtype; importance = column sum / number of rows that saw the column."""
+
+    def __init__(self, last_length: int = 20, max_length: int = 0):
+        self.last_length, self.max_length = last_length, max_length
+        self.kv_seq_len = 0
+        self.next_line = 0
+        self.weights = None
+
+    def update(self, attn_weights: torch.Tensor) -> None:
+        if self.weights is None:
+            self.weights = torch.zeros(self.last_length, self.max_length, dtype=attn_weights.dtype)
+        if attn_weights.shape[2] > 1:
+            rows = attn_weights if attn_weights.shape[2] < self.last_length else attn_weights[:, :, -self.last_length:, :]
+            line = rows.sum(0).sum(0)
+            self.weights[:line.shape[0], :line.shape[1]] = line
+        else:
+            line = attn_weights.sum(0).sum(0)
+            self.weights[self.next_line:self.next_line + 1, :line.shape[1]] = line
+        self.kv_seq_len = line.shape[1]
+        self.next_line = (self.next_line + line.shape[0]) % self.last_length
+
+    def importance(self) -> torch.Tensor:
+        count = torch.arange(self.kv_seq_len, 0, -1, dtype=self.weights.dtype)
+        count[:-self.last_length] = self.last_length
+        return self.weights[:, :self.kv_seq_len].sum(0) / count
+
+
+class DecodeLayerOracle:
+    """The cache-side state machine of ``LlamaAttention_hqe.forward`` (model/llama_hqe.py:55-251) without
+    the projections, the rotary embedding and ``o_proj``: prefill builds ``(None,)*39 + (K, V, len)``
+    (:186), a decode step appends to ``new_K/new_V`` (:131-133) and attends over the tuple (:136), every
+    call feeds the ring (:199) and, once 32 un-quantised tokens exist, derives the class sizes (:216-224),
+    ranks blocks (:228), compresses (:230-231) and rescales the ratios for the next increment (:233-239).
+    ``observed`` lets a test feed the ring with another implementation's probabilities so that both walk
+    through identical policy decisions."""
+
+    def __init__(self, head_dim: int, bit_0: float, bit_4: float, bit_2: float, bit_1: float = 0.0,
+                 times_range: bool = True, last_length: int = 20, max_length: int = 0, scalar_div: str = "recip"):
+        self.head_dim = head_dim
+        self.times_range = times_range
+        self.scalar_div = scalar_div
+        self.ratio_e_0 = torch.tensor([bit_0], dtype=torch.float32)
+        self.ratio_e = self.ratio_e_0.clone()
+        self.ratio_q = torch.tensor([bit_4, bit_2, bit_1], dtype=torch.float32)
+        self.current_length = 0
+        self.history_reserve_length = 0
+        self.ring = ImportanceRing(last_length, max_length)
+
+    def step(self, q, k, v, attention_mask=None, past_key_value=None, auxiliary_parameters=None, observed=None):
+        """q (B,Hq,L,D), k/v (B,Hkv,L,D) after rotary.  Returns (attn_output (B,Hq,L,D) fp16,
+        attn_weights, new tuple, auxiliary_parameters)."""
+        L = k.shape[-2]
+        self.current_length += L
+        kv_seq_len = L + (past_key_value[-1] if past_key_value is not None else 0)
+        if past_key_value is not None:
+            new_K = torch.cat((past_key_value[-3], k), dim=2) if past_key_value[-3] is not None else k
+            new_V = torch.cat((past_key_value[-2], v), dim=2) if past_key_value[-2] is not None else v
+            past_key_value = past_key_value[:-3] + (new_K, new_V, kv_seq_len)
+            attn_weights, attn_output = qkv_matmul(q, past_key_value, attention_mask, self.head_dim,
+                                                   use_mask=False, scalar_div=self.scalar_div)
+        else:
+            n_rep = q.shape[1] // k.shape[1]
+            w = torch.matmul(q.float(), repeat_kv(k, n_rep).transpose(2, 3).float()).half()
+            w = (w.float() * (self.head_dim ** -0.5)).half()
+            if attention_mask is not None:
+                w = w + attention_mask
+                w = torch.max(w, torch.tensor(torch.finfo(torch.float16).min, dtype=torch.float16))
+            attn_weights = torch.softmax(w.float(), dim=-1).half()
+            attn_output = torch.matmul(attn_weights.float(), repeat_kv(v, n_rep).float()).half()
+            past_key_value = (None,) * 39 + (k, v, kv_seq_len)
+
+        self.ring.update(attn_weights if observed is None else observed)
+        if self.current_length >= 32:
+            residual = self.current_length % 32
+            compress_length = self.current_length - residual
+            total = self.history_reserve_length + compress_length
+            block_num = total // 32
+            importance = self.ring.importance()
+            if auxiliary_parameters is not None:
+                compress_ratio, K_bit_num, V_bit_num = auxiliary_parameters
+            else:
+                ratio_168 = torch.tensor([64 / total, 0], dtype=torch.float32)
+                compress_ratio = torch.cat((ratio_168, self.ratio_q, self.ratio_e))
+                compress_ratio[2:] = (1 - compress_ratio[0]) * compress_ratio[2:]
+                K_bit_num = torch.round(block_num * compress_ratio).to(torch.int)
+                K_bit_num = make_sum_equal(K_bit_num, block_num)
+                K_bit_num *= 32
+                V_bit_num = K_bit_num.clone()
+            eviction_len = int(K_bit_num[-1])
+            sort_importance = importance[:total].clone()
+            K_token_idx = get_block_token_idx(32, block_num, sort_importance)
+            # the reference's ranking divides its argument by the block length in place
+            # (model/public_func.py:94-96), so the policy below receives importance / 32
+            sort_importance = sort_importance / 32
+            past_key_value, ring = compress_cache(past_key_value, compress_length, self.history_reserve_length,
+                                                  K_token_idx, K_bit_num, V_bit_num, sort_importance,
+                                                  times_range=self.times_range, scalar_div=self.scalar_div,
+                                                  weights_ring=self.ring.weights)
+            if ring is not None:
+                self.ring.weights = ring
+            self.history_reserve_length += compress_length - eviction_len
+            self.current_length -= compress_length
+            if auxiliary_parameters is None:
+                next_total = (self.history_reserve_length + 32) // 32 * 32
+                add_length = next_total - self.history_reserve_length
+                self.ratio_e = (add_length * self.ratio_e_0) / (self.history_reserve_length + add_length)
+                self.ratio_q = (1 - self.ratio_e) * self.ratio_q / self.ratio_q.sum()
+            auxiliary_parameters = (compress_ratio, K_bit_num, V_bit_num)
+        else:
+            auxiliary_parameters = None
+        return attn_output, attn_weights, past_key_value, auxiliary_parameters

@@ -23,6 +23,7 @@ def main():
         dict(name="2bit_ramp_two_words", bit=2, codes=[(i * 7) % 4 for i in range(32)]),
         dict(name="4bit_ramp", bit=4, codes=list(range(16))),
         dict(name="8bit_top_bit", bit=8, codes=[255, 0, 128, 1, 2, 3, 4, 200]),
+        dict(name="1bit_pattern", bit=1, codes=[1, 0, 0, 1, 1, 1, 0, 0] * 3 + [0, 0, 0, 0, 0, 0, 0, 1]),
     ]
     for c in cases:
         c["words_u32"] = pack(c["codes"], c["bit"])
@@ -31,7 +32,10 @@ def main():
     codes = [0] * 6 + [1] * 10 + [2] * 10 + [3] * 6
     (HERE / "quant_arange128.json").write_text(json.dumps(
         {"scale": 10.3359375, "zeros": [0, 32, 64, 96], "codes_per_group": codes,
-         "words_u32_2bit": pack(codes * 4, 2)}, indent=1))
+         "words_u32_2bit": pack(codes * 4, 2),
+         # 1 bit: scale = 31, codes = rne(k / 31): 15/31 < 0.5 < 16/31
+         "scale_1bit": 31.0, "codes_per_group_1bit": [0] * 16 + [1] * 16,
+         "words_u32_1bit": pack(([0] * 16 + [1] * 16) * 4, 1)}, indent=1))
 
 
 if __name__ == "__main__":

@@ -8,9 +8,9 @@ B, H, D = 1, 2, 128
 
 # (new tokens this step, residual kept fp16, [fp16, 8, 4, 2, 1, evict] token counts over history+new)
 STEPS = [
-    dict(n_new=256 + 7, counts=[64, 32, 64, 64, 0, 32]),
-    dict(n_new=64 + 3, counts=[32, 32, 64, 128, 0, 32]),       # 7 carried + 64+3 new -> compress 64, residual 10
-    dict(n_new=96, counts=[32, 0, 64, 192, 0, 64]),
+    dict(n_new=256 + 7, counts=[64, 32, 64, 32, 32, 32]),
+    dict(n_new=64 + 3, counts=[32, 32, 64, 96, 32, 32]),       # 7 carried + 64+3 new -> compress 64, residual 10
+    dict(n_new=96, counts=[32, 0, 64, 128, 64, 64]),
 ]
 
 

@@ -13,7 +13,7 @@ def _close(a, b):
     torch.testing.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 @pytest.mark.parametrize("T", [32, 992, 4096])
 def test_qk_shape(dev, bit, T):
     from hqekv_amd.matmul import cuda_bmm_fA_qB_uniform_group
@@ -28,7 +28,7 @@ def test_qk_shape(dev, bit, T):
     _close(out, O.gemv_uniform_group(32, q, code, s, z, bit))
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 @pytest.mark.parametrize("T", [32, 160, 2080])
 def test_pv_shape(dev, bit, T):
     from hqekv_amd.matmul import cuda_bmm_fA_qB_uniform_group

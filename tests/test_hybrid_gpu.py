@@ -36,6 +36,9 @@ CASES = [
     dict(B=1, Hq=4, Hkv=4, T=512 + 31, D=128, fractions=(0.25, 0.0, 0.5, 0.0, 0.25), residual=31, seed=4),
     dict(B=1, Hq=16, Hkv=2, T=1024, D=128, fractions=(0.0, 1.0, 0.0, 0.0, 0.0), residual=0, seed=5),
     dict(B=3, Hq=8, Hkv=1, T=640 + 5, D=128, fractions=(0.1, 0.2, 0.3, 0.3, 0.1), residual=5, seed=6),
+    # with the uniform 1-bit class of the 'uniform_group' strategy (32 codes per word)
+    dict(B=1, Hq=8, Hkv=2, T=2048 + 9, D=128, fractions=(0.05, 0.1, 0.2, 0.25, 0.3, 0.1), residual=9, seed=7),
+    dict(B=2, Hq=4, Hkv=1, T=1024, D=128, fractions=(0.0, 0.0, 0.0, 0.0, 1.0, 0.0), residual=0, seed=8),
 ]
 
 

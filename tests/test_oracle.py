@@ -18,7 +18,7 @@ def test_pack_known_answer_lsb_first():
     w = O.pack_along_last_dim(q, 2)
     assert w.item() == -454761244 and (w.item() & 0xFFFFFFFF) == 0xE4E4E4E4
     # one code in slot i sets exactly bits [i*b, i*b+b)
-    for bit in (2, 4, 8):
+    for bit in (1, 2, 4, 8):
         pf = 32 // bit
         for i in range(pf):
             q = torch.zeros(1, 1, 1, pf, dtype=torch.int32)
@@ -26,7 +26,7 @@ def test_pack_known_answer_lsb_first():
             assert (O.pack_along_last_dim(q, bit).item() & 0xFFFFFFFF) == ((2 ** bit - 1) << (i * bit))
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_pack_unpack_round_trip_every_value_in_every_slot(bit):
     pf = 32 // bit
     vals = torch.arange(2 ** bit, dtype=torch.int32)
@@ -58,6 +58,13 @@ def test_quantise_known_answer_arange():
         assert O.unpack_codes(code, 2).flatten().tolist() == expect * 4
     g = json.loads((GOLDEN / "quant_arange128.json").read_text())
     assert [w & 0xFFFFFFFF for w in code.flatten().tolist()] == g["words_u32_2bit"]
+    # 1 bit (the uniform 1-bit class): scale = mx - mn = 31, code = [k >= 16]
+    code1, scale1, mn1 = O.uniform_group_quantize_pack_last_dim(x, 32, 1)
+    assert scale1.flatten().tolist() == [g["scale_1bit"]] * 4 and mn1.flatten().tolist() == [0.0, 32.0, 64.0, 96.0]
+    assert [w & 0xFFFFFFFF for w in code1.flatten().tolist()] == g["words_u32_1bit"] == [0xFFFF0000] * 4
+    # half of the range is a tie and goes to the even code 0
+    tie = torch.tensor([0.0, 1.0, 2.0] + [0.0] * 29, dtype=torch.float16).reshape(1, 1, 1, 32)
+    assert O.unpack_codes(O.uniform_group_quantize_pack_last_dim(tie, 32, 1)[0], 1).flatten().tolist()[:3] == [0, 0, 1]
 
 
 def test_quantise_8bit_identity_on_integers():
@@ -70,7 +77,7 @@ def test_quantise_8bit_identity_on_integers():
     assert torch.equal(O.uniform_group_dequantize_unpack_last_dim(code, scale, mn, 32, 8), x)
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_quantise_invariants(bit):
     g = torch.Generator().manual_seed(bit)
     x = (torch.randn(2, 2, 16, 128, generator=g) * 3).half()
@@ -101,7 +108,7 @@ def test_quantise_constant_group_and_scalar_division_modes():
     # the two scalar-division rules differ by at most one fp16 ulp of the scale
     g = torch.Generator().manual_seed(5)
     y = torch.randn(1, 4, 64, 256, generator=g).half()
-    for bit in (2, 4, 8):
+    for bit in (1, 2, 4, 8):
         a = O.uniform_group_quantize_pack_last_dim(y, 32, bit, "recip")[1].float()
         b = O.uniform_group_quantize_pack_last_dim(y, 32, bit, "true")[1].float()
         assert ((a - b).abs() <= b.abs() * 2.0 ** -10).all()
@@ -238,3 +245,30 @@ def test_token_range_closed_form():
     assert r.tolist() == [5.0, 0.5]
     assert O.calculate_token_range(v, r).tolist() == [5.0, 0.5, 5.0, 0.5]
     assert O.calculate_token_range(None, r) is None
+
+
+def test_layer_state_machine_bookkeeping():
+    """Prompt + decode steps through the oracle's layer: every token is in exactly one class or the
+    residual or was evicted, probabilities sum to one, class sizes follow the ratios."""
+    D, B, Hq, Hkv, T0 = 128, 1, 4, 2, 400
+    orc = O.DecodeLayerOracle(D, bit_0=0.25, bit_4=0.25, bit_2=0.5, max_length=T0 + 40)
+    g = torch.Generator().manual_seed(5)
+    pkv, evicted = None, 0
+    for step in range(41):
+        L = T0 if step == 0 else 1
+        q = torch.randn(B, Hq, L, D, generator=g).half()
+        k = torch.randn(B, Hkv, L, D, generator=g).half()
+        v = torch.randn(B, Hkv, L, D, generator=g).half()
+        mask = torch.triu(torch.full((L, L), torch.finfo(torch.float16).min, dtype=torch.float16), 1)[None, None] if step == 0 else None
+        out, w, pkv, aux = orc.step(q, k, v, mask, pkv, None)
+        assert torch.allclose(w.float().sum(-1), torch.ones(B, Hq, L), atol=2e-2)
+        if aux is not None:
+            evicted += int(aux[1][-1])
+            assert int(aux[1].sum()) % 32 == 0 and int(aux[1][0]) == 64 and int(aux[1][1]) == 0
+        kept = sum(pkv[s].shape[2] for s in (O.V16, O.V_BASE[8], O.V_BASE[4], O.V_BASE[2], O.V_BASE[1]) if pkv[s] is not None)
+        resid = 0 if pkv[O.NEW_V] is None else pkv[O.NEW_V].shape[2]
+        assert kept == orc.history_reserve_length and resid == orc.current_length
+        assert kept + resid + evicted == T0 + step == int(pkv[O.KV_SEQ_LEN])
+        idx = torch.cat([pkv[s + 1] for s in (O.V16, O.V_BASE[8], O.V_BASE[4], O.V_BASE[2], O.V_BASE[1]) if pkv[s] is not None])
+        assert torch.equal(torch.sort(idx)[0], torch.arange(kept))
+    assert evicted > 0

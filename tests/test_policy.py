@@ -82,8 +82,8 @@ def test_oracle_policy_matches_history_model():
             got = dense[:, :, 32 * p:32 * p + 32]
             assert torch.equal(got, exp), (side, p, bid, chain)
     # class membership: the number of tokens per class equals the model's count of final precisions
-    for side, slots in (("K", (0, 4, 12, 20)), ("V", (2, 8, 16, 24))):
-        for bits, s in zip((16, 8, 4, 2), slots):
+    for side, slots in (("K", (0, 4, 12, 20, 28)), ("V", (2, 8, 16, 24, 32))):
+        for bits, s in zip((16, 8, 4, 2, 1), slots):
             want = 32 * sum(1 for _, ch in model[side] if ch[-1] == bits)
             have = 0 if final[s + 1] is None else final[s + 1].numel()
             assert have == want, (side, bits, have, want)
@@ -93,7 +93,7 @@ def test_oracle_policy_invariants_every_step():
     caches, log, _ = PC.run(_oracle_compress)
     for pkv, st in zip(caches, log):
         kept = st["history"] + st["compress_length"] - st["counts"][5]
-        for slots in ((1, 5, 13, 21), (3, 9, 17, 25)):
+        for slots in ((1, 5, 13, 21, 29), (3, 9, 17, 25, 33)):
             idx = torch.cat([pkv[s] for s in slots if pkv[s] is not None])
             assert sorted(idx.tolist()) == list(range(kept)), "class positions partition the survivors"
             for s in slots:
@@ -101,7 +101,7 @@ def test_oracle_policy_invariants_every_step():
                     assert pkv[s].numel() % 32 == 0 and pkv[s].dtype == torch.int64
         assert pkv[38].numel() == kept
         # shapes of a quantised class agree with its index
-        for b, s in ((8, 4), (4, 12), (2, 20)):
+        for b, s in ((8, 4), (4, 12), (2, 20), (1, 28)):
             if pkv[s] is not None:
                 n = pkv[s + 1].numel()
                 assert pkv[s].shape == (PC.B, PC.H, PC.D, n * b // 32) and pkv[s + 2].shape == (PC.B, PC.H, PC.D, n // 32)

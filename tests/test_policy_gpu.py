@@ -87,7 +87,9 @@ def test_policy_errors(dev):
     with pytest.raises(ValueError, match="invalid quant_strategy"):
         KV_cache_hqe_2(pkv, 64, 0, ks, six, six, imp, "bogus")
     with pytest.raises(NotImplementedError):
-        KV_cache_hqe_2(pkv, 64, 0, ks, torch.tensor([32, 0, 0, 0, 32, 0], dtype=torch.int32), six, imp, "uniform_group")
+        # a populated 1-bit class under this strategy would be the normal-quantile one
+        KV_cache_hqe_2(pkv, 64, 0, ks, torch.tensor([32, 0, 0, 0, 32, 0], dtype=torch.int32), six, imp,
+                       "high_uniform_group_low_normal_group")
     with pytest.raises(ValueError):
         KV_cache_hqe_2(pkv, 48, 0, ks, six, six, imp, "uniform_group")
     with pytest.raises(ValueError):

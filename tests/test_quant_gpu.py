@@ -15,7 +15,7 @@ def _data(shape, seed, outliers=True):
     return x.half()
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_quant_rows_bit_exact(dev, bit):
     from hqekv_amd import pack_unpack as P
     x = _data((2, 3, 96, 256), 10 + bit)
@@ -27,7 +27,7 @@ def test_quant_rows_bit_exact(dev, bit):
     assert torch.equal(mn.cpu().view(torch.int16), om.view(torch.int16))
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_quant_k_transposed_view_bit_exact(dev, bit):
     """K reaches the quantiser as the transpose(2, 3) view of token-major memory (quant/hqe_2.py:32-35)."""
     from hqekv_amd import pack_unpack as P
@@ -43,7 +43,7 @@ def test_quant_k_transposed_view_bit_exact(dev, bit):
     assert torch.equal(mn.cpu().view(torch.int16), om.view(torch.int16))
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_quant_matches_torch_chain_on_device(dev, bit):
     """The reference's own torch op chain (quant/pack_unpack.py:166-175) evaluated ON THE GPU, which pins
     the tensor / python-int rule and the fp32 divide of the device against the HIP kernel."""
@@ -69,7 +69,7 @@ def test_quant_degenerate_and_extreme_groups(dev):
     x[0, 0, 1, :] = torch.linspace(-60000, 60000, 64).half()
     x[0, 0, 2, 0] = 6e-8                       # denormal range
     x[0, 0, 3, :] = torch.arange(64).half() / 1024
-    for bit in (2, 4, 8):
+    for bit in (1, 2, 4, 8):
         code, scale, mn = P.uniform_group_quantize_pack_last_dim(x.to(dev), 32, bit)
         oc, os_, om = O.uniform_group_quantize_pack_last_dim(x, 32, bit)
         assert torch.equal(code.cpu(), oc), bit
@@ -79,7 +79,7 @@ def test_quant_degenerate_and_extreme_groups(dev):
         assert torch.equal(dq.cpu()[0, 0, 0, :32], x[0, 0, 0, :32])
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_dequant_and_unpack_bit_exact(dev, bit):
     from hqekv_amd import pack_unpack as P
     x = _data((1, 2, 64, 512), 40 + bit)
@@ -93,7 +93,7 @@ def test_dequant_and_unpack_bit_exact(dev, bit):
     assert torch.equal(fq.cpu().view(torch.int16), ref.view(torch.int16))
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_pack_roundtrip(dev, bit):
     from hqekv_amd import pack_unpack as P
     g = torch.Generator().manual_seed(bit)
@@ -103,7 +103,7 @@ def test_pack_roundtrip(dev, bit):
     assert torch.equal(P.unpack_along_last_dim(code, bit).cpu().to(torch.int32), q)
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 def test_append_into_capacity_window(dev, bit):
     """Quantise new tokens straight into a window of capacity-sized cache buffers: the bytes written
     equal a stand-alone quantisation and nothing outside the window changes."""
@@ -169,7 +169,7 @@ def test_dequant_keeps_the_two_fp16_roundings(dev):
     assert out[0, 0, 0, 0].item() == 2052.0 and out[0, 0, 0, 1].item() == 2050.0
 
 
-@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
 @pytest.mark.parametrize("magnitude", [2.0 ** -21, 2.0 ** -14, 9000.0])
 def test_quant_denormal_and_near_overflow_ranges_both_layouts(dev, bit, magnitude):
     """Scales that are fp16 denormals, underflow to zero, or sit next to overflow; constant and one-hot groups."""
