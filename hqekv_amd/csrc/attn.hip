@@ -169,22 +169,33 @@ __device__ __forceinline__ void consume_words(uint32_t w0, uint32_t w1, half2_t 
 // another's arithmetic).
 constexpr int QK_TPL = 8;               // tokens per lane in every channel-major class
 constexpr int QK_TILE = 64 * QK_TPL;    // tokens per workgroup tile
-constexpr int QK_UNR = 8;               // row pairs whose loads are in flight together, per wave
+constexpr int QK_UNR = 4;               // row pairs per block; two blocks of loads are in flight per wave
 
 __host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
   return (bits == 16 && token_major) ? 64 : QK_TILE;
 }
 
+// What a lane holds of one block of QK_UNR row pairs of a quantised class (32-bit members only: a struct
+// with 16-bit members is not kept in registers).
+template <int BITS>
+struct QkBlock {
+  static constexpr int NW = BITS == 8 ? 2 : 1;  // packed words per lane per row
+  uint32_t w0[QK_UNR][NW], w1[QK_UNR][NW];
+  uint32_t s0[QK_UNR], s1[QK_UNR], z0[QK_UNR], z1[QK_UNR];  // fp16 bit patterns, zero-extended
+};
+
 // Accumulate one quantised tile: 512 tokens x D channels.  A lane owns 8 consecutive tokens: a byte of a
 // packed word at 1 bit (four lanes read the same word), half a word at 2 bits, one word at 4 bits, two
-// words at 8 bits.
-// QK_UNR row pairs at a time: every load of a block is issued before its first use, and the rolled outer
-// loop keeps the code small enough to stay in the instruction cache from one launch to the next.
-template <int BITS, int NREP, int QK_WAVES>
+// words at 8 bits.  The loads of a wave's first block are issued before the query is staged (stage_q ends
+// with the workgroup barrier), and each later block is requested while the previous one is consumed, so a
+// wave always has one block of loads in flight; the rolled loop keeps the code small enough to stay in the
+// instruction cache from one launch to the next.
+template <int BITS, int NREP, int QK_WAVES, typename StageQ>
 __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int D, int wave,
-                                                    const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
+                                                    StageQ &&stage_q, const half2_t *q2s,
+                                                    float (&acc)[NREP][QK_TPL]) {
   constexpr int PF = 32 / BITS;
-  constexpr int NW = BITS == 8 ? 2 : 1;  // packed words per lane per row
+  constexpr int NW = QkBlock<BITS>::NW;
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t wpr = n / PF;   // words per row
   const uint32_t gpr = n >> 5;   // groups per row
@@ -197,10 +208,8 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
   const rsrc_t rs = make_rsrc(sg.scale + (int64_t)bh * D * gpr, (uint32_t)D * gpr * 2u);
   const rsrc_t rz = make_rsrc(sg.zero + (int64_t)bh * D * gpr, (uint32_t)D * gpr * 2u);
   const int DP = D >> 1;
-#pragma unroll 1
-  for (int dp0 = wave; dp0 < DP; dp0 += QK_WAVES * QK_UNR) {
-    uint32_t w0[QK_UNR][NW], w1[QK_UNR][NW];
-    half_t s0[QK_UNR], s1[QK_UNR], z0[QK_UNR], z1[QK_UNR];
+
+  auto load = [&](int dp0, QkBlock<BITS> &r) {
 #pragma unroll
     for (int k = 0; k < QK_UNR; ++k) {
       const int dpk = dp0 + QK_WAVES * k;
@@ -208,15 +217,16 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
       const uint32_t crow = d * wpr * 4u, grow = d * gpr * 2u;   // scalar row offsets
 #pragma unroll
       for (int j = 0; j < NW; ++j) {
-        w0[k][j] = buf_u32(rc, wofs + 4 * j, crow);
-        w1[k][j] = buf_u32(rc, wofs + 4 * j, crow + wpr * 4u);
+        r.w0[k][j] = buf_u32(rc, wofs + 4 * j, crow);
+        r.w1[k][j] = buf_u32(rc, wofs + 4 * j, crow + wpr * 4u);
       }
-      s0[k] = buf_f16(rs, gofs, grow);
-      s1[k] = buf_f16(rs, gofs, grow + gpr * 2u);
-      z0[k] = buf_f16(rz, gofs, grow);
-      z1[k] = buf_f16(rz, gofs, grow + gpr * 2u);
+      r.s0[k] = buf_u16(rs, gofs, grow);
+      r.s1[k] = buf_u16(rs, gofs, grow + gpr * 2u);
+      r.z0[k] = buf_u16(rz, gofs, grow);
+      r.z1[k] = buf_u16(rz, gofs, grow + gpr * 2u);
     }
-    HQ_LOADS_ABOVE();
+  };
+  auto compute = [&](int dp0, const QkBlock<BITS> &r) {
 #pragma unroll
     for (int k = 0; k < QK_UNR; ++k) {
       const int dp = dp0 + QK_WAVES * k;
@@ -224,36 +234,52 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
       half2_t q2[NREP];
 #pragma unroll
       for (int h = 0; h < NREP; ++h) q2[h] = q2s[dp * NREP + h];
-      const half2_t s2 = pack_h2(s0[k], s1[k]), z2 = pack_h2(z0[k], z1[k]);
+      const half2_t s2 = half_pair<0>(r.s0[k], r.s1[k]), z2 = half_pair<0>(r.z0[k], r.z1[k]);
       if (BITS == 1) {
-        const uint32_t a0 = w0[k][0] >> sh2, a1 = w1[k][0] >> sh2;
+        const uint32_t a0 = r.w0[k][0] >> sh2, a1 = r.w1[k][0] >> sh2;
         consume_byte<1, NREP, QK_TPL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
       } else if (BITS == 2) {
-        const uint32_t a0 = w0[k][0] >> sh2, a1 = w1[k][0] >> sh2;
+        const uint32_t a0 = r.w0[k][0] >> sh2, a1 = r.w1[k][0] >> sh2;
         consume_byte<2, NREP, QK_TPL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
         consume_byte<2, NREP, QK_TPL>(byte_pair<1>(a0, a1), s2, z2, q2, acc, 4);
       } else if (BITS == 4) {
-        consume_byte<4, NREP, QK_TPL>(byte_pair<0>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 0);
-        consume_byte<4, NREP, QK_TPL>(byte_pair<1>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 2);
-        consume_byte<4, NREP, QK_TPL>(byte_pair<2>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 4);
-        consume_byte<4, NREP, QK_TPL>(byte_pair<3>(w0[k][0], w1[k][0]), s2, z2, q2, acc, 6);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<0>(r.w0[k][0], r.w1[k][0]), s2, z2, q2, acc, 0);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<1>(r.w0[k][0], r.w1[k][0]), s2, z2, q2, acc, 2);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<2>(r.w0[k][0], r.w1[k][0]), s2, z2, q2, acc, 4);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<3>(r.w0[k][0], r.w1[k][0]), s2, z2, q2, acc, 6);
       } else {
 #pragma unroll
         for (int j = 0; j < NW; ++j) {
-          consume_byte<8, NREP, QK_TPL>(byte_pair<0>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 0);
-          consume_byte<8, NREP, QK_TPL>(byte_pair<1>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 1);
-          consume_byte<8, NREP, QK_TPL>(byte_pair<2>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 2);
-          consume_byte<8, NREP, QK_TPL>(byte_pair<3>(w0[k][j], w1[k][j]), s2, z2, q2, acc, 4 * j + 3);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<0>(r.w0[k][j], r.w1[k][j]), s2, z2, q2, acc, 4 * j + 0);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<1>(r.w0[k][j], r.w1[k][j]), s2, z2, q2, acc, 4 * j + 1);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<2>(r.w0[k][j], r.w1[k][j]), s2, z2, q2, acc, 4 * j + 2);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<3>(r.w0[k][j], r.w1[k][j]), s2, z2, q2, acc, 4 * j + 3);
         }
       }
     }
+  };
+
+  // two register blocks in turn: while one is consumed the other one's loads are in flight
+  constexpr int STEP = QK_WAVES * QK_UNR;
+  QkBlock<BITS> ba, bb;
+  load(wave, ba);
+  stage_q();
+#pragma unroll 1
+  for (int dp0 = wave; dp0 < DP; dp0 += 2 * STEP) {  // every condition below is uniform
+    if (dp0 + STEP < DP) load(dp0 + STEP, bb);
+    HQ_LOADS_ABOVE();
+    compute(dp0, ba);
+    if (dp0 + 2 * STEP < DP) load(dp0 + 2 * STEP, ba);
+    HQ_LOADS_ABOVE();
+    if (dp0 + STEP < DP) compute(dp0 + STEP, bb);
   }
 }
 
 // fp16 class stored channel-major (B,Hkv,D,T): a lane owns 8 adjacent tokens of each row
-template <int NREP, int QK_WAVES>
+template <int NREP, int QK_WAVES, typename StageQ>
 __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t t0, int bh, int D, int wave,
-                                                     const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
+                                                     StageQ &&stage_q, const half2_t *q2s,
+                                                     float (&acc)[NREP][QK_TPL]) {
   const uint32_t n = (uint32_t)sg.n_tokens;
   const half_t *kp = (const half_t *)sg.data + (int64_t)bh * D * n;
   const bool vec = (n & 7) == 0 && (((uintptr_t)kp) & 15) == 0 && t0 < n;  // rows stay 16-byte aligned
@@ -271,23 +297,27 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
     }
   };
   constexpr int UNR = 2;
-#pragma unroll 1
-  for (int dp0 = wave; dp0 < DP; dp0 += QK_WAVES * UNR) {
+  struct Rows {
     uint32_t r0[UNR][4], r1[UNR][4];
+  };
+  auto load = [&](int dp0, Rows &r) {
 #pragma unroll
     for (int k = 0; k < UNR; ++k) {
-      const uint32_t d = 2u * (uint32_t)(dp0 + QK_WAVES * k);
-      load8(kp + (size_t)d * n, r0[k]);
-      load8(kp + (size_t)(d + 1) * n, r1[k]);
+      const int dpk = dp0 + QK_WAVES * k;
+      const uint32_t d = 2u * (uint32_t)(dpk < DP ? dpk : dp0);
+      load8(kp + (size_t)d * n, r.r0[k]);
+      load8(kp + (size_t)(d + 1) * n, r.r1[k]);
     }
-    HQ_LOADS_ABOVE();
+  };
+  auto compute = [&](int dp0, const Rows &r) {
 #pragma unroll
     for (int k = 0; k < UNR; ++k) {
       const int dp = dp0 + QK_WAVES * k;
+      if (dp >= DP) break;  // uniform
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const half2_t ka = half_pair<0>(r0[k][i], r1[k][i]);  // token 2i:   (k[d], k[d+1])
-        const half2_t kb = half_pair<1>(r0[k][i], r1[k][i]);  // token 2i+1
+        const half2_t ka = half_pair<0>(r.r0[k][i], r.r1[k][i]);  // token 2i:   (k[d], k[d+1])
+        const half2_t kb = half_pair<1>(r.r0[k][i], r.r1[k][i]);  // token 2i+1
 #pragma unroll
         for (int h = 0; h < NREP; ++h) {
           const half2_t q2 = q2s[dp * NREP + h];
@@ -296,6 +326,19 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
         }
       }
     }
+  };
+  constexpr int STEP = QK_WAVES * UNR;
+  Rows ba, bb;
+  load(wave, ba);
+  stage_q();
+#pragma unroll 1
+  for (int dp0 = wave; dp0 < DP; dp0 += 2 * STEP) {  // every condition below is uniform
+    if (dp0 + STEP < DP) load(dp0 + STEP, bb);
+    HQ_LOADS_ABOVE();
+    compute(dp0, ba);
+    if (dp0 + 2 * STEP < DP) load(dp0 + 2 * STEP, ba);
+    HQ_LOADS_ABOVE();
+    if (dp0 + STEP < DP) compute(dp0 + STEP, bb);
   }
 }
 
@@ -360,43 +403,64 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
   }
 }
 
+// heads reduced per pass of the cross-wave reduction: 32 KB of LDS per pass either way
+template <int NREP, int QK_WAVES>
+struct QkReduce {
+  static constexpr int RH = QK_WAVES == 4 ? (NREP < 4 ? NREP : 4) : (NREP < 2 ? NREP : 2);
+  static constexpr int VPT = RH * QK_TILE / (QK_WAVES * 64);  // values a thread sums and stores per pass
+  static constexpr int WPH = QK_WAVES / RH;                    // waves that share a head in a pass
+  static_assert(VPT >= 1 && VPT <= QK_TPL && WPH >= 1, "reduction shape");
+};
+
 // One workgroup = one tile of one class for one (b, kv head).  The class-specific code is only the
 // accumulation; the cross-wave reduction and the (scattered) store are shared by every class.
+//
 template <int NREP, int QK_WAVES>
-__global__ __launch_bounds__(QK_WAVES * 64) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
+__global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
                                                                half_t *__restrict__ scores, int Hq,
                                                                int Hkv, int D, int64_t Tall, FuseArgs fz) {
+  using R = QkReduce<NREP, QK_WAVES>;
+  constexpr int RH = R::RH, VPT = R::VPT, WPH = R::WPH;
   extern __shared__ float smem[];
-  float *red = smem;                                                        // QK_WAVES * 2 * 8 * 64 floats
-  half2_t *q2s = reinterpret_cast<half2_t *>(smem + QK_WAVES * 2 * QK_TPL * 64);  // D/2 x NREP pairs (q[d], q[d+1])
+  float *red = smem;                                                              // QK_WAVES * RH * 512 floats
+  half2_t *q2s = reinterpret_cast<half2_t *>(smem + QK_WAVES * RH * QK_TILE);      // D/2 x NREP pairs (q[d], q[d+1])
+  __shared__ float2 wave_ml[NREP][QK_WAVES];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int bh = blockIdx.x, tile = blockIdx.y;
+  const int bh = blockIdx.x;
   const int b = bh / Hkv, hkv = bh % Hkv;
+  const int tile = blockIdx.y;
   const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads, no lazy re-reads
   if (tile >= sg.n_units) return;  // uniform: grid.y is the largest tile count of any segment
   const bool tm = sg.bits == 16 && sg.token_major;
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t t0 = (uint32_t)tile * QK_TILE + lane * QK_TPL;
   const uint32_t ts = t0 < n ? t0 : 0;  // lanes past the end recompute token 0 and store nothing
-  // positions of this lane's 8 tokens: requested first (branch-free, so the loads overlap), used last
-  int64_t pos[QK_TPL];
+  // the VPT values this thread reduces and stores in every pass: head hl of the pass, tokens tok .. tok+VPT-1
+  const int hl = (int)(threadIdx.x * VPT) / QK_TILE;
+  const uint32_t tok = (uint32_t)tile * QK_TILE + (threadIdx.x * VPT) % QK_TILE;
+  // their positions: requested first (branch-free, so the loads overlap), used last.  Positions are below
+  // 2^31 (they index a row of Tall fp16 scores), so the low word of each int64 index is enough.
+  uint32_t pos[VPT];
   {
-    const int64_t *ip = sg.idx;
+    const uint32_t *ip = reinterpret_cast<const uint32_t *>(sg.idx);
     const bool has_idx = ip != nullptr;
 #pragma unroll
-    for (int i = 0; i < QK_TPL; ++i) {
-      const uint32_t t = min(ts + i, n - 1);
-      pos[i] = sg.pos_base + t;
-      if (has_idx) pos[i] = ip[t];
+    for (int i = 0; i < VPT; ++i) {
+      const uint32_t t = min(tok + i, n - 1);
+      pos[i] = (uint32_t)sg.pos_base + t;
+      if (has_idx) pos[i] = ip[2 * t];
     }
   }
   const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * D);
-  for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_WAVES * 64) {
-    const int h = k / (D >> 1), dp = k % (D >> 1);
-    q2s[dp * NREP + h] = as_h2(qsrc[k]);  // [dp][h]: one 16-byte LDS read fetches a row pair for 4 heads
-  }
-  __syncthreads();
+  auto stage_q = [&]() {
+    for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_WAVES * 64) {
+      const int h = k / (D >> 1), dp = k % (D >> 1);
+      q2s[dp * NREP + h] = as_h2(qsrc[k]);  // [dp][h]: one 16-byte LDS read fetches a row pair for 4 heads
+    }
+    __syncthreads();
+  };
   if (tm) {
+    stage_q();
     qk_f16_tm_tile<NREP, QK_WAVES>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
     return;
   }
@@ -407,66 +471,84 @@ __global__ __launch_bounds__(QK_WAVES * 64) void qk_hybrid_kernel(SegTable tb, c
 #pragma unroll
     for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {
-    case 1: qk_quant_accumulate<1, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
-    case 2: qk_quant_accumulate<2, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
-    case 4: qk_quant_accumulate<4, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
-    case 8: qk_quant_accumulate<8, NREP, QK_WAVES>(sg, ts, bh, D, wave, q2s, acc); break;
-    default: qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, q2s, acc);
+    case 1: qk_quant_accumulate<1, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
+    case 2: qk_quant_accumulate<2, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
+    case 4: qk_quant_accumulate<4, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
+    case 8: qk_quant_accumulate<8, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
+    default: qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, stage_q, q2s, acc);
   }
 
-  // cross-wave reduction, RH heads per pass (bounds LDS at QK_WAVES*RH*8*64*4 bytes): every wave parks
-  // its partials, then wave j of the pass sums head j over the waves and stores that head's row
-  constexpr int RH = NREP < 2 ? NREP : 2;
-  bool contig = (t0 + QK_TPL <= n);
+  // Cross-wave reduction, RH heads per pass.  Every wave parks its partial rows (token-contiguous, two
+  // 128-bit LDS writes per head); then ALL threads share the summation: a thread adds the QK_WAVES partials
+  // of VPT adjacent tokens of one head (one vector LDS read per partial, conflict-free), rounds, and stores
+  // them, so a wave writes 128 * VPT contiguous bytes of a score row.
+  bool contig = (tok + VPT <= n);
 #pragma unroll
-  for (int i = 1; i < QK_TPL; ++i) contig = contig && (pos[i] == pos[0] + i);
+  for (int i = 1; i < VPT; ++i) contig = contig && (pos[i] == pos[0] + i);
 #pragma unroll
   for (int h0 = 0; h0 < NREP; h0 += RH) {
     if (h0 > 0) __syncthreads();
 #pragma unroll
-    for (int j = 0; j < RH; ++j)
-#pragma unroll
-      for (int i = 0; i < QK_TPL; ++i) red[((wave * RH + j) * QK_TPL + i) * 64 + lane] = acc[h0 + j][i];
+    for (int j = 0; j < RH; ++j) {
+      float4 *dst = reinterpret_cast<float4 *>(red + (wave * RH + j) * QK_TILE + lane * QK_TPL);
+      dst[0] = make_float4(acc[h0 + j][0], acc[h0 + j][1], acc[h0 + j][2], acc[h0 + j][3]);
+      dst[1] = make_float4(acc[h0 + j][4], acc[h0 + j][5], acc[h0 + j][6], acc[h0 + j][7]);
+    }
     __syncthreads();
-    if (wave < RH) {
-      const int h = h0 + wave;
-      half_t v[QK_TPL];
-      float m_lane = -INFINITY;
+    const int h = h0 + hl;
+    float a[VPT];
 #pragma unroll
-      for (int i = 0; i < QK_TPL; ++i) {
-        float a = 0.f;
+    for (int i = 0; i < VPT; ++i) a[i] = 0.f;
 #pragma unroll
-        for (int w = 0; w < QK_WAVES; ++w) a += red[((w * RH + wave) * QK_TPL + i) * 64 + lane];
-        v[i] = (half_t)a;
-        if (fz.stats) {  // the fp16 steps of the reference epilogue: round the score, scale, round again
-          v[i] = (half_t)((float)v[i] * fz.inv_sqrt_d);
-          if (t0 + i < n) m_lane = fmaxf(m_lane, (float)v[i]);
-        }
+    for (int w = 0; w < QK_WAVES; ++w) {
+      float part[VPT];
+      __builtin_memcpy(part, red + (w * RH + hl) * QK_TILE + (threadIdx.x * VPT) % QK_TILE, VPT * 4);
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) a[i] += part[i];
+    }
+    half_t v[VPT];
+    float m_lane = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      v[i] = (half_t)a[i];
+      if (fz.stats) {  // the fp16 steps of the reference epilogue: round the score, scale, round again
+        v[i] = (half_t)((float)v[i] * fz.inv_sqrt_d);
+        if (tok + i < n) m_lane = fmaxf(m_lane, (float)v[i]);
       }
-      if (fz.stats) {
-        const float m = wave_max(m_lane);
-        float l_lane = 0.f;
+    }
+    if (fz.stats) {  // (max, sum exp) of this wave's 64 * VPT tokens; merged per head after the last pass
+      const float m = wave_max(m_lane);
+      float l_lane = 0.f;
 #pragma unroll
-        for (int i = 0; i < QK_TPL; ++i)
-          if (t0 + i < n) l_lane += __expf((float)v[i] - m);
-        const float l = wave_sum(l_lane);
-        if (lane == 0)
-          fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
-      }
-      if (t0 < n) {
-        half_t *row = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
-        // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
-        // 128-bit store per head row; otherwise 2-byte scatters through idx
-        if (contig && (((uintptr_t)(row + pos[0])) & 15) == 0) {
-          uint4 raw;
-          __builtin_memcpy(&raw, v, 16);
-          *reinterpret_cast<uint4 *>(row + pos[0]) = raw;
-        } else {
+      for (int i = 0; i < VPT; ++i)
+        if (tok + i < n) l_lane += __expf((float)v[i] - m);
+      const float l = wave_sum(l_lane);
+      if (lane == 0) wave_ml[h][wave - hl * WPH] = make_float2(m, l);
+    }
+    if (tok < n) {
+      half_t *srow = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+      // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
+      // vector store; otherwise 2-byte scatters through idx
+      if (contig && (((uintptr_t)(srow + pos[0])) & (VPT * 2 - 1)) == 0) {
+        __builtin_memcpy(__builtin_assume_aligned(srow + pos[0], VPT * 2), v, VPT * 2);
+      } else {
 #pragma unroll
-          for (int i = 0; i < QK_TPL; ++i)
-            if (t0 + i < n) row[pos[i]] = v[i];
-        }
+        for (int i = 0; i < VPT; ++i)
+          if (tok + i < n) srow[pos[i]] = v[i];
       }
+    }
+  }
+  if (fz.stats) {
+    __syncthreads();
+    if (threadIdx.x < NREP) {
+      const int h = threadIdx.x;
+      float m = -INFINITY, l = 0.f;
+#pragma unroll
+      for (int w = 0; w < WPH; ++w) m = fmaxf(m, wave_ml[h][w].x);
+#pragma unroll
+      for (int w = 0; w < WPH; ++w)
+        if (wave_ml[h][w].y > 0.f) l += wave_ml[h][w].y * __expf(wave_ml[h][w].x - m);
+      fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
     }
   }
 }
@@ -973,7 +1055,8 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
   static const char *force = getenv("HQEKV_QK_WAVES");
   const int waves = force ? atoi(force) : ((int64_t)tb.total_units * B * Hkv <= 1024 ? 8 : 4);
   dim3 grid((unsigned)(B * Hkv), (unsigned)tb.max_units, (unsigned)tb.nseg), block((unsigned)waves * 64);
-  const size_t shmem = (size_t)(nrep * D + waves * 2 * QK_TPL * 64) * sizeof(float);
+  const int rh = waves == 4 ? (nrep < 4 ? nrep : 4) : (nrep < 2 ? nrep : 2);  // QkReduce::RH
+  const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
 #define LAUNCH(N_, W_)                                                                                        \
   hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
                      (int)Hq, (int)Hkv, (int)D, Tall, fz)

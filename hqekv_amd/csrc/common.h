@@ -53,6 +53,10 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
 __device__ __forceinline__ uint32_t buf_u32(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
   return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)row_off, 0);
 }
+// a 16-bit element, zero-extended into a 32-bit register
+__device__ __forceinline__ uint32_t buf_u16(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  return (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, (int)row_off, 0);
+}
 __device__ __forceinline__ half_t buf_f16(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
   const unsigned short u = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, (int)row_off, 0);
   half_t h;
