@@ -948,34 +948,36 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
 // (quant/csrc/gemv_cuda_wv_uniform.cu:110).  One workgroup per (b, hq) row and 128 channels; CB_SLICES
 // slices of the chunk list are summed in parallel (strided, ascending within a slice, eight requests in
 // flight per thread), then the slices in order.
-constexpr int CB_SLICES = 8;
-__global__ __launch_bounds__(1024) void pv_combine_kernel(const float *__restrict__ partial,
-                                                          half_t *__restrict__ out, int n_chunks,
-                                                          int64_t n_bhq, int D) {
-  __shared__ float sh[CB_SLICES][128];
+constexpr int CB_CH = 32;      // channels per workgroup
+constexpr int CB_SLICES = 32;  // chunk slices per workgroup: slice s adds chunks s, s + 32, ...
+__global__ __launch_bounds__(CB_CH * CB_SLICES) void pv_combine_kernel(const float *__restrict__ partial,
+                                                                      half_t *__restrict__ out, int n_chunks,
+                                                                      int64_t n_bhq, int D) {
+  __shared__ float sh[CB_SLICES / 2][CB_CH];
   const int64_t r = blockIdx.x;
-  const int d = threadIdx.x % 128, sl = threadIdx.x / 128;
-  const int d0 = blockIdx.y * 128;
+  const int d = threadIdx.x % CB_CH, sl = threadIdx.x / CB_CH;  // a wave holds two slices of the 32 channels
+  const int d0 = blockIdx.y * CB_CH;
   const bool in = d0 + d < D;
   const float *src = partial + r * D + d0 + (in ? d : 0);
   const int64_t cstride = n_bhq * D;
   float v = 0.f;
-  for (int c0 = sl; c0 < n_chunks; c0 += CB_SLICES * 8) {
-    float t[8];
+  for (int c0 = sl; c0 < n_chunks; c0 += CB_SLICES * 4) {
+    float t[4];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < 4; ++k) {
       const int c = c0 + k * CB_SLICES;
       t[k] = c < n_chunks ? src[(int64_t)c * cstride] : 0.f;
     }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) v += t[k];
+    for (int k = 0; k < 4; ++k) v += t[k];
   }
-  sh[sl][d] = v;
+  v += xor_f(v, 32);  // the wave's two slices
+  if ((threadIdx.x & 63) < CB_CH) sh[threadIdx.x >> 6][d] = v;
   __syncthreads();
-  if (sl == 0 && in) {
+  if (threadIdx.x < CB_CH && in) {
     float t = sh[0][d];
 #pragma unroll
-    for (int k = 1; k < CB_SLICES; ++k) t += sh[k][d];
+    for (int k = 1; k < CB_SLICES / 2; ++k) t += sh[k][d];
     out[r * D + d0 + d] = (half_t)t;
   }
 }
@@ -1114,7 +1116,7 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
     if (rc) return rc;
   }
   if (!(stages & 2)) return HQEKV_OK;
-  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq, (unsigned)((D + 127) / 128)), dim3(128 * CB_SLICES), 0, st, partial,
+  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq, (unsigned)((D + CB_CH - 1) / CB_CH)), dim3(CB_CH * CB_SLICES), 0, st, partial,
                      (half_t *)out, (int)tb.total_units, n_bhq, (int)D);
   return check_launch("pv_combine_kernel");
 }
