@@ -205,6 +205,21 @@ def bench_quantize(args):
     exact = bool(torch.equal(b["kc"][..., off // 16:].cpu(), okc) and torch.equal(b["ks"][..., off // 32:].cpu(), oks)
                  and torch.equal(b["kz"][..., off // 32:].cpu(), okz) and torch.equal(b["vc"][:, :, off:].cpu(), ovc)
                  and torch.equal(b["vs"][:, :, off:].cpu(), ovs) and torch.equal(b["vz"][:, :, off:].cpu(), ovz))
+    # CPU baseline: the oracle's quantiser (torch CPU ops) on a bounded sample, one KV head of K and of V
+    cpu = None
+    if not args.no_cpu:
+        cores = min(16, os.cpu_count() or 1)
+        torch.set_num_threads(cores)
+        ks, vs = K0[:, :1].transpose(2, 3).contiguous(), V0[:, :1].contiguous()
+        times = []
+        for i in range(4):
+            t0 = time.perf_counter()
+            O.uniform_group_quantize_pack_last_dim(ks, 32, 2)
+            O.uniform_group_quantize_pack_last_dim(vs, 32, 2)
+            if i:
+                times.append(time.perf_counter() - t0)
+        cpu = dict(value=statistics.median(times) * 1e6 * H, unit="us", cores=cores, kind="port",
+                   sample=f"K + V of ONE of the {H} KV heads at 2 bit, time x{H}; median of 3 after 1 warm-up")
     dom = max(res[2]["k_us"], res[2]["v_us"])
     out = {"metric": "us per quantize-and-pack of 8192 new tokens (K + V, 2-bit) & GB/s", "value": res[2]["us_k_plus_v"],
            "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -215,6 +230,8 @@ def bench_quantize(args):
            "roofline": {"bound": "hbm", "kernel": "quant_k_tokenmajor_kernel<2>" if res[2]["k_us"] >= res[2]["v_us"] else "quant_rows_kernel<2>",
                         "achieved": round(res[2]["bytes_per_tensor"] / dom / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                         "frac": round(res[2]["bytes_per_tensor"] / dom / 1e3 / HBM_PEAK_GBPS, 4), "traffic": None}}
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
     print(json.dumps(out))
 
 
