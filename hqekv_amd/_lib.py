@@ -20,12 +20,15 @@ FUSE_SOFTMAX = 1
 ONLY_QK = 0x100
 ONLY_PV = 0x200
 ONLY_COMBINE = 0x400
+LAYOUT_TOKEN_MAJOR = 1   # fp16 K segment stored (B,Hkv,T,D)
+LAYOUT_NORMAL1 = 2       # 1-bit segment in normal-quantile coding (scale = std, zero = mean)
 
 # every symbol include/hqekv.h declares
 EXPORTS = (
     "hqekv_version", "hqekv_last_error",
     "hqekv_quant_pack_rows", "hqekv_quant_pack_k_tokenmajor", "hqekv_dequant_unpack_rows", "hqekv_pack_i32",
     "hqekv_selftest_quant_division",
+    "hqekv_normal1_quant_pack_rows", "hqekv_normal1_quant_pack_k_tokenmajor", "hqekv_normal1_dequant_unpack_rows",
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
     "hqekv_decode_workspace_bytes", "hqekv_decode_attn",
@@ -36,7 +39,7 @@ class Seg(C.Structure):
     """Mirror of ``struct hqekv_seg``."""
     _fields_ = [
         ("bits", C.c_int32),
-        ("token_major", C.c_int32),
+        ("layout", C.c_int32),
         ("n_tokens", C.c_int64),
         ("pos_base", C.c_int64),
         ("data", C.c_void_p),
@@ -59,6 +62,9 @@ _PROTOS = {
     "hqekv_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "hqekv_pack_i32": (C.c_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "hqekv_selftest_quant_division": (C.c_int, [_vp, _vp]),
+    "hqekv_normal1_quant_pack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "hqekv_normal1_quant_pack_k_tokenmajor": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "hqekv_normal1_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "hqekv_gemv_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64, _int]),
     "hqekv_gemv_uniform_group": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
     "hqekv_qk_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
@@ -122,7 +128,7 @@ def make_segs(items) -> "C.Array[Seg]":
     arr = (Seg * max(1, len(items)))()
     for s, it in zip(arr, items):
         s.bits = it["bits"]
-        s.token_major = int(it.get("token_major", 0))
+        s.layout = LAYOUT_TOKEN_MAJOR if it.get("token_major") else int(it.get("layout", 0))
         s.n_tokens = it["n_tokens"]
         s.pos_base = int(it.get("pos_base", 0))
         s.data = ptr(it["data"])

@@ -49,15 +49,7 @@ def _f16_k_item(k16: torch.Tensor, idx, keep: list) -> dict:
     return dict(bits=16, n_tokens=T, data=data, idx=idx, token_major=tm)
 
 
-def _check_one_bit(pkv: tuple, base: int, low_uniform: bool) -> None:
-    if pkv[base] is not None and not low_uniform:
-        raise NotImplementedError(
-            "under 'high_uniform_group_low_normal_group' the 1-bit class is the normal-quantile one, which is "
-            "not built (the uniform 1-bit class of 'uniform_group' is)")
-
-
 def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True) -> Tuple[List[dict], int, int]:
-    _check_one_bit(pkv, K_BASE[1], low_uniform)
     items = []
     nh_kv = D = None
     if pkv[K16] is not None:
@@ -73,7 +65,9 @@ def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = Tru
             nh_kv, D = code.shape[1], code.shape[2]
             idx = _idx(pkv[base + 1], n, dev)
             keep += [code, sc, zr, idx]
-            items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx))
+            # the 1-bit class holds (std, mean) and normal-quantile codes unless the strategy is 'uniform_group'
+            layout = _lib.LAYOUT_NORMAL1 if (b == 1 and not low_uniform) else 0
+            items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx, layout=layout))
     new_K = pkv[NEW_K]
     if new_K is not None and new_K.shape[2] > 0:
         nk = new_K.contiguous()
@@ -85,7 +79,6 @@ def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = Tru
 
 
 def value_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True) -> Tuple[List[dict], int, int]:
-    _check_one_bit(pkv, V_BASE[1], low_uniform)
     items = []
     nh_kv = D = None
     if pkv[V16] is not None:
@@ -103,7 +96,9 @@ def value_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = T
             nh_kv, D = code.shape[1], code.shape[3] * (32 // b)
             idx = _idx(pkv[base + 1], n, dev)
             keep += [code, sc, zr, idx]
-            items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx))
+            # the 1-bit class holds (std, mean) and normal-quantile codes unless the strategy is 'uniform_group'
+            layout = _lib.LAYOUT_NORMAL1 if (b == 1 and not low_uniform) else 0
+            items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx, layout=layout))
     new_V = pkv[NEW_V]
     if new_V is not None and new_V.shape[2] > 0:
         nv = new_V.contiguous()
@@ -218,14 +213,14 @@ class DecodePlan:
     """
 
     def __init__(self, q_like: torch.Tensor, pkv: tuple, mask=None, Tall: Optional[int] = None,
-                 flags: Optional[int] = None):
+                 flags: Optional[int] = None, low_uniform: bool = True):
         _lib.require_gpu(q_like, "q")
         B, Hq, _, D = q_like.shape
         self.dev = q_like.device
         self.Tall = int(Tall) if Tall is not None else value_length(pkv)
         self._keep: list = []
-        k_items, hk, _ = key_segments(pkv, self.dev, self.Tall, self._keep)
-        v_items, hv, _ = value_segments(pkv, self.dev, self.Tall, self._keep)
+        k_items, hk, _ = key_segments(pkv, self.dev, self.Tall, self._keep, low_uniform)
+        v_items, hv, _ = value_segments(pkv, self.dev, self.Tall, self._keep, low_uniform)
         self.Hkv = hk if hk is not None else hv
         if self.Hkv is None:
             raise ValueError("invalid past_key_value")

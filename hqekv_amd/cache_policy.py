@@ -72,11 +72,24 @@ def _none_if_empty(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     return None if x is None or x.numel() == 0 else x
 
 
+LOW_NORMAL = "high_uniform_group_low_normal_group"
+
+
+def _quantize(x: torch.Tensor, bits: int, strategy: str):
+    """8/4/2 bit: the uniform quantiser; 1 bit: uniform under 'uniform_group', normal-quantile under
+    'high_uniform_group_low_normal_group' (quant/hqe_2.py:482-492)."""
+    if bits == 1 and strategy == LOW_NORMAL:
+        return PU.normal_group_quantize_pack_last_dim(x, BLOCK, 1)
+    return PU.uniform_group_quantize_pack_last_dim(x, BLOCK, bits)
+
+
+def _dequantize(c: "_Cls", bits: int, strategy: str) -> torch.Tensor:
+    if bits == 1 and strategy == LOW_NORMAL:
+        return PU.normal_group_dequantize_unpack_last_dim(c.data, c.scale, c.zero, BLOCK, 1)
+    return PU.uniform_group_dequantize_unpack_last_dim(c.data, c.scale, c.zero, BLOCK, bits)
+
+
 def _check_low_bits(bits: int, strategy: str) -> None:
-    if bits == 1 and strategy != "uniform_group":
-        raise NotImplementedError(
-            "under 'high_uniform_group_low_normal_group' a populated 1-bit class needs the normal-quantile "
-            "quantisers, which are not built; use 'uniform_group' (uniform 1-bit class) or a zero 1-bit share")
     if strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
         raise NotImplementedError(f"quant_strategy '{strategy}' uses quantiser families that are not built")
 
@@ -108,18 +121,18 @@ def _k_split(c: _Cls, bits: int, mask: torch.Tensor):
     return part(sel, mask), part(keep, ~mask)
 
 
-def _k_to_fp16(c: _Cls, bits: int) -> torch.Tensor:
+def _k_to_fp16(c: _Cls, bits: int, strategy: str = "uniform_group") -> torch.Tensor:
     if bits == 16:
         return c.data
-    return PU.uniform_group_dequantize_unpack_last_dim(c.data, c.scale, c.zero, BLOCK, bits)
+    return _dequantize(c, bits, strategy)
 
 
-def _k_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int) -> None:
+def _k_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int, strategy: str = "uniform_group") -> None:
     """x is (B, H, D, n) fp16, possibly the transposed view of token-major memory."""
     if bits == 16:
         dst.data = _cat(dst.data, x, 3)
     else:
-        code, scale, zero = PU.uniform_group_quantize_pack_last_dim(x, BLOCK, bits)
+        code, scale, zero = _quantize(x, bits, strategy)
         dst.data, dst.scale, dst.zero = _cat(dst.data, code, 3), _cat(dst.scale, scale, 3), _cat(dst.zero, zero, 3)
     dst.idx = _cat(dst.idx, idx, 0)
 
@@ -141,17 +154,17 @@ def _v_split(c: _Cls, bits: int, mask: torch.Tensor):
     return part(sel), part(keep)
 
 
-def _v_to_fp16(c: _Cls, bits: int) -> torch.Tensor:
+def _v_to_fp16(c: _Cls, bits: int, strategy: str = "uniform_group") -> torch.Tensor:
     if bits == 16:
         return c.data
-    return PU.uniform_group_dequantize_unpack_last_dim(c.data, c.scale, c.zero, BLOCK, bits)
+    return _dequantize(c, bits, strategy)
 
 
-def _v_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int) -> None:
+def _v_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int, strategy: str = "uniform_group") -> None:
     if bits == 16:
         dst.data = _cat(dst.data, x, 2)
     else:
-        code, scale, zero = PU.uniform_group_quantize_pack_last_dim(x, BLOCK, bits)
+        code, scale, zero = _quantize(x, bits, strategy)
         dst.data, dst.scale, dst.zero = _cat(dst.data, code, 2), _cat(dst.scale, scale, 2), _cat(dst.zero, zero, 2)
     dst.idx = _cat(dst.idx, idx, 0)
 
@@ -223,7 +236,7 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
                     _check_low_bits(tgt_bits, strategy)
                 sel_idx = new_idx[m]
                 moved = take_new(m)  # (B, H, n, D)
-                append(side[tgt_bits], moved.transpose(2, 3) if is_k else moved, sel_idx, tgt_bits)
+                append(side[tgt_bits], moved.transpose(2, 3) if is_k else moved, sel_idx, tgt_bits, strategy)
         for src_bits in CLASS_BITS:
             if src_bits <= tgt_bits:
                 break
@@ -235,7 +248,7 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
                 continue
             _check_low_bits(tgt_bits, strategy)
             moved, side[src_bits] = split(c, src_bits, m)
-            append(side[tgt_bits], to16(moved, src_bits), moved.idx, tgt_bits)
+            append(side[tgt_bits], to16(moved, src_bits, strategy), moved.idx, tgt_bits, strategy)
 
     if evict is not None:
         _rerank(side)
@@ -308,7 +321,7 @@ def reconstruct(past_key_value: tuple, quant_strategy: str, block_size: int = 32
     elif v_side[16].data is not None:
         D = v_side[16].data.shape[3]
     else:
-        b = next(b for b in (8, 4, 2) if v_side[b].data is not None)
+        b = next(b for b in (8, 4, 2, 1) if v_side[b].data is not None)
         D = v_side[b].data.shape[3] * (32 // b)
     K = torch.zeros(B, H, T, D, dtype=torch.float16, device=dev)
     V = torch.zeros(B, H, T, D, dtype=torch.float16, device=dev)
@@ -316,9 +329,9 @@ def reconstruct(past_key_value: tuple, quant_strategy: str, block_size: int = 32
         if b == 1 and (k_side[b].data is not None or v_side[b].data is not None):
             _check_low_bits(1, quant_strategy)
         if k_side[b].data is not None:
-            K[:, :, k_side[b].idx, :] = _k_to_fp16(k_side[b], b).transpose(2, 3)
+            K[:, :, k_side[b].idx, :] = _k_to_fp16(k_side[b], b, quant_strategy).transpose(2, 3)
         if v_side[b].data is not None:
-            V[:, :, v_side[b].idx, :] = _v_to_fp16(v_side[b], b)
+            V[:, :, v_side[b].idx, :] = _v_to_fp16(v_side[b], b, quant_strategy)
     if new_K is not None:
         K[:, :, T - new_K.shape[2]:, :] = new_K
     if new_V is not None:

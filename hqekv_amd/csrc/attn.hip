@@ -36,7 +36,7 @@ struct SegDev {
   int64_t pos_base;
   int64_t n_tokens;
   int32_t bits;
-  int32_t token_major;
+  int32_t layout;      // HQEKV_LAYOUT_*: 1 = fp16 K stored token-major, 2 = 1-bit normal-quantile coding
   int32_t unit_begin;  // first chunk of this segment in the p.V partial buffer
   int32_t n_units;     // tiles (q.K^T) or chunks (p.V) of this segment; blockIdx.z selects the segment
 };
@@ -131,14 +131,28 @@ __device__ __forceinline__ half2_t dequant_pair(half2_t c, half2_t s2, half2_t z
   return m + z2;
 }
 
+// 1-bit normal-quantile coding (quant/pack_unpack.py:371-375): x = rnd16(rnd16(centre[c] * std) + mean)
+// with centre = -+k, k = fp16(0.6745).  rnd16(-+k * std) = -+a with a = rnd16(k * std), so with a2 formed
+// once per group the value is the single rounding of (2c - 1) * a + mean: two packed fused ops.
+#define HQ_NORMAL1_CENTER ((_Float16)0.67431640625f)  // fp16(norm.ppf(0.75))
+__device__ __forceinline__ half2_t normal1_spread(half2_t std2) {
+  return std2 * (half2_t){HQ_NORMAL1_CENTER, HQ_NORMAL1_CENTER};
+}
+__device__ __forceinline__ half2_t dequant_pair_normal1(half2_t c, half2_t a2, half2_t mean2) {
+  const half2_t t = __builtin_elementwise_fma(c, (half2_t){(_Float16)2, (_Float16)2}, (half2_t){(_Float16)-1, (_Float16)-1});
+  return __builtin_elementwise_fma(t, a2, mean2);
+}
+
 // Consume one byte pair: 8/BITS dequantised pairs, each dotted with NREP operand pairs.
-template <int BITS, int NREP, int PF>
+// NORMAL (1 bit only): s2 is the spread a2 = rnd16(k * std), z2 the mean.
+template <int BITS, int NREP, int PF, bool NORMAL = false>
 __device__ __forceinline__ void consume_byte(uint32_t u, half2_t s2, half2_t z2, const half2_t (&a2)[NREP],
                                              float (&acc)[NREP][PF], int tok0) {
   constexpr int FPB = 8 / BITS;
 #define HQ_FIELD(I_)                                                                     \
   if constexpr (I_ < FPB) {                                                                      \
-    const half2_t x2 = dequant_pair(field_pair<BITS, (I_ < FPB ? I_ : 0)>(u), s2, z2);  \
+    const half2_t c2_ = field_pair<BITS, (I_ < FPB ? I_ : 0)>(u);                        \
+    const half2_t x2 = NORMAL ? dequant_pair_normal1(c2_, s2, z2) : dequant_pair(c2_, s2, z2);  \
     _Pragma("unroll") for (int h = 0; h < NREP; ++h)                                     \
         acc[h][tok0 + I_] = __builtin_amdgcn_fdot2(x2, a2[h], acc[h][tok0 + I_], false); \
   }
@@ -190,7 +204,7 @@ struct QkBlock {
 // with the workgroup barrier), and each later block is requested while the previous one is consumed, so a
 // wave always has one block of loads in flight; the rolled loop keeps the code small enough to stay in the
 // instruction cache from one launch to the next.
-template <int BITS, int NREP, int QK_WAVES, typename StageQ>
+template <int BITS, int NREP, int QK_WAVES, bool NORMAL, typename StageQ>
 __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int D, int wave,
                                                     StageQ &&stage_q, const half2_t *q2s,
                                                     float (&acc)[NREP][QK_TPL]) {
@@ -234,10 +248,12 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
       half2_t q2[NREP];
 #pragma unroll
       for (int h = 0; h < NREP; ++h) q2[h] = q2s[dp * NREP + h];
-      const half2_t s2 = half_pair<0>(r.s0[k], r.s1[k]), z2 = half_pair<0>(r.z0[k], r.z1[k]);
+      half2_t s2 = half_pair<0>(r.s0[k], r.s1[k]);
+      const half2_t z2 = half_pair<0>(r.z0[k], r.z1[k]);
+      if (NORMAL) s2 = normal1_spread(s2);
       if (BITS == 1) {
         const uint32_t a0 = r.w0[k][0] >> sh2, a1 = r.w1[k][0] >> sh2;
-        consume_byte<1, NREP, QK_TPL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
+        consume_byte<1, NREP, QK_TPL, NORMAL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
       } else if (BITS == 2) {
         const uint32_t a0 = r.w0[k][0] >> sh2, a1 = r.w1[k][0] >> sh2;
         consume_byte<2, NREP, QK_TPL>(byte_pair<0>(a0, a1), s2, z2, q2, acc, 0);
@@ -431,7 +447,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   const int tile = blockIdx.y;
   const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads, no lazy re-reads
   if (tile >= sg.n_units) return;  // uniform: grid.y is the largest tile count of any segment
-  const bool tm = sg.bits == 16 && sg.token_major;
+  const bool tm = sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR;
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t t0 = (uint32_t)tile * QK_TILE + lane * QK_TPL;
   const uint32_t ts = t0 < n ? t0 : 0;  // lanes past the end recompute token 0 and store nothing
@@ -471,10 +487,13 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
 #pragma unroll
     for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {
-    case 1: qk_quant_accumulate<1, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
-    case 2: qk_quant_accumulate<2, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
-    case 4: qk_quant_accumulate<4, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
-    case 8: qk_quant_accumulate<8, NREP, QK_WAVES>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
+    case 1:
+      if (sg.layout == HQEKV_LAYOUT_NORMAL1) qk_quant_accumulate<1, NREP, QK_WAVES, true>(sg, ts, bh, D, wave, stage_q, q2s, acc);
+      else qk_quant_accumulate<1, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc);
+      break;
+    case 2: qk_quant_accumulate<2, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
+    case 4: qk_quant_accumulate<4, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
+    case 8: qk_quant_accumulate<8, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
     default: qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, stage_q, q2s, acc);
   }
 
@@ -765,7 +784,7 @@ __device__ __forceinline__ void pv_commit(const PvPair<NREP, NG> &pr, half_t *co
 // word at 2 bits, one word at 4 bits, two words at 8 bits, 16 bytes of fp16), 4 token pairs per wave step, so the reduction over
 // tokens needs only two butterfly steps across lanes.  Code words are requested one step-block ahead of
 // their use, and the staging requests of a block are issued before the previous block is consumed.
-template <int BITS, int NREP, int D>
+template <int BITS, int NREP, int D, bool NORMAL = false>
 __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh, int wave, int lane,
                                          half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
                                          float (&acc)[NREP][PV_CPL], bool fused, const float *sm_ml) {
@@ -844,10 +863,12 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
             }
           } else {
             const uint2 sz = st.sz[tp][g];
-            const half2_t s2 = as_h2(sz.x), z2 = as_h2(sz.y);
+            half2_t s2 = as_h2(sz.x);
+            const half2_t z2 = as_h2(sz.y);
+            if (NORMAL) s2 = normal1_spread(s2);
             if (BITS == 1) {
               const uint32_t a0 = cur.w0[k][0] >> sh2, a1 = cur.w1[k][0] >> sh2;
-              consume_byte<1, NREP, PV_CPL>(byte_pair<0>(a0, a1), s2, z2, p2, acc, 0);
+              consume_byte<1, NREP, PV_CPL, NORMAL>(byte_pair<0>(a0, a1), s2, z2, p2, acc, 0);
             } else if (BITS == 2) {
               const uint32_t a0 = cur.w0[k][0] >> sh2, a1 = cur.w1[k][0] >> sh2;
               consume_byte<2, NREP, PV_CPL>(byte_pair<0>(a0, a1), s2, z2, p2, acc, 0);
@@ -919,7 +940,10 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
 #pragma unroll
     for (int i = 0; i < PV_CPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {  // (the first barrier inside pv_chunk also publishes sm_ml)
-    case 1: pv_chunk<1, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
+    case 1:
+      if (sg.layout == HQEKV_LAYOUT_NORMAL1) pv_chunk<1, NREP, D, true>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
+      else pv_chunk<1, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
+      break;
     case 2: pv_chunk<2, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
     case 4: pv_chunk<4, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
     case 8: pv_chunk<8, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
@@ -1020,9 +1044,11 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
     d.pos_base = s.pos_base;
     d.n_tokens = s.n_tokens;
     d.bits = s.bits;
-    d.token_major = is_k ? (s.bits == 16 && s.token_major) : 0;
+    d.layout = (is_k && s.bits == 16 && s.layout == HQEKV_LAYOUT_TOKEN_MAJOR) ? HQEKV_LAYOUT_TOKEN_MAJOR
+               : (s.bits == 1 && s.layout == HQEKV_LAYOUT_NORMAL1)              ? HQEKV_LAYOUT_NORMAL1
+                                                                                : 0;
     d.unit_begin = (int32_t)units;
-    const int64_t per = is_k ? qk_tile_tokens(s.bits, d.token_major) : chunk_tokens;
+    const int64_t per = is_k ? qk_tile_tokens(s.bits, d.layout == HQEKV_LAYOUT_TOKEN_MAJOR) : chunk_tokens;
     const int64_t nu = (s.n_tokens + per - 1) / per;
     d.n_units = (int32_t)nu;
     if (nu > max_units) max_units = nu;
@@ -1209,7 +1235,7 @@ static int decode_layout(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_se
   int64_t tiles = 0;
   for (int k = 0; k < n_k; ++k)
     if (k_segs[k].n_tokens > 0) {
-      const int64_t per = qk_tile_tokens(k_segs[k].bits, k_segs[k].bits == 16 && k_segs[k].token_major);
+      const int64_t per = qk_tile_tokens(k_segs[k].bits, k_segs[k].bits == 16 && k_segs[k].layout == HQEKV_LAYOUT_TOKEN_MAJOR);
       tiles += (k_segs[k].n_tokens + per - 1) / per;
     }
   if (tiles == 0) tiles = 1;

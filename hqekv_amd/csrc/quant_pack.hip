@@ -232,6 +232,127 @@ __global__ __launch_bounds__(512) void quant_k_tokenmajor_kernel(
   }
 }
 
+// ---------------------------------------------------------------- 1-bit normal-quantile quantiser
+// quant/pack_unpack.py:218-253 with bit == 1: std, mean = torch.std_mean(group) (unbiased; fp32
+// accumulation, results rounded to fp16), v = rnd16(rnd16(x - mean) / std), code = searchsorted([0, inf], v)
+// = [v > 0].  Only the sign of v and whether it underflows to zero matter:
+//   code = (u > 0) and (u > std * 2^-25),  u = rnd16(x - mean)
+// (u / std rounds to a positive fp16 exactly when it exceeds half the smallest denormal; std == 0 gives
+// +inf -> 1, std == inf gives 0).  A NaN -- 0/0 of a constant group -- becomes code 0.
+// The statistics are a two-pass fp32 evaluation (mean = sum / 32, M2 = sum (x - mean)^2, std =
+// sqrt(M2 / 31)); torch's own accumulation order is not specified, so the last bit of std / mean can
+// differ from a given torch build in rare cases.
+struct Normal1Stats {
+  half_t mean_h, std_h;
+  float thr;  // std * 2^-25
+};
+__device__ __forceinline__ Normal1Stats normal1_finish(float sum, float m2) {
+  Normal1Stats st;
+  st.mean_h = (half_t)(sum * (1.0f / 32.0f));
+  st.std_h = (half_t)__builtin_sqrtf(m2 / 31.0f);
+  st.thr = (float)st.std_h * 0x1p-25f;
+  return st;
+}
+__device__ __forceinline__ uint32_t normal1_code(half_t u, float thr) {
+  const float uf = (float)u;
+  return (uf > 0.0f && uf > thr) ? 1u : 0u;
+}
+
+// rows: 4 lanes per 32-element group, 8 contiguous fp16 per lane (same decomposition as quant_rows_kernel)
+__global__ __launch_bounds__(256) void normal1_rows_kernel(
+    const half_t *__restrict__ x, int64_t xo, int64_t xr, uint32_t *__restrict__ code, int64_t co,
+    int64_t cr, half_t *__restrict__ stdv, half_t *__restrict__ meanv, int64_t so, int64_t sr,
+    uint32_t groups_per_row, int gpr_shift, uint32_t groups_per_slab, uint32_t blocks_per_slab) {
+  const uint32_t o = blockIdx.x / blocks_per_slab;
+  const uint32_t blk = blockIdx.x - o * blocks_per_slab;
+  const uint32_t gin = blk * 64u + (threadIdx.x >> 2);
+  const uint32_t sub = threadIdx.x & 3;
+  if (gin >= groups_per_slab) return;  // the four lanes of a group leave together
+  uint32_t r, g;
+  if (gpr_shift >= 0) {
+    r = gin >> gpr_shift;
+    g = gin & (groups_per_row - 1u);
+  } else {
+    r = gin / groups_per_row;
+    g = gin - r * groups_per_row;
+  }
+  const uint4 raw = *reinterpret_cast<const uint4 *>(x + (int64_t)o * xo + (int64_t)r * xr + g * 32u + sub * 8u);
+  half_t v[8];
+  __builtin_memcpy(v, &raw, 16);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sum += (float)v[i];
+  sum += xor_f(sum, 1);
+  sum += xor_f(sum, 2);
+  const float mean_f = sum * (1.0f / 32.0f);
+  float m2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float d = (float)v[i] - mean_f;
+    m2 += d * d;
+  }
+  m2 += xor_f(m2, 1);
+  m2 += xor_f(m2, 2);
+  const Normal1Stats st = normal1_finish(sum, m2);
+  uint32_t b8 = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) b8 |= normal1_code((half_t)((float)v[i] - (float)st.mean_h), st.thr) << i;
+  const uint32_t b16 = b8 | (xor_u(b8, 1) << 8);
+  const uint32_t other = xor_u(b16, 2);
+  if (sub == 0) {
+    code[(int64_t)o * co + (int64_t)r * cr + g] = b16 | (other << 16);
+    stdv[(int64_t)o * so + (int64_t)r * sr + g] = st.std_h;
+    meanv[(int64_t)o * so + (int64_t)r * sr + g] = st.mean_h;
+  }
+}
+
+// K handed over token-major: same decomposition as quant_k_tokenmajor_kernel (a lane owns two channels of
+// one 32-token group)
+__global__ __launch_bounds__(512) void normal1_k_tokenmajor_kernel(
+    const half_t *__restrict__ x, int64_t xo, int64_t xt, uint32_t *__restrict__ code, int64_t co,
+    int64_t cr, half_t *__restrict__ stdv, half_t *__restrict__ meanv, int64_t so, int64_t sr,
+    uint32_t D, uint32_t n_groups) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t cp = lane & 7u, tg = lane >> 3;
+  const uint32_t G0 = blockIdx.x * QK_GROUPS_PER_BLOCK;
+  const uint32_t G = G0 + tg;
+  const int64_t o = blockIdx.y;
+  const uint32_t row_b = (uint32_t)xt * 2u;
+  const uint32_t groups_here = min((uint32_t)QK_GROUPS_PER_BLOCK, n_groups - G0);
+  const rsrc_t rx = make_rsrc(x + o * xo + (int64_t)G0 * 32 * xt, (groups_here * 32u - 1u) * row_b + D * 2u);
+  for (uint32_t c0 = wv * 16u; c0 < D; c0 += 128u) {
+    const uint32_t c = c0 + cp * 2u;
+    const bool live = (G < n_groups) && (c < D);
+    const uint32_t voff = live ? tg * 32u * row_b + c * 2u : 0u;
+    half2_t t[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) t[k] = bits_h2(buf_u32(rx, voff, (uint32_t)k * row_b));
+#pragma unroll
+    for (int ch = 0; ch < 2; ++ch) {
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < 32; ++k) sum += (float)t[k][ch];
+      const float mean_f = sum * (1.0f / 32.0f);
+      float m2 = 0.f;
+#pragma unroll
+      for (int k = 0; k < 32; ++k) {
+        const float d = (float)t[k][ch] - mean_f;
+        m2 += d * d;
+      }
+      const Normal1Stats st = normal1_finish(sum, m2);
+      uint32_t w = 0;
+#pragma unroll
+      for (int k = 0; k < 32; ++k) w |= normal1_code((half_t)((float)t[k][ch] - (float)st.mean_h), st.thr) << k;
+      if (live) {
+        code[o * co + (int64_t)(c + ch) * cr + G] = w;
+        stdv[o * so + (int64_t)(c + ch) * sr + G] = st.std_h;
+        meanv[o * so + (int64_t)(c + ch) * sr + G] = st.mean_h;
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- exhaustive check of the division
 // Every pair of fp16 bit patterns (u, s): v' = rnd16(f32(u) * group_recip(f32(s))) against the correctly
 // rounded v = rnd16(f32(u) / f32(s)), and the 8-bit codes rne(clamp(., 0, 255)) of both (the 4- and 2-bit
@@ -287,7 +408,8 @@ __global__ __launch_bounds__(256) void selftest_division_kernel(unsigned long lo
 
 // ---------------------------------------------------------------- unpack (+ dequantise)
 // One packed word per thread.  out = rnd16(rnd16(c * scale) + zero) (quant/pack_unpack.py:331-332).
-template <int BITS, bool DEQUANT>
+// NORMAL (1 bit): out = rnd16(rnd16(+-k * std) + mean), k = fp16(0.6745) (quant/pack_unpack.py:371-375).
+template <int BITS, bool DEQUANT, bool NORMAL = false>
 __global__ __launch_bounds__(256) void dequant_rows_kernel(
     const uint32_t *__restrict__ code, int64_t co, int64_t cr, const half_t *__restrict__ scale,
     const half_t *__restrict__ zero, int64_t so, int64_t sr, half_t *__restrict__ out, int64_t oo,
@@ -310,7 +432,10 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(
 #pragma unroll
   for (int i = 0; i < PF; ++i) {
     const float c = (float)code_at<BITS>(w, i);
-    if (DEQUANT) {
+    if (NORMAL) {
+      const half_t m = (half_t)((c != 0.f ? 0.67431640625f : -0.67431640625f) * s);
+      vals[i] = (half_t)((float)m + z);
+    } else if (DEQUANT) {
       const half_t m = (half_t)(c * s);  // exact product, one rounding
       vals[i] = (half_t)((float)m + z);  // second rounding
     } else {
@@ -400,6 +525,68 @@ extern "C" int hqekv_quant_pack_k_tokenmajor(const void *x, int64_t xo, int64_t 
   if (bits == 1) LAUNCH(1); else if (bits == 2) LAUNCH(2); else if (bits == 4) LAUNCH(4); else LAUNCH(8);
 #undef LAUNCH
   return check_launch("quant_k_tokenmajor_kernel");
+}
+
+extern "C" int hqekv_normal1_quant_pack_rows(const void *x, int64_t xo, int64_t xr, void *code, int64_t co,
+                                             int64_t cr, void *stdv, void *meanv, int64_t so, int64_t sr,
+                                             int64_t n_outer, int64_t n_rows, int64_t L, void *stream) {
+  if (n_outer < 0 || n_rows < 0 || L < 0 || L % 32 != 0)
+    return fail(HQEKV_E_ARG, "normal1_quant_pack_rows: L=%lld must be a non-negative multiple of 32", (long long)L);
+  const int64_t n_groups = n_outer * n_rows * (L / 32);
+  if (n_groups == 0) return HQEKV_OK;
+  if (!x || !code || !stdv || !meanv) return fail(HQEKV_E_ARG, "normal1_quant_pack_rows: null pointer");
+  if (((uintptr_t)x & 15) || (xo % 8) || (xr % 8))
+    return fail(HQEKV_E_ALIGN, "normal1_quant_pack_rows: x rows must be 16-byte aligned");
+  const int64_t gpr = L / 32, gps = n_rows * gpr;
+  const int64_t bps = (gps + 63) / 64;
+  if (gps > 0x7fffffffLL || bps * n_outer > 0x7fffffffLL)
+    return fail(HQEKV_E_ARG, "normal1_quant_pack_rows: too many groups");
+  int shift = -1;
+  if ((gpr & (gpr - 1)) == 0) for (shift = 0; (1LL << shift) < gpr; ++shift) {}
+  hipLaunchKernelGGL(normal1_rows_kernel, dim3((unsigned)(bps * n_outer)), dim3(256), 0, (hipStream_t)stream,
+                     (const half_t *)x, xo, xr, (uint32_t *)code, co, cr, (half_t *)stdv, (half_t *)meanv, so, sr,
+                     (uint32_t)gpr, shift, (uint32_t)gps, (uint32_t)bps);
+  return check_launch("normal1_rows_kernel");
+}
+
+extern "C" int hqekv_normal1_quant_pack_k_tokenmajor(const void *x, int64_t xo, int64_t xt, void *code,
+                                                     int64_t co, int64_t cr, void *stdv, void *meanv,
+                                                     int64_t so, int64_t sr, int64_t n_outer, int64_t T,
+                                                     int64_t D, void *stream) {
+  if (n_outer < 0 || T < 0 || T % 32 != 0 || D <= 0 || D % 2 != 0)
+    return fail(HQEKV_E_ARG, "normal1_quant_pack_k_tokenmajor: need T %% 32 == 0 and even D (T=%lld D=%lld)",
+                (long long)T, (long long)D);
+  if (n_outer == 0 || T == 0) return HQEKV_OK;
+  if (!x || !code || !stdv || !meanv) return fail(HQEKV_E_ARG, "normal1_quant_pack_k_tokenmajor: null pointer");
+  if (((uintptr_t)x & 3) || (xo % 2) || (xt % 2))
+    return fail(HQEKV_E_ALIGN, "normal1_quant_pack_k_tokenmajor: x rows must be 4-byte aligned");
+  if (n_outer > 65535) return fail(HQEKV_E_ARG, "normal1_quant_pack_k_tokenmajor: n_outer > 65535");
+  if (xt < D || xt > (1LL << 22) || D > (1LL << 22) || T / 32 > 0x7fffffffLL)
+    return fail(HQEKV_E_ARG, "normal1_quant_pack_k_tokenmajor: need D <= xt <= 2^22 (xt=%lld D=%lld)", (long long)xt, (long long)D);
+  const int64_t n_groups = T / 32;
+  dim3 grid((unsigned)((n_groups + QK_GROUPS_PER_BLOCK - 1) / QK_GROUPS_PER_BLOCK), (unsigned)n_outer);
+  hipLaunchKernelGGL(normal1_k_tokenmajor_kernel, grid, dim3(512), 0, (hipStream_t)stream, (const half_t *)x, xo, xt,
+                     (uint32_t *)code, co, cr, (half_t *)stdv, (half_t *)meanv, so, sr, (uint32_t)D, (uint32_t)n_groups);
+  return check_launch("normal1_k_tokenmajor_kernel");
+}
+
+extern "C" int hqekv_normal1_dequant_unpack_rows(const void *code, int64_t co, int64_t cr, const void *stdv,
+                                                 const void *meanv, int64_t so, int64_t sr, void *out,
+                                                 int64_t oo, int64_t orow, int64_t n_outer, int64_t n_rows,
+                                                 int64_t L, void *stream) {
+  if (n_outer < 0 || n_rows < 0 || L < 0 || L % 32 != 0)
+    return fail(HQEKV_E_ARG, "normal1_dequant_unpack_rows: bad L=%lld", (long long)L);
+  const int64_t n_words = n_outer * n_rows * (L / 32);
+  if (n_words == 0) return HQEKV_OK;
+  if (!code || !out || !stdv || !meanv) return fail(HQEKV_E_ARG, "normal1_dequant_unpack_rows: null pointer");
+  if (((uintptr_t)out & 7) || (oo % 4) || (orow % 4))
+    return fail(HQEKV_E_ALIGN, "normal1_dequant_unpack_rows: out rows must be 8-byte aligned");
+  const int64_t blocks = (n_words + 255) / 256;
+  if (blocks > 0x7fffffffLL) return fail(HQEKV_E_ARG, "normal1_dequant_unpack_rows: too many words");
+  hipLaunchKernelGGL((dequant_rows_kernel<1, true, true>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const uint32_t *)code, co, cr, (const half_t *)stdv, (const half_t *)meanv, so, sr,
+                     (half_t *)out, oo, orow, n_rows, L / 32, n_words);
+  return check_launch("dequant_rows_kernel");
 }
 
 extern "C" int hqekv_selftest_quant_division(void *counts, void *stream) {

@@ -67,9 +67,8 @@ cuda_bmm_fA_qB_wv_uniform_group = cuda_bmm_fA_qB_uniform_group
 def _hq_tuple(m16, m16_idx, m8, m8_idx, s8, z8, m4, m4_idx, s4, z4, m2, m2_idx, s2, z2,
               m1, m1_idx, s1, z1, new, is_k: bool) -> tuple:
     """Lay the positional arguments of the *_group_hq wrappers into the slots of a 42-tuple."""
-    # m1/s1/z1: the uniform 1-bit class ('uniform_group'); the normal-quantile class of the other strategy
-    # would arrive here with (std, mean) in place of (scale, zero) and cannot be told apart, so callers
-    # of these wrappers own that distinction, as upstream
+    # m1/s1/z1: upstream's fused wrappers take the 1-bit class as (codes, std_1, means_1), the normal-quantile
+    # coding (quant/matmul.py:351-373); the segments are built with that layout by the callers below
     t = [None] * 42
     kb, vb = _att.K_BASE, _att.V_BASE
     base = kb if is_k else vb
@@ -112,7 +111,7 @@ def cuda_bmm_forward_qk_group_hq(group_size, nh_kv, in_vector, matrix_16, matrix
                     matrix_1, matrix_1_idx, std_1, means_1, new_K, True)
     dev = in_vector.device
     keep: list = []
-    items, hk, dk = _att.key_segments(pkv, dev, Tall, keep)
+    items, hk, dk = _att.key_segments(pkv, dev, Tall, keep, low_uniform=False)  # (std_1, means_1): normal-quantile class
     if hk != nh_kv or dk != D:
         raise ValueError("cache shape does not match nh_kv / head_dim")
     out = torch.zeros(B, nh_q, 1, Tall, dtype=torch.float16, device=dev)
@@ -142,7 +141,7 @@ def cuda_bmm_forward_wv_group_hq(group_size, nh_kv, in_vector, matrix_16, matrix
                     matrix_1, matrix_1_idx, std_1, means_1, new_V, False)
     dev = in_vector.device
     keep: list = []
-    items, hv, D = _att.value_segments(pkv, dev, Tall, keep)
+    items, hv, D = _att.value_segments(pkv, dev, Tall, keep, low_uniform=False)
     if not items:
         raise ValueError('invalid matrix.')
     if hv != nh_kv:

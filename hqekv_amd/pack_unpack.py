@@ -24,7 +24,7 @@ _QUANTILES = {}
 
 
 def _normal_tables():
-    # quant/pack_unpack.py:6-14 -- kept for importers; the 1-bit normal class itself is not built
+    # quant/pack_unpack.py:6-14 -- kept for importers; the kernels hold the 1-bit entries as constants
     if not _QUANTILES:
         from scipy.stats import norm
         ub = {n: torch.tensor(norm.ppf(torch.arange(0, 1, 1 / (2 ** n)) + 1 / (2 ** n)), dtype=torch.float32)
@@ -186,6 +186,77 @@ def uniform_group_fake_quant(data: torch.Tensor, group_size: int, bit: int):
     return uniform_group_dequantize_unpack_last_dim(code, scale, mn, group_size, bit)
 
 
+def normal_group_quantize_pack_last_dim(data: torch.Tensor, group_size: int, bit: int):
+    """The 1-bit normal-quantile quantiser (quant/pack_unpack.py:218-253 with bit == 1):
+    -> ``(code (B,nh,D,T/32) int32, std (B,nh,D,T/32) fp16, mean (B,nh,D,T/32) fp16)``, code = [x > mean] after
+    the reference's fp16 steps.  Other bit widths of the normal family are not built."""
+    _check_group(group_size)
+    if bit != 1:
+        raise NotImplementedError("only the 1-bit table of the normal-quantile family is on the decode path")
+    _lib.require_gpu(data, "data")
+    if data.dtype != torch.float16:
+        raise TypeError("data must be float16")
+    B, nh, R, L = data.shape
+    if L % GROUP:
+        raise ValueError("last dim must be a multiple of 32")
+    dev = data.device
+    code = torch.empty(B, nh, R, L // 32, dtype=torch.int32, device=dev)
+    std = torch.empty(B, nh, R, L // GROUP, dtype=torch.float16, device=dev)
+    mean = torch.empty_like(std)
+    if data.numel() == 0:
+        return code, std, mean
+    lib = _lib.load()
+    st = _lib.stream_ptr(dev)
+    with torch.cuda.device(dev):
+        tm = (data.stride(2) == 1 and data.stride(3) == R and data.stride(1) == R * L
+              and data.stride(0) == nh * R * L and R % 2 == 0 and R > 1)
+        if tm:   # the transposed view of token-major K, read in place
+            _lib.check(lib.hqekv_normal1_quant_pack_k_tokenmajor(
+                data.data_ptr(), R * L, R, code.data_ptr(), code.stride(1), code.stride(2),
+                std.data_ptr(), mean.data_ptr(), std.stride(1), std.stride(2), B * nh, L, R, st),
+                "normal_group_quantize_pack_last_dim")
+        else:
+            if not data.is_contiguous():
+                data = data.contiguous()
+            _lib.check(lib.hqekv_normal1_quant_pack_rows(
+                data.data_ptr(), R * L, L, code.data_ptr(), code.stride(1), code.stride(2),
+                std.data_ptr(), mean.data_ptr(), std.stride(1), std.stride(2), B * nh, R, L, st),
+                "normal_group_quantize_pack_last_dim")
+    return code, std, mean
+
+
+def normal_group_dequantize_unpack_last_dim(code: torch.Tensor, std: torch.Tensor, mean: torch.Tensor,
+                                            group_size: int, bit: int) -> torch.Tensor:
+    """fp16 ``rnd16(rnd16(+-fp16(0.6745) * std) + mean)`` of shape (B, nh, D, T) (quant/pack_unpack.py:356-376,
+    bit == 1)."""
+    _check_group(group_size)
+    if bit != 1:
+        raise NotImplementedError("only the 1-bit table of the normal-quantile family is on the decode path")
+    _lib.require_gpu(code, "code")
+    B, nh, D, Td = code.shape
+    T = Td * 32
+    if code.dtype != torch.int32 or std.dtype != torch.float16 or mean.dtype != torch.float16:
+        raise TypeError("code must be int32, std/mean float16")
+    if tuple(std.shape) != (B, nh, D, T // GROUP) or tuple(mean.shape) != tuple(std.shape):
+        raise ValueError("std/mean shapes do not match the codes")
+    code, std, mean = code.contiguous(), std.contiguous(), mean.contiguous()
+    out = torch.empty(B, nh, D, T, dtype=torch.float16, device=code.device)
+    with torch.cuda.device(code.device):
+        _lib.check(_lib.load().hqekv_normal1_dequant_unpack_rows(
+            code.data_ptr(), 0, Td, std.data_ptr(), mean.data_ptr(), 0, T // GROUP,
+            out.data_ptr(), 0, T, 1, B * nh * D, T, _lib.stream_ptr(code.device)),
+            "normal_group_dequantize_unpack_last_dim")
+    return out
+
+
+def normal_group_fake_quant(data: torch.Tensor, group_size: int, bit: int):
+    """quant/pack_unpack.py:195-216 for bit == 1 (``bit == 0`` returns 0)."""
+    if bit == 0:
+        return 0
+    code, std, mean = normal_group_quantize_pack_last_dim(data, group_size, bit)
+    return normal_group_dequantize_unpack_last_dim(code, std, mean, group_size, bit)
+
+
 def _not_built(name):
     def f(*a, **k):
         raise NotImplementedError(
@@ -199,6 +270,3 @@ uniform_quantize_pack_last_dim = _not_built("uniform_quantize_pack_last_dim")
 uniform_dequantize_unpack_last_dim = _not_built("uniform_dequantize_unpack_last_dim")
 normal_quantize_pack_last_dim = _not_built("normal_quantize_pack_last_dim")
 normal_dequantize_unpack_last_dim = _not_built("normal_dequantize_unpack_last_dim")
-normal_group_quantize_pack_last_dim = _not_built("normal_group_quantize_pack_last_dim")
-normal_group_dequantize_unpack_last_dim = _not_built("normal_group_dequantize_unpack_last_dim")
-normal_group_fake_quant = _not_built("normal_group_fake_quant")

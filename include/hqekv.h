@@ -80,6 +80,28 @@ int hqekv_dequant_unpack_rows(const void *code, int64_t code_outer_stride, int64
                               int64_t out_row_stride, int64_t n_outer, int64_t n_rows, int64_t L,
                               int bits, void *stream);
 
+/* The 1-bit normal-quantile class of the 'high_uniform_group_low_normal_group' strategy: replaces
+ * normal_group_quantize_pack_last_dim / normal_group_dequantize_unpack_last_dim with bit == 1
+ * (quant/pack_unpack.py:218-253, 356-376; 2-entry tables of :6-14: bounds [0, inf], centres -+0.6745).
+ * Same shapes, strides and alignment rules as the uniform entry points above, 32 codes per word;
+ * `stdv` / `meanv` take the places of scale / zero (unbiased std and mean of each group, fp16).
+ * code = [rnd16(rnd16(x - mean) / std) > 0]; dequantised x = rnd16(rnd16(+-fp16(0.6745) * std) + mean).
+ */
+int hqekv_normal1_quant_pack_rows(const void *x, int64_t x_outer_stride, int64_t x_row_stride,
+                                  void *code, int64_t code_outer_stride, int64_t code_row_stride,
+                                  void *stdv, void *meanv, int64_t sz_outer_stride, int64_t sz_row_stride,
+                                  int64_t n_outer, int64_t n_rows, int64_t L, void *stream);
+int hqekv_normal1_quant_pack_k_tokenmajor(const void *x, int64_t x_outer_stride, int64_t x_token_stride,
+                                          void *code, int64_t code_outer_stride, int64_t code_row_stride,
+                                          void *stdv, void *meanv, int64_t sz_outer_stride,
+                                          int64_t sz_row_stride, int64_t n_outer, int64_t T, int64_t D,
+                                          void *stream);
+int hqekv_normal1_dequant_unpack_rows(const void *code, int64_t code_outer_stride, int64_t code_row_stride,
+                                      const void *stdv, const void *meanv, int64_t sz_outer_stride,
+                                      int64_t sz_row_stride, void *out, int64_t out_outer_stride,
+                                      int64_t out_row_stride, int64_t n_outer, int64_t n_rows, int64_t L,
+                                      void *stream);
+
 /* No counterpart in the reference: a device-side proof obligation of the quantiser above.  The kernels
  * evaluate the reference's v = u / scale (quant/pack_unpack.py:173, fp16 operands, fp32 divide, fp16
  * result) as u * (1/scale); this call compares the two over all 2^32 pairs of fp16 bit patterns.
@@ -119,9 +141,14 @@ int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale
  * quant/csrc/gemv_cuda_uniform.cu:945); idx == NULL means position = pos_base + j (used for
  * the fp16 residual at the tail).  Evicted tokens are simply absent from every segment.
  */
+#define HQEKV_LAYOUT_TOKEN_MAJOR 1 /* K segment with bits == 16 stored (B,Hkv,T,D): the residual new_K   */
+#define HQEKV_LAYOUT_NORMAL1 2     /* bits == 1 only: normal-quantile coding, scale = std, zero = mean:  */
+                                   /* x = rnd16(rnd16(+-0.6745 * std) + mean), the 1-bit class of the   */
+                                   /* 'high_uniform_group_low_normal_group' strategy                    */
+                                   /* (quant/pack_unpack.py:356-376, quant/hqe_matmul.py:371-374)       */
 typedef struct hqekv_seg {
   int32_t bits;          /* 16, 8, 4, 2 or 1                                           */
-  int32_t token_major;   /* K segments with bits == 16 only: 1 = (B,Hkv,T,D) residual   */
+  int32_t layout;        /* HQEKV_LAYOUT_*: 0 = as listed at the top of this file       */
   int64_t n_tokens;      /* multiple of 32 unless bits == 16                           */
   int64_t pos_base;      /* used when idx == NULL                                      */
   const void *data;      /* codes (int32) or fp16 values                               */

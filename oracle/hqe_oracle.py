@@ -130,6 +130,42 @@ def uniform_group_dequantize_unpack_last_dim(
     return x.reshape(B, nh, D, T)
 
 
+# --------------------------------------------------------------------------- 1-bit normal-quantile class
+# quant/pack_unpack.py:6-14 for n = 1: upper bounds norm.ppf([0.5, 1.0]) = [0, inf], centres
+# norm.ppf([0.25, 0.75]) = -+0.6744897501960817 (fp32), used in the group's dtype: fp16 0.67431640625.
+NORMAL1_CENTER = 0.6744897501960817
+
+
+def normal_group_quantize_pack_last_dim(data: torch.Tensor, group_size: int, bit: int = 1):
+    """quant/pack_unpack.py:218-253 for bit == 1: ``std, mean = torch.std_mean(group)`` (unbiased, fp32
+    accumulation, rounded to fp16), ``v = rnd16(rnd16(x - mean) / std)``, code = searchsorted([0, inf], v)
+    = [v > 0]; packed 32 codes per word.  A NaN (0/0 of a constant group) is stored as code 0 (the reference
+    would index past its 2-entry tables)."""
+    assert bit == 1, "only the 1-bit table is on the path"
+    B, nh, D, T = data.shape
+    assert data.dtype == torch.float16 and T % group_size == 0
+    g = data.reshape(B * nh * D, T // group_size, group_size)
+    std, mean = torch.std_mean(g, dim=-1, keepdim=True)
+    v = (g - mean) / std
+    q = (v > 0).to(torch.int32).reshape(B, nh, D, T)
+    shp = (B, nh, D, T // group_size)
+    return pack_along_last_dim(q, 1), std.reshape(shp), mean.reshape(shp)
+
+
+def normal_group_dequantize_unpack_last_dim(code, std, mean, group_size: int, bit: int = 1):
+    """quant/pack_unpack.py:356-376 for bit == 1: x = rnd16(rnd16(centre[c] * std) + mean), the centre in
+    the group's dtype."""
+    assert bit == 1
+    B, nh, D, Td = code.shape
+    T = Td * 32
+    c = unpack_codes(code, 1).reshape(B, nh, D, T // group_size, group_size).to(torch.int64)
+    center = torch.tensor([-NORMAL1_CENTER, NORMAL1_CENTER], dtype=torch.float32)
+    x = center[c].to(std.dtype)
+    x = x * std.unsqueeze(-1)
+    x = x + mean.unsqueeze(-1)
+    return x.reshape(B, nh, D, T)
+
+
 def uniform_group_fake_quant(data: torch.Tensor, group_size: int, bit: int, scalar_div: str = "recip"):
     """quant/pack_unpack.py:134-154 (quantise then dequantise without packing)."""
     if bit == 0:
@@ -150,6 +186,23 @@ def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
         return x
     B, H, a, b = x.shape
     return x[:, :, None].expand(B, H, n_rep, a, b).reshape(B, H * n_rep, a, b)
+
+
+LOW_NORMAL_STRATEGY = "high_uniform_group_low_normal_group"
+
+
+def class_quantize(x, bits: int, scalar_div: str = "recip", low_normal: bool = False):
+    """The quantiser a class uses: uniform for 8/4/2 bit; for 1 bit uniform under 'uniform_group' and
+    normal-quantile under 'high_uniform_group_low_normal_group' (quant/hqe_2.py:482-492)."""
+    if bits == 1 and low_normal:
+        return normal_group_quantize_pack_last_dim(x, 32, 1)
+    return uniform_group_quantize_pack_last_dim(x, 32, bits, scalar_div)
+
+
+def class_dequantize(code, s, z, bits: int, low_normal: bool = False):
+    if bits == 1 and low_normal:
+        return normal_group_dequantize_unpack_last_dim(code, s, z, 32, 1)
+    return uniform_group_dequantize_unpack_last_dim(code, s, z, 32, bits)
 
 
 def gemv_uniform_group(group_size, fA, qB, scales, zeros, bits) -> torch.Tensor:
@@ -211,14 +264,12 @@ def qkv_matmul(
     ``round_per_class=True`` keeps the reference's ``attn_output +=`` in fp16 after every
     class; ``False`` accumulates every class in fp32 and rounds once (what a fused kernel does).
     Under 'uniform_group' the 1-bit class is a uniform class like the others (quant/hqe_matmul.py:375-377);
-    under 'high_uniform_group_low_normal_group' it is the normal-quantile class, which is not restated:
-    a populated 1-bit class raises there.
+    under 'high_uniform_group_low_normal_group' it is the normal-quantile class (:371-374).
     """
     if quant_strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
         raise ValueError("invalid quant_strategy")
     pkv = past_key_value
-    if quant_strategy != "uniform_group" and (pkv[K_BASE[1]] is not None or pkv[V_BASE[1]] is not None):
-        raise NotImplementedError("1-bit normal-quantile class is outside the oracle")
+    low_normal = quant_strategy == LOW_NORMAL_STRATEGY
     new_K, new_V = pkv[NEW_K], pkv[NEW_V]
     B, Hq, _, D = q.shape
     real_len = 0
@@ -245,7 +296,8 @@ def qkv_matmul(
     for b in BITS:
         base = K_BASE[b]
         if pkv[base] is not None:
-            w[..., pkv[base + 1]] = gemv_uniform_group(block_size, q, pkv[base], pkv[base + 2], pkv[base + 3], b)
+            dqk = class_dequantize(pkv[base], pkv[base + 2], pkv[base + 3], b, low_normal)
+            w[..., pkv[base + 1]] = torch.matmul(q.float(), repeat_kv(dqk, n_rep).float()).to(torch.float16)
     if new_K is not None:
         w[..., real_len - new_len:] = torch.matmul(
             q.float(), repeat_kv(new_K, n_rep).transpose(2, 3).float()).half()
@@ -264,7 +316,7 @@ def qkv_matmul(
     for b in BITS:
         base = V_BASE[b]
         if pkv[base] is not None:
-            dq = uniform_group_dequantize_unpack_last_dim(pkv[base], pkv[base + 2], pkv[base + 3], group_size, b)
+            dq = class_dequantize(pkv[base], pkv[base + 2], pkv[base + 3], b, low_normal)
             _add(torch.matmul(w[..., pkv[base + 1]].float(), repeat_kv(dq, n_rep).float()))
     if new_V is not None:
         _add(torch.matmul(w[..., real_len - new_len:].float(), repeat_kv(new_V, n_rep).float()))
@@ -358,18 +410,18 @@ def _units_from_class(data, idx, scale, zero, bits, is_k):
     return units
 
 
-def _unit_fp16(u):
+def _unit_fp16(u, low_normal=False):
     if u["bits"] == 16:
         return u["x"]
     c, s, z = u["x"]
-    return uniform_group_dequantize_unpack_last_dim(c, s, z, 32, u["bits"])
+    return class_dequantize(c, s, z, u["bits"], low_normal)
 
 
-def _unit_requant(u, bits, scalar_div):
-    x = _unit_fp16(u)
+def _unit_requant(u, bits, scalar_div, low_normal=False):
+    x = _unit_fp16(u, low_normal)
     if bits == 16:
         return dict(idx=u["idx"], bits=16, x=x)
-    return dict(idx=u["idx"], bits=bits, x=uniform_group_quantize_pack_last_dim(x, 32, bits, scalar_div))
+    return dict(idx=u["idx"], bits=bits, x=class_quantize(x, bits, scalar_div, low_normal))
 
 
 def _class_from_units(units, bits, is_k):
@@ -383,7 +435,7 @@ def _class_from_units(units, bits, is_k):
             torch.cat([u["x"][1] for u in units], dim=dim), torch.cat([u["x"][2] for u in units], dim=dim))
 
 
-def _policy_side(pkv, new, history, sorted_idx, bit_num, is_k, scalar_div):
+def _policy_side(pkv, new, history, sorted_idx, bit_num, is_k, scalar_div, low_normal=False):
     """-> ({bits: units}, surviving positions before re-ranking or None if nothing was to be evicted)."""
     slots = K_BASE if is_k else V_BASE
     cls = {}
@@ -425,10 +477,10 @@ def _policy_side(pkv, new, history, sorted_idx, bit_num, is_k, scalar_div):
                 for g in range(len(moved) // 32):
                     grp = moved[32 * g:32 * g + 32]
                     x = torch.cat([u["x"] for u in grp], dim=2).transpose(2, 3).contiguous()   # (B,H,D,32)
-                    cls[tb].append(_unit_requant(dict(idx=torch.cat([u["idx"] for u in grp]), bits=16, x=x), tb, scalar_div))
+                    cls[tb].append(_unit_requant(dict(idx=torch.cat([u["idx"] for u in grp]), bits=16, x=x), tb, scalar_div, low_normal))
             else:
                 for u in moved:
-                    cls[tb].append(_unit_requant(dict(idx=u["idx"], bits=16, x=u["x"]), tb, scalar_div))
+                    cls[tb].append(_unit_requant(dict(idx=u["idx"], bits=16, x=u["x"]), tb, scalar_div, low_normal))
         for sb in _CLASS_BITS:
             if sb <= tb:
                 break
@@ -437,7 +489,7 @@ def _policy_side(pkv, new, history, sorted_idx, bit_num, is_k, scalar_div):
                 hit = [int(v) in tset for v in u["idx"].tolist()]
                 assert all(hit) or not any(hit)
                 if hit[0]:
-                    cls[tb].append(_unit_requant(u, tb, scalar_div))
+                    cls[tb].append(_unit_requant(u, tb, scalar_div, low_normal))
                 else:
                     stay.append(u)
             cls[sb] = stay
@@ -452,11 +504,13 @@ def _policy_side(pkv, new, history, sorted_idx, bit_num, is_k, scalar_div):
 
 def compress_cache(past_key_value: tuple, compress_length: int, history_length: int, K_sorted_idx, K_bit_num,
                    V_bit_num, token_importance, *, times_range: bool = True, scalar_div: str = "recip",
-                   weights_ring: Optional[torch.Tensor] = None):
+                   weights_ring: Optional[torch.Tensor] = None, quant_strategy: str = "uniform_group"):
     """One compression step; 6-entry bit_num = KV_cache_hqe_2, 5-entry = KV_cache_compress.
     Returns (new 42-tuple, ring of recent attention rows after eviction or None).  The 1-bit class is the
-    uniform one of the 'uniform_group' strategy (quant/hqe_2.py:482-484)."""
+    uniform one under 'uniform_group' and the normal-quantile one under
+    'high_uniform_group_low_normal_group' (quant/hqe_2.py:482-492)."""
     pkv = past_key_value
+    low_normal = quant_strategy == LOW_NORMAL_STRATEGY
     new_K, new_V = pkv[NEW_K], pkv[NEW_V]
     res_K = new_K[:, :, compress_length:, :].clone()
     res_V = new_V[:, :, compress_length:, :].clone()
@@ -465,8 +519,8 @@ def compress_cache(past_key_value: tuple, compress_length: int, history_length: 
     V_norm = calculate_token_range(new_V, pkv[V_TOKEN_NORM])
     V_score = token_importance * V_norm if times_range else token_importance.clone()
     V_sorted_idx = get_block_token_idx(32, total // 32, V_score)
-    k_cls, _ = _policy_side(pkv, new_K, history_length, K_sorted_idx, K_bit_num, True, scalar_div)
-    v_cls, v_alive = _policy_side(pkv, new_V, history_length, V_sorted_idx, V_bit_num, False, scalar_div)
+    k_cls, _ = _policy_side(pkv, new_K, history_length, K_sorted_idx, K_bit_num, True, scalar_div, low_normal)
+    v_cls, v_alive = _policy_side(pkv, new_V, history_length, V_sorted_idx, V_bit_num, False, scalar_div, low_normal)
     if v_alive is not None:
         keep = torch.tensor(v_alive, dtype=torch.int64)
         V_norm = V_norm[keep]
@@ -489,10 +543,11 @@ def compress_cache(past_key_value: tuple, compress_length: int, history_length: 
     return tuple(t), weights_ring
 
 
-def reconstruct_cache(past_key_value: tuple):
+def reconstruct_cache(past_key_value: tuple, quant_strategy: str = "uniform_group"):
     """Dense fp16 (K, V) (B,H,kv_seq_len,D) from the tuple (quant/hybrid_quant.py:732-846, with the 4-bit V
     class restored unconditionally)."""
     pkv = past_key_value
+    low_normal = quant_strategy == LOW_NORMAL_STRATEGY
     T = int(pkv[KV_SEQ_LEN])
     ref = next(x for x in (pkv[NEW_V], pkv[V16]) if x is not None) if (pkv[NEW_V] is not None or pkv[V16] is not None) else None
     if ref is not None:
@@ -509,10 +564,10 @@ def reconstruct_cache(past_key_value: tuple):
     for b in BITS:
         s = K_BASE[b]
         if pkv[s] is not None:
-            K[:, :, pkv[s + 1]] = uniform_group_dequantize_unpack_last_dim(pkv[s], pkv[s + 2], pkv[s + 3], 32, b).transpose(2, 3)
+            K[:, :, pkv[s + 1]] = class_dequantize(pkv[s], pkv[s + 2], pkv[s + 3], b, low_normal).transpose(2, 3)
         s = V_BASE[b]
         if pkv[s] is not None:
-            V[:, :, pkv[s + 1]] = uniform_group_dequantize_unpack_last_dim(pkv[s], pkv[s + 2], pkv[s + 3], 32, b)
+            V[:, :, pkv[s + 1]] = class_dequantize(pkv[s], pkv[s + 2], pkv[s + 3], b, low_normal)
     if pkv[NEW_K] is not None:
         K[:, :, T - pkv[NEW_K].shape[2]:] = pkv[NEW_K]
         V[:, :, T - pkv[NEW_V].shape[2]:] = pkv[NEW_V]
@@ -559,8 +614,10 @@ class DecodeLayerOracle:
     through identical policy decisions."""
 
     def __init__(self, head_dim: int, bit_0: float, bit_4: float, bit_2: float, bit_1: float = 0.0,
-                 times_range: bool = True, last_length: int = 20, max_length: int = 0, scalar_div: str = "recip"):
+                 times_range: bool = True, last_length: int = 20, max_length: int = 0, scalar_div: str = "recip",
+                 quant_strategy: str = "uniform_group"):
         self.head_dim = head_dim
+        self.quant_strategy = quant_strategy
         self.times_range = times_range
         self.scalar_div = scalar_div
         self.ratio_e_0 = torch.tensor([bit_0], dtype=torch.float32)
@@ -581,7 +638,7 @@ class DecodeLayerOracle:
             new_V = torch.cat((past_key_value[-2], v), dim=2) if past_key_value[-2] is not None else v
             past_key_value = past_key_value[:-3] + (new_K, new_V, kv_seq_len)
             attn_weights, attn_output = qkv_matmul(q, past_key_value, attention_mask, self.head_dim,
-                                                   use_mask=False, scalar_div=self.scalar_div)
+                                                   self.quant_strategy, use_mask=False, scalar_div=self.scalar_div)
         else:
             n_rep = q.shape[1] // k.shape[1]
             w = torch.matmul(q.float(), repeat_kv(k, n_rep).transpose(2, 3).float()).half()
@@ -619,7 +676,8 @@ class DecodeLayerOracle:
             past_key_value, ring = compress_cache(past_key_value, compress_length, self.history_reserve_length,
                                                   K_token_idx, K_bit_num, V_bit_num, sort_importance,
                                                   times_range=self.times_range, scalar_div=self.scalar_div,
-                                                  weights_ring=self.ring.weights)
+                                                  weights_ring=self.ring.weights,
+                                                  quant_strategy=self.quant_strategy)
             if ring is not None:
                 self.ring.weights = ring
             self.history_reserve_length += compress_length - eviction_len

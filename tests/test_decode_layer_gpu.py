@@ -30,9 +30,19 @@ def _causal_mask(T):
     return torch.triu(m, diagonal=1)[None, None]
 
 
-def _same_tuple(got, want, where):
+def _same_tuple(got, want, where, normal=False):
     assert len(got) == len(want) == 42
     for i, (a, b) in enumerate(zip(got, want)):
+        if normal and i in (28, 30, 31, 32, 34, 35) and a is not None and b is not None:
+            # normal-quantile 1-bit class: std / mean may differ in the last fp16 place in rare groups
+            # (torch.std_mean's accumulation order is not pinned), and with them the odd code next to the mean
+            a = a.cpu()
+            assert a.shape == b.shape and a.dtype == b.dtype, (where, i)
+            if a.dtype == torch.float16:
+                assert torch.allclose(a.float(), b.float(), rtol=2e-3, atol=1e-6), (where, i)
+            else:
+                assert float((a != b).float().mean()) < 0.02, (where, i)
+            continue
         if i == 41:
             assert int(a) == int(b), (where, i)
             continue
@@ -47,14 +57,18 @@ def _same_tuple(got, want, where):
             assert torch.equal(a, b), (where, i)
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,T0,steps", [(1, 8, 2, 300, 72), (2, 4, 4, 96, 40)])
-def test_layer_in_lockstep_with_oracle(dev, B, Hq, Hkv, T0, steps):
+@pytest.mark.parametrize("B,Hq,Hkv,T0,steps,strategy,bit_1", [
+    (1, 8, 2, 300, 72, "uniform_group", 0.0),
+    (2, 4, 4, 96, 40, "uniform_group", 0.0),
+    (1, 8, 2, 300, 72, "high_uniform_group_low_normal_group", 0.25),   # the reference's shipped default
+])
+def test_layer_in_lockstep_with_oracle(dev, B, Hq, Hkv, T0, steps, strategy, bit_1):
     from hqekv_amd.decode_layer import HqeAttentionLayer
     D = 128
-    ratios = dict(bit_0=0.2, bit_4=0.3, bit_2=0.5, bit_1=0.0)
-    layer = HqeAttentionLayer(D, **ratios)
+    ratios = dict(bit_0=0.2, bit_4=0.3, bit_2=0.5 - bit_1, bit_1=bit_1)
+    layer = HqeAttentionLayer(D, **ratios, quant_strategy=strategy)
     layer.set_max_length(T0 + steps)
-    orc = O.DecodeLayerOracle(D, **ratios, max_length=T0 + steps)
+    orc = O.DecodeLayerOracle(D, **ratios, max_length=T0 + steps, quant_strategy=strategy)
 
     pkv_g = pkv_o = None
     compressions = 0
@@ -86,7 +100,7 @@ def test_layer_in_lockstep_with_oracle(dev, B, Hq, Hkv, T0, steps):
         assert torch.allclose(ring_g.float(), orc.ring.weights.float(), rtol=2e-3, atol=1e-3), where
         assert layer.last_weights.next_line == orc.ring.next_line, where
         orc.ring.weights.copy_(ring_g)
-        _same_tuple(pkv_g, pkv_o, where)
+        _same_tuple(pkv_g, pkv_o, where, normal=strategy != "uniform_group")
     assert compressions >= 2
     kept = sum(pkv_g[s].shape[2] for s in (2, 8, 16, 24, 32) if pkv_g[s] is not None)
     assert kept == layer.history_reserve_length

@@ -60,6 +60,29 @@ def test_hqe2_matches_oracle(dev, case, permute, fused, monkeypatch):
     torch.testing.assert_close(w.float().sum(-1).cpu(), torch.ones(case["B"], case["Hq"], 1), rtol=0, atol=5e-3)
 
 
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "general"])
+def test_low_normal_strategy_one_bit_class(dev, fused, monkeypatch):
+    """'high_uniform_group_low_normal_group': the 1-bit class holds normal-quantile codes with (std, mean)."""
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    from hqekv_amd.quant_matmul_hq import qkv_matmul
+    monkeypatch.setenv("HQEKV_UNFUSED", "0" if fused else "1")
+    strategy = "high_uniform_group_low_normal_group"
+    B, Hq, Hkv, T, D, residual = 1, 8, 2, 2048 + 11, 128, 11
+    q, K, V = synth.make_qkv(B, Hq, Hkv, T, D, 21)
+    classes = synth.split_blocks(T - residual, (0.05, 0.1, 0.2, 0.25, 0.3, 0.1), 21)
+    cache = synth.build_cache(K, V, classes, residual, lambda x, g, b: O.class_quantize(x, b, low_normal=True))
+    w_ref, o_ref = O.qkv_matmul(q, cache, None, D, strategy, use_mask=False)
+    w, o = qkv_matmul_hqe_2(q.to(dev), synth.cache_to(cache, dev), None, D, strategy)
+    _close(w, w_ref, "attn_weights")
+    _close(o, o_ref, "attn_output")
+    # the same cache read as uniform 1-bit is a different function: the layouts are told apart
+    w_u, _ = qkv_matmul_hqe_2(q.to(dev), synth.cache_to(cache, dev), None, D, "uniform_group")
+    assert not torch.allclose(w_u.float().cpu(), w_ref.float(), rtol=RTOL, atol=ATOL)
+    w2, o2 = qkv_matmul(q.to(dev), synth.cache_to(cache, dev), None, D, strategy)
+    _close(w2, w_ref, "qkv_matmul attn_weights")
+    _close(o2, o_ref, "qkv_matmul attn_output")
+
+
 def test_qkv_matmul_with_mask(dev):
     from hqekv_amd.quant_matmul_hq import qkv_matmul, qkv_matmul_hq
     case = CASES[1]

@@ -272,3 +272,39 @@ def test_layer_state_machine_bookkeeping():
         idx = torch.cat([pkv[s + 1] for s in (O.V16, O.V_BASE[8], O.V_BASE[4], O.V_BASE[2], O.V_BASE[1]) if pkv[s] is not None])
         assert torch.equal(torch.sort(idx)[0], torch.arange(kept))
     assert evicted > 0
+
+
+# ------------------------------------------------------------------ 1-bit normal-quantile class
+def test_normal1_known_answer_and_closed_form():
+    """arange(32): mean 15.5, unbiased std sqrt(88) = 9.3808 -> fp16 9.3828; code = [k > 15.5]; the two
+    dequantised values are rnd16(mean -+ rnd16(fp16(0.6745) * std)), worked out with numpy float16."""
+    import numpy as np
+    x = torch.arange(0, 32, dtype=torch.float16).reshape(1, 1, 1, 32)
+    code, std, mean = O.normal_group_quantize_pack_last_dim(x, 32, 1)
+    assert (code.item() & 0xFFFFFFFF) == 0xFFFF0000
+    assert mean.item() == 15.5 and std.item() == float(np.float16(np.sqrt(88.0)))
+    k16 = np.float16(0.6744897501960817)
+    assert float(k16) == 0.67431640625
+    a = np.float16(k16 * np.float16(std.item()))
+    lo, hi = np.float16(np.float16(15.5) - a), np.float16(np.float16(15.5) + a)
+    dq = O.normal_group_dequantize_unpack_last_dim(code, std, mean, 32, 1).flatten().tolist()
+    assert dq == [float(lo)] * 16 + [float(hi)] * 16
+
+
+def test_normal1_statistics_and_sign_rule():
+    import numpy as np
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(2, 2, 8, 128, generator=g) * 3 + 1).half()
+    code, std, mean = O.normal_group_quantize_pack_last_dim(x, 32, 1)
+    xg = x.reshape(-1, 32).double().numpy()
+    # unbiased (n - 1) standard deviation and plain mean, within one fp16 step of the float64 values
+    ref_std, ref_mean = xg.std(axis=1, ddof=1), xg.mean(axis=1)
+    assert np.all(np.abs(std.flatten().double().numpy() - ref_std) <= ref_std * 2 ** -10)
+    assert np.all(np.abs(mean.flatten().double().numpy() - ref_mean) <= np.maximum(np.abs(ref_mean), 2 ** -10) * 2 ** -10)
+    # the code is the sign of x - mean (fp16), ties and negatives to 0
+    c = O.unpack_codes(code, 1).reshape(-1, 32)
+    u = (x.reshape(-1, 32) - mean.reshape(-1, 1))
+    assert torch.equal(c, (u > 0).to(torch.int32))
+    # a constant group stores code 0 everywhere
+    z = torch.full((1, 1, 1, 32), 2.5, dtype=torch.float16)
+    assert O.normal_group_quantize_pack_last_dim(z, 32, 1)[0].item() == 0

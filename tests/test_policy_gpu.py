@@ -24,7 +24,10 @@ def _same(a, b, what):
         assert a == b, what
 
 
-def test_hqe2_policy_bit_exact_over_three_compressions(dev):
+@pytest.mark.parametrize("strategy", ["uniform_group", "high_uniform_group_low_normal_group"])
+def test_hqe2_policy_bit_exact_over_three_compressions(dev, strategy):
+    """Under the second strategy the 1-bit class is quantised with the normal-quantile rule (std, mean in the
+    scale / zero slots); everything else is unchanged."""
     from hqekv_amd.hqe_2 import KV_cache_hqe_2
     from hqekv_amd.public_func import get_block_token_idx, last_attn_weights
 
@@ -35,17 +38,33 @@ def test_hqe2_policy_bit_exact_over_three_compressions(dev):
     ring = {"cpu": ring0.clone()}
 
     def prod(pkv, cl, hist, ks, kb, vb, imp):
-        return KV_cache_hqe_2(pkv, cl, hist, ks, kb, vb, imp, "uniform_group", lw)
+        return KV_cache_hqe_2(pkv, cl, hist, ks, kb, vb, imp, strategy, lw)
 
     def orac(pkv, cl, hist, ks, kb, vb, imp):
-        out, ring["cpu"] = O.compress_cache(pkv, cl, hist, ks, kb, vb, imp, weights_ring=ring["cpu"])
+        out, ring["cpu"] = O.compress_cache(pkv, cl, hist, ks, kb, vb, imp, weights_ring=ring["cpu"],
+                                            quant_strategy=strategy)
         return out
 
     got, _, _ = PC.run(prod, to_dev=lambda x: x.to(dev),
                        rank_blocks=lambda bs, bn, imp: get_block_token_idx(bs, bn, imp.to(dev)).cpu())
     want, _, _ = PC.run(orac)
+    normal = strategy != "uniform_group"
     for step, (g, w) in enumerate(zip(got, want)):
         for slot in range(42):
+            if normal and slot in (28, 30, 31, 32, 34, 35) and g[slot] is not None:
+                # std / mean of the normal-quantile class: torch.std_mean's accumulation order is not pinned,
+                # so the last fp16 place (and with it the odd code next to the mean) may differ in rare groups
+                a, b = g[slot].cpu(), w[slot]
+                assert a.shape == b.shape and a.dtype == b.dtype
+                if a.dtype == torch.int32:
+                    diff = (a ^ b).to(torch.int64) & 0xFFFFFFFF
+                    flipped = sum(int(((diff >> k) & 1).sum()) for k in range(32))
+                    assert flipped <= 0.002 * a.numel() * 32, (step, slot, flipped)
+                else:
+                    d = (a.float() - b.float()).abs()
+                    step16 = torch.exp2(torch.floor(torch.log2(b.float().abs().clamp_min(2.0 ** -14))) - 10)
+                    assert bool((d <= step16).all()) and float((d > 0).float().mean()) < 0.01, (step, slot)
+                continue
             _same(g[slot], w[slot], f"step {step} slot {slot}")
     _same(lw.weights, ring["cpu"], "ring of recent attention rows after eviction")
 
@@ -87,9 +106,8 @@ def test_policy_errors(dev):
     with pytest.raises(ValueError, match="invalid quant_strategy"):
         KV_cache_hqe_2(pkv, 64, 0, ks, six, six, imp, "bogus")
     with pytest.raises(NotImplementedError):
-        # a populated 1-bit class under this strategy would be the normal-quantile one
-        KV_cache_hqe_2(pkv, 64, 0, ks, torch.tensor([32, 0, 0, 0, 32, 0], dtype=torch.int32), six, imp,
-                       "high_uniform_group_low_normal_group")
+        # the per-row / all-normal quantiser families are not part of this library
+        KV_cache_hqe_2(pkv, 64, 0, ks, six, six, imp, "normal_group")
     with pytest.raises(ValueError):
         KV_cache_hqe_2(pkv, 48, 0, ks, six, six, imp, "uniform_group")
     with pytest.raises(ValueError):
