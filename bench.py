@@ -32,6 +32,7 @@ WORKLOADS = {
     "c1": "Llama-3.1-8B shape, B=1, ctx 4096: 3968 tokens 2-bit + 128 fp16 residual",
     "c2": "Llama-3.1-8B shape, B=1, ctx 32768 hybrid: fp16 5% / 8-bit 15% / 4-bit 30% / 2-bit 30% / evicted 20%",
     "c4": "Qwen3-8B shape, B=8, ctx 65536 hybrid: fp16 10% / 4-bit 20% / 2-bit 50% / evicted 20%",
+    "c5": "decode-attention share of config 5: Llama-3.1-8B shape, B=4, ctx 131072 hybrid: fp16 2% / 8-bit 3% / 4-bit 25% / 2-bit 50% / evicted 20% (2.56 bit average), 32 layers resident",
     "c3": "quantize-and-pack: 8 KV heads x 128 x 8192 new fp16 tokens appended at token 24576 of a 32768-token cache",
 }
 
@@ -102,7 +103,7 @@ def cpu_baseline(name: str, n_iter: int = 5):
     B = cfg["B"]
     sample = "one layer-step, all batch rows"
     scale = 1.0
-    if name == "c4":  # bounded sample: one batch row, scaled by B
+    if B > 1:  # bounded sample: one batch row, scaled by B
         cfg = dict(cfg, B=1)
         sample = f"one layer-step of ONE batch row, time x{B}"
         scale = float(B)
@@ -269,7 +270,7 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    n_layers = args.layers or {"c1": 64, "c2": 32, "c4": 4}[args.workload]
+    n_layers = args.layers or {"c1": 64, "c2": 32, "c4": 4, "c5": 32}[args.workload]
     layers = build_layers(args.workload, n_layers, dev)
     plans = [DecodePlan(q, cache) for q, cache in layers]
     qs = [q.contiguous() for q, _ in layers]
@@ -362,6 +363,11 @@ def main():
                      "bytes_per_launch": dom_bytes, "avg_us": round(dom_us, 3)},
     }
 
+    if args.workload == "c5":
+        # one generated token passes through every resident layer once
+        out["decode_attention_only"] = {"layers": n_layers, "us_per_token_step": round(us_per_step * n_layers, 1),
+                                        "tokens_per_s_attention_only": round(cfg["B"] / (us_per_step * n_layers * 1e-6), 1),
+                                        "note": "the model's projections, MLP and prompt pass are outside this path"}
     if not args.no_cpu:
         base, (q_cpu, cache_cpu, ref) = cpu_baseline(args.workload)
         out["cpu_baseline"] = base

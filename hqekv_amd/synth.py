@@ -132,6 +132,8 @@ CONFIGS = {
     "c1": dict(B=1, Hq=32, Hkv=8, D=128, T=4096, residual=128, fractions=(0.0, 0.0, 0.0, 1.0, 0.0), seed=1235),
     "c2": dict(B=1, Hq=32, Hkv=8, D=128, T=32768, residual=0, fractions=(0.05, 0.15, 0.30, 0.30, 0.20), seed=1236),
     "c4": dict(B=8, Hq=32, Hkv=8, D=128, T=65536, residual=0, fractions=(0.10, 0.0, 0.20, 0.50, 0.20), seed=1238),
+    # the decode-attention share of configuration 5: average 2.56 bit per kept-or-evicted element
+    "c5": dict(B=4, Hq=32, Hkv=8, D=128, T=131072, residual=0, fractions=(0.02, 0.03, 0.25, 0.50, 0.20), seed=1239),
 }
 
 
