@@ -183,7 +183,9 @@ __device__ __forceinline__ void consume_words(uint32_t w0, uint32_t w1, half2_t 
 // another's arithmetic).
 constexpr int QK_TPL = 8;               // tokens per lane in every channel-major class
 constexpr int QK_TILE = 64 * QK_TPL;    // tokens per workgroup tile
-constexpr int QK_UNR = 4;               // row pairs per block; two blocks of loads are in flight per wave
+// row pairs per register block (two blocks of loads are in flight per wave): 2 with 8 waves per tile, where
+// the smaller blocks keep the kernel at 4 waves per SIMD; 4 with 4 waves per tile
+__host__ __device__ constexpr int qk_unr(int waves) { return waves == 8 ? 2 : 4; }
 
 __host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
   return (bits == 16 && token_major) ? 64 : QK_TILE;
@@ -191,7 +193,7 @@ __host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
 
 // What a lane holds of one block of QK_UNR row pairs of a quantised class (32-bit members only: a struct
 // with 16-bit members is not kept in registers).
-template <int BITS>
+template <int BITS, int QK_UNR>
 struct QkBlock {
   static constexpr int NW = BITS == 8 ? 2 : 1;  // packed words per lane per row
   uint32_t w0[QK_UNR][NW], w1[QK_UNR][NW];
@@ -209,7 +211,9 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
                                                     StageQ &&stage_q, const half2_t *q2s,
                                                     float (&acc)[NREP][QK_TPL]) {
   constexpr int PF = 32 / BITS;
-  constexpr int NW = QkBlock<BITS>::NW;
+  constexpr int QK_UNR = qk_unr(QK_WAVES);
+  using Block = QkBlock<BITS, QK_UNR>;
+  constexpr int NW = Block::NW;
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t wpr = n / PF;   // words per row
   const uint32_t gpr = n >> 5;   // groups per row
@@ -223,7 +227,7 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
   const rsrc_t rz = make_rsrc(sg.zero + (int64_t)bh * D * gpr, (uint32_t)D * gpr * 2u);
   const int DP = D >> 1;
 
-  auto load = [&](int dp0, QkBlock<BITS> &r) {
+  auto load = [&](int dp0, Block &r) {
 #pragma unroll
     for (int k = 0; k < QK_UNR; ++k) {
       const int dpk = dp0 + QK_WAVES * k;
@@ -240,7 +244,7 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
       r.z1[k] = buf_u16(rz, gofs, grow + gpr * 2u);
     }
   };
-  auto compute = [&](int dp0, const QkBlock<BITS> &r) {
+  auto compute = [&](int dp0, const Block &r) {
 #pragma unroll
     for (int k = 0; k < QK_UNR; ++k) {
       const int dp = dp0 + QK_WAVES * k;
@@ -277,7 +281,7 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
 
   // two register blocks in turn: while one is consumed the other one's loads are in flight
   constexpr int STEP = QK_WAVES * QK_UNR;
-  QkBlock<BITS> ba, bb;
+  Block ba, bb;
   load(wave, ba);
   stage_q();
 #pragma unroll 1
