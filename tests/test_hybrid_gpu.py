@@ -218,6 +218,33 @@ def test_fused_path_is_deterministic_and_reusable(dev):
     _close(o0, orr.cpu(), "fused vs general attn_output")
 
 
+@pytest.mark.parametrize("flags", [1, 0], ids=["fused", "general"])
+def test_plan_replayed_from_a_hip_graph(dev, flags):
+    """A captured decode step (no allocation, no memset inside) replayed several times with new queries,
+    eager launches and synchronisations in between: every replay equals the eager result bit for bit."""
+    from hqekv_amd.attention import DecodePlan
+    q, cache = _case(**CASES[1])
+    c = synth.cache_to(cache, dev)
+    plan = DecodePlan(q.to(dev), c, flags=flags)
+    eager = DecodePlan(q.to(dev), c, flags=flags)
+    q_static = q.to(dev).clone()
+    plan.run(q_static)                       # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.run(q_static)
+    g = torch.Generator().manual_seed(99)
+    for rep in range(4):
+        q_new = torch.randn(q.shape, generator=g).half().to(dev)
+        q_static.copy_(q_new)
+        graph.replay()
+        torch.cuda.synchronize()
+        w_g, o_g = plan.weights.clone(), plan.out.clone()
+        w_e, o_e = [x.clone() for x in eager.run(q_new)]   # the program's own eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(w_g, w_e) and torch.equal(o_g, o_e), rep
+
+
 def test_config2_full_size_against_oracle(dev):
     """BASELINE config 2 at its full size (B=1, 32 query heads, 8 KV heads, context 32768, hybrid split with
     20 % evicted): caches built by the HIP quantiser are bit-identical to the oracle's, attention within
