@@ -246,7 +246,7 @@ def test_plan_replayed_from_a_hip_graph(dev, flags):
 
 
 def test_config2_full_size_against_oracle(dev):
-    """BASELINE config 2 at its full size (B=1, 32 query heads, 8 KV heads, context 32768, hybrid split with
+    """Benchmark configuration 2 at its full size (B=1, 32 query heads, 8 KV heads, context 32768, hybrid split with
     20 % evicted): caches built by the HIP quantiser are bit-identical to the oracle's, attention within
     tolerance, and the probabilities of every head sum to one."""
     from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
