@@ -199,6 +199,17 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
     """Run one compression on one side.  ``new`` is (B, H, n_new, D) fp16 (token-major for K and V alike)."""
     dev = new.device
     new_idx = torch.arange(history, history + new.shape[2], device=dev, dtype=torch.int64)
+    # membership of a position in a target set through one label per position (what the reference asks with
+    # torch.isin per class, quant/hqe_2.py:552-659): label[p] = index of the target list that holds p
+    total = history + new.shape[2]
+    label = torch.full((total,), -1, dtype=torch.int8, device=dev)
+    for ti, tgt in enumerate(targets):
+        if tgt is not None:
+            label[tgt.to(dev)] = ti
+
+    def member(idx: torch.Tensor, ti: int) -> torch.Tensor:
+        return label[idx] == ti
+
     split, to16, append = (_k_split, _k_to_fp16, _k_append) if is_k else (_v_split, _v_to_fp16, _v_append)
     evict = targets[5] if len(targets) > 5 else None
 
@@ -211,14 +222,14 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
 
     # 1. eviction: dropped tokens leave every tensor
     if evict is not None:
-        m = torch.isin(new_idx, evict)
+        m = member(new_idx, 5)
         if bool(m.any()):
             take_new(m)
         for b in CLASS_BITS:
             c = side[b]
             if c.idx is None:
                 continue
-            m = torch.isin(c.idx, evict)
+            m = member(c.idx, 5)
             if bool(m.any()):
                 _, side[b] = split(c, b, m)
         if on_evict is not None:
@@ -230,7 +241,7 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
         if tgt_idx is None:
             continue
         if new_idx.numel():
-            m = torch.isin(new_idx, tgt_idx)
+            m = member(new_idx, ti)
             if bool(m.any()):
                 if tgt_bits < 16:
                     _check_low_bits(tgt_bits, strategy)
@@ -243,7 +254,7 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
             c = side[src_bits]
             if c.idx is None:
                 continue
-            m = torch.isin(c.idx, tgt_idx)
+            m = member(c.idx, ti)
             if not bool(m.any()):
                 continue
             _check_low_bits(tgt_bits, strategy)
