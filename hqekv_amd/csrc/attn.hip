@@ -38,16 +38,26 @@ struct SegDev {
   int32_t bits;
   int32_t layout;      // HQEKV_LAYOUT_*: 1 = fp16 K stored token-major, 2 = 1-bit normal-quantile coding
   int32_t unit_begin;  // first chunk of this segment in the p.V partial buffer
-  int32_t n_units;     // tiles (q.K^T) or chunks (p.V) of this segment; blockIdx.z selects the segment
+  int32_t n_units;     // tiles (q.K^T) or chunks (p.V) of this segment
 };
 
 struct SegTable {
   SegDev seg[HQEKV_MAX_SEGS];
   int32_t nseg;
   int32_t total_units;
-  int32_t max_units;   // grid.y: the largest n_units of any segment
+  int32_t max_units;   // the largest n_units of any segment
   int32_t pad_;
+  int32_t begin[HQEKV_MAX_SEGS];  // unit_begin of every segment (INT32_MAX past nseg): one scalar load finds a unit's segment
 };
+
+// grid.y enumerates the units of all segments back to back (no idle workgroups): unit u belongs to the last
+// segment whose first unit is <= u.  Branch-free on the eight begins, which arrive in one scalar load.
+__device__ __forceinline__ int seg_of_unit(const SegTable &tb, int u) {
+  int s = -1;
+#pragma unroll
+  for (int k = 0; k < HQEKV_MAX_SEGS; ++k) s += (u >= tb.begin[k]) ? 1 : 0;
+  return s;
+}
 
 // Optional fusion of the softmax into the two GEMV launches (valid when no mask is added and the K
 // classes as well as the V classes each cover every position exactly once):
@@ -62,9 +72,9 @@ struct FuseArgs {
   float inv_sqrt_d;
 };
 
-// A workgroup learns its segment and its tile/chunk from its (remapped) block id, so everything it
-// needs from the kernel arguments is fetched in one batch at the top of the kernel (a scalar load that
-// misses costs about a microsecond; a lookup through the table would chain several of them).
+// A workgroup learns its segment and its tile/chunk from its block id with two scalar loads at the top of
+// the kernel: the eight unit begins, then the segment's 64-byte entry (a scalar load that misses costs about
+// a microsecond; walking the table entry by entry would chain several of them).
 
 // Workgroups are handed to the 8 XCDs round-robin in launch order, and each XCD has its own L2.
 // Neighbouring tiles of one (b, kv head) slab share cache lines (a tile's row segment is shorter than a
@@ -448,9 +458,8 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int bh = blockIdx.x;
   const int b = bh / Hkv, hkv = bh % Hkv;
-  const int tile = blockIdx.y;
-  const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads, no lazy re-reads
-  if (tile >= sg.n_units) return;  // uniform: grid.y is the largest tile count of any segment
+  const SegDev sg = tb.seg[seg_of_unit(tb, blockIdx.y)];  // by value: one batch of scalar loads, no lazy re-reads
+  const int tile = (int)blockIdx.y - sg.unit_begin;
   const bool tm = sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR;
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t t0 = (uint32_t)tile * QK_TILE + lane * QK_TPL;
@@ -907,9 +916,9 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
   __shared__ float red[PV_WAVES * NREP * D];
   __shared__ PvStage<NREP, D / 32> st;
   __shared__ float sm_ml[2 * NREP];  // fused mode: (max, 1 / sum exp) of each query head's row
-  const int bh = blockIdx.x, ux = blockIdx.y;
-  const SegDev sg = tb.seg[blockIdx.z];  // by value: one batch of scalar loads
-  if (ux >= sg.n_units) return;  // uniform: grid.y is the largest chunk count of any segment
+  const int bh = blockIdx.x;
+  const SegDev sg = tb.seg[seg_of_unit(tb, blockIdx.y)];  // by value: one batch of scalar loads
+  const int ux = (int)blockIdx.y - sg.unit_begin;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = bh / Hkv, hkv = bh % Hkv;
   const int chunk_id = sg.unit_begin + ux;
@@ -1059,9 +1068,11 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
     units += nu;
     if (nu > 65535) return fail(HQEKV_E_ARG, "%s: segment %d needs %lld work units (limit 65535)", who, k, (long long)nu);
   }
+  if (units > 65535) return fail(HQEKV_E_UNSUPPORTED, "%s: %lld work units in one launch (limit 65535)", who, (long long)units);
   tb->nseg = m;
   tb->total_units = (int32_t)units;
   tb->max_units = (int32_t)max_units;
+  for (int k = 0; k < HQEKV_MAX_SEGS; ++k) tb->begin[k] = k < m ? tb->seg[k].unit_begin : 0x7fffffff;
   tb->pad_ = 0;
   (void)D;
   return HQEKV_OK;
@@ -1086,7 +1097,7 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
   // few tiles: 8 waves per tile; many tiles (several workgroups queue up per CU): 4 waves per tile
   static const char *force = getenv("HQEKV_QK_WAVES");
   const int waves = force ? atoi(force) : ((int64_t)tb.total_units * B * Hkv <= 1024 ? 8 : 4);
-  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.max_units, (unsigned)tb.nseg), block((unsigned)waves * 64);
+  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units), block((unsigned)waves * 64);
   const int rh = waves == 4 ? (nrep < 4 ? nrep : 4) : (nrep < 2 ? nrep : 2);  // QkReduce::RH
   const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
 #define LAUNCH(N_, W_)                                                                                        \
@@ -1129,7 +1140,7 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
   const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
   if (tb.total_units > 0 && (stages & 1)) {
-    dim3 grid((unsigned)(B * Hkv), (unsigned)tb.max_units, (unsigned)tb.nseg), block(PV_THREADS);
+    dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units), block(PV_THREADS);
 #define LAUNCH(N_, D_)                                                                                   \
   hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
                      (int)Hkv, Tall, chunk, n_bhq, fz)
