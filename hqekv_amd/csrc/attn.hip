@@ -372,7 +372,10 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
   }
 }
 
-// fp16 residual stored token-major (B,Hkv,T,D): a wave walks tokens, lanes split the channels
+// fp16 residual stored token-major (B,Hkv,T,D), one 64-token tile per workgroup.
+// D == 128: a wave takes 8 tokens at a time, 8 lanes per token, 16 channels (two 128-bit loads) per lane, so
+// all of a wave's loads are in flight together and a token's dot product is reduced across 8 lanes.
+// Other D: a wave walks its tokens one by one, lanes split the channels.
 template <int NREP, int QK_WAVES>
 __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int bh, int b, int hkv, int D,
                                                int Hq, int64_t Tall, int wave, int lane, const half2_t *q2s,
@@ -380,35 +383,76 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
   const int64_t n = sg.n_tokens;
   const half_t *kb = (const half_t *)sg.data + (int64_t)bh * n * D;
   const int DP = D >> 1;
+  constexpr int TPW = 64 / QK_WAVES;  // tokens per wave
   float m_run[NREP], l_run[NREP];  // running softmax statistics of this wave's tokens (fused mode)
 #pragma unroll
   for (int h = 0; h < NREP; ++h) {
     m_run[h] = -INFINITY;
     l_run[h] = 0.f;
   }
-#pragma unroll 1
-  for (int k = 0; k < 64 / QK_WAVES; ++k) {
-    const int64_t t = (int64_t)tile * 64 + wave * (64 / QK_WAVES) + k;
-    if (t >= n) break;  // uniform per wave
-    float part[NREP];
+  if (D == 128) {
+    const int lg = lane & 7, tsub = lane >> 3;
 #pragma unroll
-    for (int h = 0; h < NREP; ++h) part[h] = 0.f;
-    for (int dp = lane; dp < DP; dp += 64) {
-      const half2_t kk = *reinterpret_cast<const half2_t *>(kb + t * D + 2 * dp);
+    for (int r = 0; r < TPW / 8; ++r) {
+      const int64_t t = (int64_t)tile * 64 + wave * TPW + r * 8 + tsub;
+      const bool valid = t < n;
+      const int64_t tc = valid ? t : n - 1;
+      const uint4 *src = reinterpret_cast<const uint4 *>(kb + tc * 128 + lg * 16);
+      const uint4 lo = src[0], hi = src[1];
+      const uint32_t pos = sg.idx ? reinterpret_cast<const uint32_t *>(sg.idx)[2 * tc] : (uint32_t)(sg.pos_base + tc);
+      const uint32_t kw[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      float part[NREP];
 #pragma unroll
-      for (int h = 0; h < NREP; ++h) part[h] = __builtin_amdgcn_fdot2(kk, q2s[dp * NREP + h], part[h], false);
-    }
-    const int64_t pos = sg.idx ? sg.idx[t] : sg.pos_base + t;
+      for (int h = 0; h < NREP; ++h) part[h] = 0.f;
 #pragma unroll
-    for (int h = 0; h < NREP; ++h) {
-      half_t r = (half_t)wave_sum(part[h]);
-      if (fz.stats) {
-        r = (half_t)((float)r * fz.inv_sqrt_d);
-        const float x = (float)r, mn = fmaxf(m_run[h], x);
-        l_run[h] = l_run[h] * __expf(m_run[h] - mn) + __expf(x - mn);
-        m_run[h] = mn;
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int h = 0; h < NREP; ++h)
+          part[h] = __builtin_amdgcn_fdot2(as_h2(kw[j]), q2s[(lg * 8 + j) * NREP + h], part[h], false);
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) {
+        float v = part[h];
+        v += xor_f(v, 1);
+        v += xor_f(v, 2);
+        v += xor_f(v, 4);
+        half_t rr = (half_t)v;
+        if (fz.stats) {
+          rr = (half_t)((float)rr * fz.inv_sqrt_d);
+          const float x = valid ? (float)rr : -INFINITY;
+          const float mn = fmaxf(m_run[h], wave_max(x));
+          const float e = (valid && lg == 0) ? __expf(x - mn) : 0.f;
+          const float keep = (m_run[h] == mn) ? 1.f : __expf(m_run[h] - mn);  // also covers -inf == -inf
+          l_run[h] = l_run[h] * keep + wave_sum(e);
+          m_run[h] = mn;
+        }
+        if (valid && lg == 0) scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = rr;
       }
-      if (lane == 0) scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = r;
+    }
+  } else {
+#pragma unroll 1
+    for (int k = 0; k < TPW; ++k) {
+      const int64_t t = (int64_t)tile * 64 + wave * TPW + k;
+      if (t >= n) break;  // uniform per wave
+      float part[NREP];
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) part[h] = 0.f;
+      for (int dp = lane; dp < DP; dp += 64) {
+        const half2_t kk = *reinterpret_cast<const half2_t *>(kb + t * D + 2 * dp);
+#pragma unroll
+        for (int h = 0; h < NREP; ++h) part[h] = __builtin_amdgcn_fdot2(kk, q2s[dp * NREP + h], part[h], false);
+      }
+      const int64_t pos = sg.idx ? sg.idx[t] : sg.pos_base + t;
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) {
+        half_t r = (half_t)wave_sum(part[h]);
+        if (fz.stats) {
+          r = (half_t)((float)r * fz.inv_sqrt_d);
+          const float x = (float)r, mn = fmaxf(m_run[h], x);
+          l_run[h] = l_run[h] * __expf(m_run[h] - mn) + __expf(x - mn);
+          m_run[h] = mn;
+        }
+        if (lane == 0) scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = r;
+      }
     }
   }
   if (fz.stats) {  // one (m, l) pair per head for the whole 64-token tile
