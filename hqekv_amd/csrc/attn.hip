@@ -1006,17 +1006,39 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
     case 8: pv_chunk<8, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
     default: pv_chunk<16, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
   }
-  // lanes 16 and 32 apart hold the same channels of other tokens
+  // Lanes 16, 32 and 48 apart hold the same channels of other tokens.  Their sum is needed in lanes 0-15
+  // only: two lane-row swaps on the vector ALU per value (a swap exchanges rows of 16 lanes between two
+  // registers: the odd rows of the first with the even rows of the second, then the upper half of the first
+  // with the lower half of the second) instead of two trips through the LDS crossbar, which 16 waves per CU
+  // saturate (2.8 us of a 9 us workgroup life at 32k context).
   const int cl = lane & 15;
 #pragma unroll
-  for (int h = 0; h < NREP; ++h)
+  for (int h = 0; h < NREP; ++h) {
+    float v[PV_CPL], o[PV_CPL];
 #pragma unroll
-    for (int i = 0; i < PV_CPL; ++i) {
-      float v = acc[h][i];
-      v += xor_f(v, 16);
-      v += xor_f(v, 32);
-      if (lane < 16) red[(wave * NREP + h) * D + cl * PV_CPL + i] = v;
+    for (int i = 0; i < PV_CPL; ++i) v[i] = o[i] = acc[h][i];
+    static_assert(PV_CPL == 8, "the swap batches below name eight register pairs");
+    // The swaps need idle issue slots between a vector-ALU write of their operands and themselves, and
+    // between themselves and the first read of their results; the compiler does not see into the asm, so
+    // each batch of eight independent swaps carries its own (generous) wait states.
+#define HQ_SWAP8(OP_)                                                                                         \
+  asm volatile("s_nop 7\n\t" OP_ " %0, %8\n\t" OP_ " %1, %9\n\t" OP_ " %2, %10\n\t" OP_ " %3, %11\n\t"         \
+               OP_ " %4, %12\n\t" OP_ " %5, %13\n\t" OP_ " %6, %14\n\t" OP_ " %7, %15\n\ts_nop 7"               \
+               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), \
+                 "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]))
+    HQ_SWAP8("v_permlane16_swap_b32");  // rows 0 and 2: o = the old rows 1 and 3
+#pragma unroll
+    for (int i = 0; i < PV_CPL; ++i) v[i] = o[i] = v[i] + o[i];
+    HQ_SWAP8("v_permlane32_swap_b32");  // row 0: o = the old row 2
+#undef HQ_SWAP8
+#pragma unroll
+    for (int i = 0; i < PV_CPL; ++i) v[i] += o[i];
+    if (lane < 16) {
+      float4 *dst = reinterpret_cast<float4 *>(red + (wave * NREP + h) * D + cl * PV_CPL);
+      dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+      dst[1] = make_float4(v[4], v[5], v[6], v[7]);
     }
+  }
   __syncthreads();
   for (int k = threadIdx.x; k < NREP * D; k += PV_THREADS) {
     const float v = red[k] + red[NREP * D + k] + red[2 * NREP * D + k] + red[3 * NREP * D + k];
