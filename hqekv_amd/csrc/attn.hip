@@ -411,10 +411,10 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
           part[h] = __builtin_amdgcn_fdot2(as_h2(kw[j]), q2s[(lg * 8 + j) * NREP + h], part[h], false);
 #pragma unroll
       for (int h = 0; h < NREP; ++h) {
-        float v = part[h];
-        v += xor_f(v, 1);
-        v += xor_f(v, 2);
-        v += xor_f(v, 4);
+        float v = part[h];  // the token's 8 lanes: two quad permutes, then the half-row mirror joins the quads
+        v += dpp_f<0xB1>(v);
+        v += dpp_f<0x4E>(v);
+        v += dpp_f<0x141>(v);
         half_t rr = (half_t)v;
         if (fz.stats) {
           rr = (half_t)((float)rr * fz.inv_sqrt_d);

@@ -32,16 +32,36 @@ __device__ __forceinline__ uint32_t xor_u(uint32_t v, int m) {
   return (uint32_t)__shfl_xor((int)v, m, HQ_WAVE);
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += xor_f(v, m);
-  return v;
+// Wave-wide reductions without the LDS crossbar: four DPP steps reduce each row of 16 lanes in place
+// (quad permutes for lanes 1 and 2 apart, then the two mirrors), two lane-row swaps bring the four row
+// results into row 0, and lane 0 is broadcast.  The swaps need idle issue slots before and after them
+// that the compiler does not insert around inline asm.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, xor_f(v, m));
-  return v;
+__device__ __forceinline__ void row_swap16(float &a, float &b) {
+  asm volatile("s_nop 7\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 7" : "+v"(a), "+v"(b));
 }
+__device__ __forceinline__ void row_swap32(float &a, float &b) {
+  asm volatile("s_nop 7\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 7" : "+v"(a), "+v"(b));
+}
+#define HQ_WAVE_REDUCE(OP_)                                              \
+  v = OP_(v, dpp_f<0xB1>(v));  /* quad_perm [1,0,3,2] */                \
+  v = OP_(v, dpp_f<0x4E>(v));  /* quad_perm [2,3,0,1] */                \
+  v = OP_(v, dpp_f<0x141>(v)); /* row_half_mirror     */                \
+  v = OP_(v, dpp_f<0x140>(v)); /* row_mirror          */                \
+  float o = v;                                                           \
+  row_swap16(v, o); /* rows 0 and 2: o = rows 1 and 3 */                 \
+  v = OP_(v, o);                                                         \
+  o = v;                                                                 \
+  row_swap32(v, o); /* row 0: o = row 2 */                               \
+  v = OP_(v, o);                                                         \
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+__device__ __forceinline__ float hq_add(float a, float b) { return a + b; }
+__device__ __forceinline__ float wave_sum(float v) { HQ_WAVE_REDUCE(hq_add) }
+__device__ __forceinline__ float wave_max(float v) { HQ_WAVE_REDUCE(fmaxf) }
+#undef HQ_WAVE_REDUCE
 
 // Buffer addressing: a 128-bit descriptor per (b, head) slab in scalar registers, a per-lane byte offset
 // that never changes, and the row offset in a scalar register -- no vector ALU work per load, and reads
