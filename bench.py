@@ -311,17 +311,30 @@ def main():
     elapsed = time_region(timed, sync)
     us_per_step = elapsed / K * 1e6
 
-    # per-kernel averages (HIP events on the launch stream), back-to-back over all layers
+    # per-kernel averages (HIP events on the launch stream), one kind of kernel back-to-back over all layers;
+    # replayed from a HIP graph (unless --no-graph) so that the host's launch rate does not show in the
+    # figure of a short kernel
     from hqekv_amd import _lib
     reps = 5
     fused = bool(plans[0].flags & _lib.FUSE_SOFTMAX)
-    qk_us = event_avg_us(lambda: [p.run(q, only=_lib.ONLY_QK) for p, q in zip(plans, qs)], n_layers, reps)
+
+    def part_us(launch_all):
+        if args.no_graph:
+            return event_avg_us(launch_all, n_layers, reps)
+        launch_all()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            launch_all()
+        return event_avg_us(g.replay, n_layers, reps)
+
+    qk_us = part_us(lambda: [p.run(q, only=_lib.ONLY_QK) for p, q in zip(plans, qs)])
     sm_us = 0.0
     if not fused:  # the general path has a softmax launch of its own; time it and take it out of the q.K^T figure
-        sm_us = event_avg_us(lambda: [p.run_softmax() for p in plans], n_layers, reps)
+        sm_us = part_us(lambda: [p.run_softmax() for p in plans])
         qk_us -= sm_us
-    pv_us = event_avg_us(lambda: [p.run(q, only=_lib.ONLY_PV) for p, q in zip(plans, qs)], n_layers, reps)
-    cb_us = event_avg_us(lambda: [p.run(q, only=_lib.ONLY_COMBINE) for p, q in zip(plans, qs)], n_layers, reps)
+    pv_us = part_us(lambda: [p.run(q, only=_lib.ONLY_PV) for p, q in zip(plans, qs)])
+    cb_us = part_us(lambda: [p.run(q, only=_lib.ONLY_COMBINE) for p, q in zip(plans, qs)])
     for p, q in zip(plans, qs):  # leave consistent outputs behind
         p.run(q)
     dominant = "qk_hybrid_kernel" if qk_us >= pv_us else "pv_hybrid_kernel"
