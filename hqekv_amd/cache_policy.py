@@ -15,12 +15,14 @@ survivors (quant/hqe_2.py:661-670).
 
 The reference re-copies whole class tensors with boolean masks; here a move gathers only the moved
 columns / rows with ``index_select`` and quantises them with one fused kernel (K straight from the
-token-major residual, no transpose copy).
+token-major residual, no transpose copy).  Which token goes where is worked out on host copies of the
+position arrays (numpy), so a compression waits for the device only to fetch the two block rankings.
 """
 from __future__ import annotations
 
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from . import pack_unpack as PU
@@ -34,31 +36,56 @@ _STRATEGIES = ("uniform", "normal", "uniform_group", "normal_group", "high_unifo
 
 
 class _Cls:
-    """One precision class of one side (K or V): data, positions, scale, zero."""
-    __slots__ = ("data", "idx", "scale", "zero")
+    """One precision class of one side (K or V): data, positions, scale, zero.
 
-    def __init__(self, data=None, idx=None, scale=None, zero=None):
-        self.data, self.idx, self.scale, self.zero = data, idx, scale, zero
+    ``idx_h`` is the host copy (numpy int64) of the positions; the bookkeeping of a compression -- which
+    tokens move where -- is done on it, so the device is only asked to gather rows / columns and to quantise.
+    ``idx`` (the device tensor the tuple carries) is None while the host copy is ahead of it."""
+    __slots__ = ("data", "idx", "scale", "zero", "idx_h")
+
+    def __init__(self, data=None, idx=None, scale=None, zero=None, idx_h=None):
+        self.data, self.idx, self.scale, self.zero, self.idx_h = data, idx, scale, zero, idx_h
 
     @property
     def empty(self) -> bool:
         return self.data is None
 
 
-def _read_side(pkv: tuple, slots: Dict[int, int]) -> Dict[int, _Cls]:
+def _host_idx(t: torch.Tensor) -> np.ndarray:
+    """Host copy of a position tensor.  Tensors made by this module carry theirs along (no device
+    round trip); for anyone else's the copy is fetched, which waits for the device."""
+    h = getattr(t, "_hq_host", None)
+    if h is None or h.shape[0] != t.numel():
+        h = t.detach().to("cpu", torch.int64).numpy()
+    return h
+
+
+def _to_dev(a: np.ndarray, dev) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(dev)
+
+
+def _dev_idx(h: np.ndarray, dev) -> torch.Tensor:
+    t = _to_dev(h, dev)
+    t._hq_host = h   # never modified afterwards
+    return t
+
+
+def _read_side(pkv: tuple, slots: Dict[int, int], host: bool = False) -> Dict[int, _Cls]:
     out = {}
     for b in CLASS_BITS:
         s = slots[b]
-        if b == 16:
-            out[b] = _Cls(pkv[s], pkv[s + 1])
-        else:
-            out[b] = _Cls(pkv[s], pkv[s + 1], pkv[s + 2], pkv[s + 3])
+        c = _Cls(pkv[s], pkv[s + 1]) if b == 16 else _Cls(pkv[s], pkv[s + 1], pkv[s + 2], pkv[s + 3])
+        if host and c.idx is not None:
+            c.idx_h = _host_idx(c.idx)
+        out[b] = c
     return out
 
 
-def _write_side(t: list, side: Dict[int, _Cls], slots: Dict[int, int]) -> None:
+def _write_side(t: list, side: Dict[int, _Cls], slots: Dict[int, int], dev=None) -> None:
     for b in CLASS_BITS:
         s, c = slots[b], side[b]
+        if c.data is not None and c.idx is None:
+            c.idx = _dev_idx(c.idx_h, dev)
         t[s], t[s + 1] = c.data, c.idx
         if b != 16:
             t[s + 2], t[s + 3] = c.scale, c.zero
@@ -66,6 +93,10 @@ def _write_side(t: list, side: Dict[int, _Cls], slots: Dict[int, int]) -> None:
 
 def _cat(a: Optional[torch.Tensor], b: torch.Tensor, dim: int) -> torch.Tensor:
     return b if a is None else torch.cat((a, b), dim=dim)
+
+
+def _cat_h(a: Optional[np.ndarray], b: np.ndarray) -> np.ndarray:
+    return b if a is None else np.concatenate((a, b))
 
 
 def _none_if_empty(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
@@ -97,26 +128,26 @@ def _check_low_bits(bits: int, strategy: str) -> None:
 # ----------------------------------------------------------------------------------------------- K side
 # K classes are channel-major (B, H, D, X): X = tokens (fp16), tokens/pf (codes), tokens/32 (scale, zero).
 
-def _group_columns(groups: torch.Tensor, per_group: int) -> torch.Tensor:
-    return (groups[:, None] * per_group + torch.arange(per_group, device=groups.device)[None, :]).reshape(-1)
-
-
-def _k_split(c: _Cls, bits: int, mask: torch.Tensor):
-    """-> (moved class, kept class); ``mask`` marks tokens of ``c`` and must cover whole 32-token groups."""
-    gm = mask.view(-1, BLOCK)
+def _k_split(c: _Cls, bits: int, mask: np.ndarray):
+    """-> (moved class, kept class); ``mask`` (host, bool) marks tokens of ``c`` and must cover whole
+    32-token groups."""
+    gm = mask.reshape(-1, BLOCK)
     if not bool((gm == gm[:, :1]).all()):
         raise ValueError("K classes move in whole 32-token groups: the selection splits a group")
     g_all = gm[:, 0]
-    sel, keep = g_all.nonzero().flatten(), (~g_all).nonzero().flatten()
+    sel, keep = np.flatnonzero(g_all), np.flatnonzero(~g_all)
     per = BLOCK if bits == 16 else BLOCK // (32 // bits)
+    dev = c.data.device
 
-    def part(groups: torch.Tensor, m: torch.Tensor) -> _Cls:
-        if groups.numel() == 0:
+    def part(groups: np.ndarray, m: np.ndarray) -> _Cls:
+        if groups.size == 0:
             return _Cls()
-        data = c.data.index_select(3, _group_columns(groups, per))
+        cols = (groups[:, None] * per + np.arange(per)[None, :]).reshape(-1)
+        data = c.data.index_select(3, _to_dev(cols, dev))
         if bits == 16:
-            return _Cls(data, c.idx[m])
-        return _Cls(data, c.idx[m], c.scale.index_select(3, groups), c.zero.index_select(3, groups))
+            return _Cls(data, idx_h=c.idx_h[m])
+        g_t = _to_dev(groups, dev)
+        return _Cls(data, None, c.scale.index_select(3, g_t), c.zero.index_select(3, g_t), c.idx_h[m])
 
     return part(sel, mask), part(keep, ~mask)
 
@@ -127,29 +158,31 @@ def _k_to_fp16(c: _Cls, bits: int, strategy: str = "uniform_group") -> torch.Ten
     return _dequantize(c, bits, strategy)
 
 
-def _k_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int, strategy: str = "uniform_group") -> None:
+def _k_append(dst: _Cls, x: torch.Tensor, idx_h: np.ndarray, bits: int, strategy: str = "uniform_group") -> None:
     """x is (B, H, D, n) fp16, possibly the transposed view of token-major memory."""
     if bits == 16:
         dst.data = _cat(dst.data, x, 3)
     else:
         code, scale, zero = _quantize(x, bits, strategy)
         dst.data, dst.scale, dst.zero = _cat(dst.data, code, 3), _cat(dst.scale, scale, 3), _cat(dst.zero, zero, 3)
-    dst.idx = _cat(dst.idx, idx, 0)
+    dst.idx_h, dst.idx = _cat_h(dst.idx_h, idx_h), None
 
 
 # ----------------------------------------------------------------------------------------------- V side
 # V classes are token-major (B, H, n, X): X = D (fp16), D/pf (codes), D/32 (scale, zero).
 
-def _v_split(c: _Cls, bits: int, mask: torch.Tensor):
-    sel, keep = mask.nonzero().flatten(), (~mask).nonzero().flatten()
+def _v_split(c: _Cls, bits: int, mask: np.ndarray):
+    sel, keep = np.flatnonzero(mask), np.flatnonzero(~mask)
+    dev = c.data.device
 
-    def part(rows: torch.Tensor) -> _Cls:
-        if rows.numel() == 0:
+    def part(rows: np.ndarray) -> _Cls:
+        if rows.size == 0:
             return _Cls()
+        r_t = _to_dev(rows, dev)
         if bits == 16:
-            return _Cls(c.data.index_select(2, rows), c.idx[rows])
-        return _Cls(c.data.index_select(2, rows), c.idx[rows], c.scale.index_select(2, rows),
-                    c.zero.index_select(2, rows))
+            return _Cls(c.data.index_select(2, r_t), idx_h=c.idx_h[rows])
+        return _Cls(c.data.index_select(2, r_t), None, c.scale.index_select(2, r_t),
+                    c.zero.index_select(2, r_t), c.idx_h[rows])
 
     return part(sel), part(keep)
 
@@ -160,77 +193,74 @@ def _v_to_fp16(c: _Cls, bits: int, strategy: str = "uniform_group") -> torch.Ten
     return _dequantize(c, bits, strategy)
 
 
-def _v_append(dst: _Cls, x: torch.Tensor, idx: torch.Tensor, bits: int, strategy: str = "uniform_group") -> None:
+def _v_append(dst: _Cls, x: torch.Tensor, idx_h: np.ndarray, bits: int, strategy: str = "uniform_group") -> None:
     if bits == 16:
         dst.data = _cat(dst.data, x, 2)
     else:
         code, scale, zero = _quantize(x, bits, strategy)
         dst.data, dst.scale, dst.zero = _cat(dst.data, code, 2), _cat(dst.scale, scale, 2), _cat(dst.zero, zero, 2)
-    dst.idx = _cat(dst.idx, idx, 0)
+    dst.idx_h, dst.idx = _cat_h(dst.idx_h, idx_h), None
 
 
 # ----------------------------------------------------------------------------------------------- engine
 
-def _targets(sorted_idx: torch.Tensor, bit_num: torch.Tensor) -> List[Optional[torch.Tensor]]:
-    """Slices of the ranked token list for (16, 8, 4, 2, 1[, evict]); None where a share is empty."""
+def _targets(sorted_idx: torch.Tensor, bit_num: torch.Tensor) -> List[Optional[np.ndarray]]:
+    """Slices (host) of the ranked token list for (16, 8, 4, 2, 1[, evict]); None where a share is empty."""
     cum = [0] + [int(v) for v in torch.cumsum(bit_num.to(torch.int64).cpu(), 0).tolist()]
-    return [sorted_idx[cum[i]:cum[i + 1]] if cum[i + 1] > cum[i] else None for i in range(len(cum) - 1)]
+    sorted_h = sorted_idx.detach().to("cpu", torch.int64).numpy()
+    return [sorted_h[cum[i]:cum[i + 1]] if cum[i + 1] > cum[i] else None for i in range(len(cum) - 1)]
 
 
-def _rerank(side: Dict[int, _Cls]) -> None:
+def _rerank(side: Dict[int, _Cls], total: int) -> None:
     """Survivors keep their order; each index becomes its rank among all survivors."""
-    parts = [side[b].idx for b in CLASS_BITS if side[b].idx is not None]
-    if not parts:
-        return
-    allv = torch.cat(parts)
-    order = torch.argsort(allv)
-    rank = torch.empty_like(order)
-    rank[order] = torch.arange(order.numel(), device=order.device, dtype=order.dtype)
-    start = 0
+    alive = np.zeros(total, dtype=np.int64)
     for b in CLASS_BITS:
-        if side[b].idx is not None:
-            n = side[b].idx.numel()
-            side[b].idx = rank[start:start + n].to(side[b].idx.dtype)
-            start += n
+        if side[b].idx_h is not None:
+            alive[side[b].idx_h] = 1
+    rank = np.cumsum(alive) - 1
+    for b in CLASS_BITS:
+        c = side[b]
+        if c.idx_h is not None:
+            c.idx_h, c.idx = rank[c.idx_h], None
 
 
-def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[torch.Tensor]], history: int,
+def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[np.ndarray]], history: int,
              is_k: bool, strategy: str, on_evict=None):
     """Run one compression on one side.  ``new`` is (B, H, n_new, D) fp16 (token-major for K and V alike)."""
     dev = new.device
-    new_idx = torch.arange(history, history + new.shape[2], device=dev, dtype=torch.int64)
+    total = history + new.shape[2]
+    new_idx = np.arange(history, total, dtype=np.int64)
     # membership of a position in a target set through one label per position (what the reference asks with
     # torch.isin per class, quant/hqe_2.py:552-659): label[p] = index of the target list that holds p
-    total = history + new.shape[2]
-    label = torch.full((total,), -1, dtype=torch.int8, device=dev)
+    label = np.full(total, -1, dtype=np.int8)
     for ti, tgt in enumerate(targets):
         if tgt is not None:
-            label[tgt.to(dev)] = ti
+            label[tgt] = ti
 
-    def member(idx: torch.Tensor, ti: int) -> torch.Tensor:
-        return label[idx] == ti
+    def member(idx_h: np.ndarray, ti: int) -> np.ndarray:
+        return label[idx_h] == ti
 
     split, to16, append = (_k_split, _k_to_fp16, _k_append) if is_k else (_v_split, _v_to_fp16, _v_append)
     evict = targets[5] if len(targets) > 5 else None
 
-    def take_new(mask: torch.Tensor) -> torch.Tensor:
+    def take_new(mask: np.ndarray) -> torch.Tensor:
         nonlocal new, new_idx
-        rows, keep = mask.nonzero().flatten(), (~mask).nonzero().flatten()
-        moved = new.index_select(2, rows)
-        new, new_idx = new.index_select(2, keep), new_idx[keep]
+        rows, keep = np.flatnonzero(mask), np.flatnonzero(~mask)
+        moved = new.index_select(2, _to_dev(rows, dev))
+        new, new_idx = new.index_select(2, _to_dev(keep, dev)), new_idx[keep]
         return moved
 
     # 1. eviction: dropped tokens leave every tensor
     if evict is not None:
         m = member(new_idx, 5)
-        if bool(m.any()):
+        if m.any():
             take_new(m)
         for b in CLASS_BITS:
             c = side[b]
-            if c.idx is None:
+            if c.idx_h is None:
                 continue
-            m = member(c.idx, 5)
-            if bool(m.any()):
+            m = member(c.idx_h, 5)
+            if m.any():
                 _, side[b] = split(c, b, m)
         if on_evict is not None:
             on_evict(side, new_idx)
@@ -240,9 +270,9 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
         tgt_bits, tgt_idx = CLASS_BITS[ti], targets[ti]
         if tgt_idx is None:
             continue
-        if new_idx.numel():
+        if new_idx.size:
             m = member(new_idx, ti)
-            if bool(m.any()):
+            if m.any():
                 if tgt_bits < 16:
                     _check_low_bits(tgt_bits, strategy)
                 sel_idx = new_idx[m]
@@ -252,17 +282,17 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[to
             if src_bits <= tgt_bits:
                 break
             c = side[src_bits]
-            if c.idx is None:
+            if c.idx_h is None:
                 continue
-            m = member(c.idx, ti)
-            if not bool(m.any()):
+            m = member(c.idx_h, ti)
+            if not m.any():
                 continue
             _check_low_bits(tgt_bits, strategy)
             moved, side[src_bits] = split(c, src_bits, m)
-            append(side[tgt_bits], to16(moved, src_bits, strategy), moved.idx, tgt_bits, strategy)
+            append(side[tgt_bits], to16(moved, src_bits, strategy), moved.idx_h, tgt_bits, strategy)
 
     if evict is not None:
-        _rerank(side)
+        _rerank(side, total)
     return new, new_idx
 
 
@@ -293,13 +323,14 @@ def compress(past_key_value: tuple, compress_length: int, history_length, K_sort
     V_score = token_importance * V_norm if times_range else token_importance.clone()
     V_sorted_idx = get_block_token_idx(BLOCK, block_num, V_score)
 
-    k_side, v_side = _read_side(pkv, K_SLOT), _read_side(pkv, V_SLOT)
+    dev = new_V.device
+    k_side, v_side = _read_side(pkv, K_SLOT, host=True), _read_side(pkv, V_SLOT, host=True)
     _migrate(k_side, new_K, _targets(K_sorted_idx, K_bit_num), history, True, quant_strategy)
 
     def after_v_eviction(side, new_idx):
         nonlocal V_norm
-        keep = [side[b].idx for b in CLASS_BITS if side[b].idx is not None] + [new_idx]
-        keep = torch.sort(torch.cat(keep))[0]
+        keep = [side[b].idx_h for b in CLASS_BITS if side[b].idx_h is not None] + [new_idx]
+        keep = _to_dev(np.sort(np.concatenate(keep)), dev)
         V_norm = V_norm[keep]
         if last_weights is not None:
             last_weights.eviction(keep)
@@ -308,8 +339,8 @@ def compress(past_key_value: tuple, compress_length: int, history_length, K_sort
              on_evict=after_v_eviction)
 
     t = list(pkv)
-    _write_side(t, k_side, K_SLOT)
-    _write_side(t, v_side, V_SLOT)
+    _write_side(t, k_side, K_SLOT, dev)
+    _write_side(t, v_side, V_SLOT, dev)
     t[38], t[39], t[40] = V_norm, res_K, res_V
     return tuple(t)
 
@@ -323,7 +354,7 @@ def reconstruct(past_key_value: tuple, quant_strategy: str, block_size: int = 32
     pkv = past_key_value
     k_side, v_side = _read_side(pkv, K_SLOT), _read_side(pkv, V_SLOT)
     new_K, new_V, T = pkv[39], pkv[40], int(pkv[41])
-    some = next((x for x in (v_side[16].data, v_side[8].data, v_side[4].data, v_side[2].data, new_V) if x is not None), None)
+    some = next((x for x in (v_side[16].data, v_side[8].data, v_side[4].data, v_side[2].data, v_side[1].data, new_V) if x is not None), None)
     if some is None:
         raise ValueError('invalid past_key_value')
     B, H, dev = some.shape[0], some.shape[1], some.device
