@@ -47,7 +47,7 @@ struct SegTable {
   int32_t total_units;
   int32_t max_units;   // the largest n_units of any segment
   int32_t pad_;
-  int32_t begin[HQEKV_MAX_SEGS];  // unit_begin of every segment (INT32_MAX past nseg): one scalar load finds a unit's segment
+  int32_t begin[HQEKV_MAX_SEGS];  // first grid.y index of every segment (INT32_MAX past nseg): one scalar load finds a workgroup's segment
 };
 
 // grid.y enumerates the units of all segments back to back (no idle workgroups): unit u belongs to the last
@@ -57,6 +57,13 @@ __device__ __forceinline__ int seg_of_unit(const SegTable &tb, int u) {
 #pragma unroll
   for (int k = 0; k < HQEKV_MAX_SEGS; ++k) s += (u >= tb.begin[k]) ? 1 : 0;
   return s;
+}
+// begin[s] without a second, dependent load from the argument segment
+__device__ __forceinline__ int begin_of_seg(const SegTable &tb, int s) {
+  int b = 0;
+#pragma unroll
+  for (int k = 0; k < HQEKV_MAX_SEGS; ++k) b += (k == s) ? tb.begin[k] : 0;
+  return b;
 }
 
 // Optional fusion of the softmax into the two GEMV launches (valid when no mask is added and the K
@@ -492,7 +499,7 @@ struct QkReduce {
 template <int NREP, int QK_WAVES>
 __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
                                                                half_t *__restrict__ scores, int Hq,
-                                                               int Hkv, int D, int64_t Tall, FuseArgs fz) {
+                                                               int Hkv, int D, int64_t Tall, FuseArgs fz, int tpw) {
   using R = QkReduce<NREP, QK_WAVES>;
   constexpr int RH = R::RH, VPT = R::VPT, WPH = R::WPH;
   extern __shared__ float smem[];
@@ -502,130 +509,154 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int bh = blockIdx.x;
   const int b = bh / Hkv, hkv = bh % Hkv;
-  const SegDev sg = tb.seg[seg_of_unit(tb, blockIdx.y)];  // by value: one batch of scalar loads, no lazy re-reads
-  const int tile = (int)blockIdx.y - sg.unit_begin;
+  // grid.y counts workgroups; a workgroup takes `tpw` consecutive tiles of one class (1 unless the
+  // environment asks for more: longer-lived workgroups stage the query once, but measured no faster)
+  const int si = seg_of_unit(tb, blockIdx.y);
+  const SegDev sg = tb.seg[si];  // by value: one batch of scalar loads, no lazy re-reads
+  const int tile_begin = ((int)blockIdx.y - begin_of_seg(tb, si)) * tpw;
+  const int tile_end = min(tile_begin + tpw, (int)sg.n_units);
   const bool tm = sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR;
   const uint32_t n = (uint32_t)sg.n_tokens;
-  const uint32_t t0 = (uint32_t)tile * QK_TILE + lane * QK_TPL;
-  const uint32_t ts = t0 < n ? t0 : 0;  // lanes past the end recompute token 0 and store nothing
-  // the VPT values this thread reduces and stores in every pass: head hl of the pass, tokens tok .. tok+VPT-1
-  const int hl = (int)(threadIdx.x * VPT) / QK_TILE;
-  const uint32_t tok = (uint32_t)tile * QK_TILE + (threadIdx.x * VPT) % QK_TILE;
-  // their positions: requested first (branch-free, so the loads overlap), used last.  Positions are below
-  // 2^31 (they index a row of Tall fp16 scores), so the low word of each int64 index is enough.
-  uint32_t pos[VPT];
-  {
-    const uint32_t *ip = reinterpret_cast<const uint32_t *>(sg.idx);
-    const bool has_idx = ip != nullptr;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const uint32_t t = min(tok + i, n - 1);
-      pos[i] = (uint32_t)sg.pos_base + t;
-      if (has_idx) pos[i] = ip[2 * t];
-    }
-  }
   const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * D);
+  // The query is staged by the first tile only; for every tile the call is the workgroup barrier between
+  // "first loads requested" and "arithmetic starts", and between two tiles' uses of the reduction buffer.
+  bool staged = false;
   auto stage_q = [&]() {
-    for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_WAVES * 64) {
-      const int h = k / (D >> 1), dp = k % (D >> 1);
-      q2s[dp * NREP + h] = as_h2(qsrc[k]);  // [dp][h]: one 16-byte LDS read fetches a row pair for 4 heads
+    if (!staged) {
+      for (int k = threadIdx.x; k < NREP * (D >> 1); k += QK_WAVES * 64) {
+        const int h = k / (D >> 1), dp = k % (D >> 1);
+        q2s[dp * NREP + h] = as_h2(qsrc[k]);  // [dp][h]: one 16-byte LDS read fetches a row pair for 4 heads
+      }
+      staged = true;
     }
     __syncthreads();
   };
   if (tm) {
-    stage_q();
-    qk_f16_tm_tile<NREP, QK_WAVES>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
+#pragma unroll 1
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+      stage_q();
+      qk_f16_tm_tile<NREP, QK_WAVES>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
+    }
     return;
   }
 
-  float acc[NREP][QK_TPL];
+  // The tile loop lives inside each class's branch (instantiated once per class by the generic lambda), so
+  // what a class keeps in registers across tiles is its own and not the union over all classes.
+  auto run_tiles = [&](auto accumulate) {
+#pragma unroll 1
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+      const uint32_t t0 = (uint32_t)tile * QK_TILE + lane * QK_TPL;
+      const uint32_t ts = t0 < n ? t0 : 0;  // lanes past the end recompute token 0 and store nothing
+      // the VPT values this thread reduces and stores in every pass: head hl of the pass, tokens tok .. tok+VPT-1
+      const int hl = (int)(threadIdx.x * VPT) / QK_TILE;
+      const uint32_t tok = (uint32_t)tile * QK_TILE + (threadIdx.x * VPT) % QK_TILE;
+      // their positions: requested first (branch-free, so the loads overlap), used last.  Positions are below
+      // 2^31 (they index a row of Tall fp16 scores), so the low word of each int64 index is enough.
+      uint32_t pos[VPT];
+      {
+        const uint32_t *ip = reinterpret_cast<const uint32_t *>(sg.idx);
+        const bool has_idx = ip != nullptr;
 #pragma unroll
-  for (int h = 0; h < NREP; ++h)
+        for (int i = 0; i < VPT; ++i) {
+          const uint32_t t = min(tok + i, n - 1);
+          pos[i] = (uint32_t)sg.pos_base + t;
+          if (has_idx) pos[i] = ip[2 * t];
+        }
+      }
+      float acc[NREP][QK_TPL];
 #pragma unroll
-    for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
+      for (int h = 0; h < NREP; ++h)
+#pragma unroll
+        for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
+      accumulate(ts, t0, acc);
+
+      // Cross-wave reduction, RH heads per pass.  Every wave parks its partial rows (token-contiguous, two
+      // 128-bit LDS writes per head); then ALL threads share the summation: a thread adds the QK_WAVES
+      // partials of VPT adjacent tokens of one head (one vector LDS read per partial, conflict-free), rounds,
+      // and stores them, so a wave writes 128 * VPT contiguous bytes of a score row.
+      bool contig = (tok + VPT <= n);
+#pragma unroll
+      for (int i = 1; i < VPT; ++i) contig = contig && (pos[i] == pos[0] + i);
+#pragma unroll
+      for (int h0 = 0; h0 < NREP; h0 += RH) {
+        if (h0 > 0) __syncthreads();
+#pragma unroll
+        for (int j = 0; j < RH; ++j) {
+          float4 *dst = reinterpret_cast<float4 *>(red + (wave * RH + j) * QK_TILE + lane * QK_TPL);
+          dst[0] = make_float4(acc[h0 + j][0], acc[h0 + j][1], acc[h0 + j][2], acc[h0 + j][3]);
+          dst[1] = make_float4(acc[h0 + j][4], acc[h0 + j][5], acc[h0 + j][6], acc[h0 + j][7]);
+        }
+        __syncthreads();
+        const int h = h0 + hl;
+        float a[VPT];
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) a[i] = 0.f;
+#pragma unroll
+        for (int w = 0; w < QK_WAVES; ++w) {
+          float part[VPT];
+          __builtin_memcpy(part, red + (w * RH + hl) * QK_TILE + (threadIdx.x * VPT) % QK_TILE, VPT * 4);
+#pragma unroll
+          for (int i = 0; i < VPT; ++i) a[i] += part[i];
+        }
+        half_t v[VPT];
+        float m_lane = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+          v[i] = (half_t)a[i];
+          if (fz.stats) {  // the fp16 steps of the reference epilogue: round the score, scale, round again
+            v[i] = (half_t)((float)v[i] * fz.inv_sqrt_d);
+            if (tok + i < n) m_lane = fmaxf(m_lane, (float)v[i]);
+          }
+        }
+        if (fz.stats) {  // (max, sum exp) of this wave's 64 * VPT tokens; merged per head after the last pass
+          const float m = wave_max(m_lane);
+          float l_lane = 0.f;
+#pragma unroll
+          for (int i = 0; i < VPT; ++i)
+            if (tok + i < n) l_lane += __expf((float)v[i] - m);
+          const float l = wave_sum(l_lane);
+          if (lane == 0) wave_ml[h][wave - hl * WPH] = make_float2(m, l);
+        }
+        if (tok < n) {
+          half_t *srow = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+          // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
+          // vector store; otherwise 2-byte scatters through idx
+          if (contig && (((uintptr_t)(srow + pos[0])) & (VPT * 2 - 1)) == 0) {
+            __builtin_memcpy(__builtin_assume_aligned(srow + pos[0], VPT * 2), v, VPT * 2);
+          } else {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+              if (tok + i < n) srow[pos[i]] = v[i];
+          }
+        }
+      }
+      if (fz.stats) {
+        __syncthreads();
+        if (threadIdx.x < NREP) {
+          const int h = threadIdx.x;
+          float m = -INFINITY, l = 0.f;
+#pragma unroll
+          for (int w = 0; w < WPH; ++w) m = fmaxf(m, wave_ml[h][w].x);
+#pragma unroll
+          for (int w = 0; w < WPH; ++w)
+            if (wave_ml[h][w].y > 0.f) l += wave_ml[h][w].y * __expf(wave_ml[h][w].x - m);
+          fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+        }
+      }
+    }
+  };
+  using Acc = float (&)[NREP][QK_TPL];
   switch (sg.bits) {
     case 1:
-      if (sg.layout == HQEKV_LAYOUT_NORMAL1) qk_quant_accumulate<1, NREP, QK_WAVES, true>(sg, ts, bh, D, wave, stage_q, q2s, acc);
-      else qk_quant_accumulate<1, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc);
+      if (sg.layout == HQEKV_LAYOUT_NORMAL1)
+        run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<1, NREP, QK_WAVES, true>(sg, ts, bh, D, wave, stage_q, q2s, acc); });
+      else
+        run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<1, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); });
       break;
-    case 2: qk_quant_accumulate<2, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
-    case 4: qk_quant_accumulate<4, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
-    case 8: qk_quant_accumulate<8, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); break;
-    default: qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, stage_q, q2s, acc);
-  }
-
-  // Cross-wave reduction, RH heads per pass.  Every wave parks its partial rows (token-contiguous, two
-  // 128-bit LDS writes per head); then ALL threads share the summation: a thread adds the QK_WAVES partials
-  // of VPT adjacent tokens of one head (one vector LDS read per partial, conflict-free), rounds, and stores
-  // them, so a wave writes 128 * VPT contiguous bytes of a score row.
-  bool contig = (tok + VPT <= n);
-#pragma unroll
-  for (int i = 1; i < VPT; ++i) contig = contig && (pos[i] == pos[0] + i);
-#pragma unroll
-  for (int h0 = 0; h0 < NREP; h0 += RH) {
-    if (h0 > 0) __syncthreads();
-#pragma unroll
-    for (int j = 0; j < RH; ++j) {
-      float4 *dst = reinterpret_cast<float4 *>(red + (wave * RH + j) * QK_TILE + lane * QK_TPL);
-      dst[0] = make_float4(acc[h0 + j][0], acc[h0 + j][1], acc[h0 + j][2], acc[h0 + j][3]);
-      dst[1] = make_float4(acc[h0 + j][4], acc[h0 + j][5], acc[h0 + j][6], acc[h0 + j][7]);
-    }
-    __syncthreads();
-    const int h = h0 + hl;
-    float a[VPT];
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) a[i] = 0.f;
-#pragma unroll
-    for (int w = 0; w < QK_WAVES; ++w) {
-      float part[VPT];
-      __builtin_memcpy(part, red + (w * RH + hl) * QK_TILE + (threadIdx.x * VPT) % QK_TILE, VPT * 4);
-#pragma unroll
-      for (int i = 0; i < VPT; ++i) a[i] += part[i];
-    }
-    half_t v[VPT];
-    float m_lane = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      v[i] = (half_t)a[i];
-      if (fz.stats) {  // the fp16 steps of the reference epilogue: round the score, scale, round again
-        v[i] = (half_t)((float)v[i] * fz.inv_sqrt_d);
-        if (tok + i < n) m_lane = fmaxf(m_lane, (float)v[i]);
-      }
-    }
-    if (fz.stats) {  // (max, sum exp) of this wave's 64 * VPT tokens; merged per head after the last pass
-      const float m = wave_max(m_lane);
-      float l_lane = 0.f;
-#pragma unroll
-      for (int i = 0; i < VPT; ++i)
-        if (tok + i < n) l_lane += __expf((float)v[i] - m);
-      const float l = wave_sum(l_lane);
-      if (lane == 0) wave_ml[h][wave - hl * WPH] = make_float2(m, l);
-    }
-    if (tok < n) {
-      half_t *srow = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
-      // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
-      // vector store; otherwise 2-byte scatters through idx
-      if (contig && (((uintptr_t)(srow + pos[0])) & (VPT * 2 - 1)) == 0) {
-        __builtin_memcpy(__builtin_assume_aligned(srow + pos[0], VPT * 2), v, VPT * 2);
-      } else {
-#pragma unroll
-        for (int i = 0; i < VPT; ++i)
-          if (tok + i < n) srow[pos[i]] = v[i];
-      }
-    }
-  }
-  if (fz.stats) {
-    __syncthreads();
-    if (threadIdx.x < NREP) {
-      const int h = threadIdx.x;
-      float m = -INFINITY, l = 0.f;
-#pragma unroll
-      for (int w = 0; w < WPH; ++w) m = fmaxf(m, wave_ml[h][w].x);
-#pragma unroll
-      for (int w = 0; w < WPH; ++w)
-        if (wave_ml[h][w].y > 0.f) l += wave_ml[h][w].y * __expf(wave_ml[h][w].x - m);
-      fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
-    }
+    case 2: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<2, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
+    case 4: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<4, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
+    case 8: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<8, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
+    default: run_tiles([&](uint32_t, uint32_t t0, Acc acc) { qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, stage_q, q2s, acc); });
   }
 }
 
@@ -1163,12 +1194,22 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
   // few tiles: 8 waves per tile; many tiles (several workgroups queue up per CU): 4 waves per tile
   static const char *force = getenv("HQEKV_QK_WAVES");
   const int waves = force ? atoi(force) : ((int64_t)tb.total_units * B * Hkv <= 1024 ? 8 : 4);
-  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units), block((unsigned)waves * 64);
+  static const char *force_tpw = getenv("HQEKV_QK_TPW");
+  const int64_t wgs = (int64_t)tb.total_units * B * Hkv;
+  (void)wgs;  // measured at B=8, 64k context: 1, 2 and 4 tiles per workgroup take 121, 121 and 128 us -- one it is
+  const int tpw = force_tpw ? (atoi(force_tpw) > 0 ? atoi(force_tpw) : 1) : 1;
+  SegTable tw = tb;  // grid.y in workgroups: ceil(tiles / tpw) per class
+  int64_t ny = 0;
+  for (int k = 0; k < HQEKV_MAX_SEGS; ++k) {
+    tw.begin[k] = k < tb.nseg ? (int32_t)ny : 0x7fffffff;
+    if (k < tb.nseg) ny += (tb.seg[k].n_units + tpw - 1) / tpw;
+  }
+  dim3 grid((unsigned)(B * Hkv), (unsigned)ny), block((unsigned)waves * 64);
   const int rh = waves == 4 ? (nrep < 4 ? nrep : 4) : (nrep < 2 ? nrep : 2);  // QkReduce::RH
   const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
 #define LAUNCH(N_, W_)                                                                                        \
-  hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
-                     (int)Hq, (int)Hkv, (int)D, Tall, fz)
+  hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_>), grid, block, shmem, st, tw, (const half_t *)q, (half_t *)scores, \
+                     (int)Hq, (int)Hkv, (int)D, Tall, fz, tpw)
 #define LAUNCH_W(N_) \
   if (waves == 8) LAUNCH(N_, 8); else LAUNCH(N_, 4)
   switch (nrep) {
