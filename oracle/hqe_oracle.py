@@ -18,12 +18,20 @@ Pinned:
                                                 mat-vec / torch.matmul
   qkv_matmul                                    permutation invariance against dense attention
   compress_cache / rerank_after_eviction        brute force against a per-block history model and Python sets
+  1-bit uniform class (bit == 1 above)          arange known answer (scale 31, words 0xFFFF0000), tie -> even code
+  normal_group_(de)quantize (1-bit table)       arange(32) known answer worked out with numpy float16, unbiased
+                                                std / mean against float64, code == sign of x - mean
+  DecodeLayerOracle / ImportanceRing            bookkeeping invariants over a prompt and 40 decode steps (every
+                                                token in one class, the residual or evicted; class sizes follow
+                                                the ratio schedule; two blocks stay fp16)
 
 Parity unpinned (no reference fixture exists and only a run of the original GPU stack
 could pin it): the last-bit behaviour of ``fp16_tensor / python_int`` on the GPU, which
 ATen evaluates as multiply-by-reciprocal.  ``scalar_div='recip'`` restates that rule,
 ``scalar_div='true'`` is the CPU rule; the GPU test-suite checks the HIP kernels against
-torch's own on-device op chain to close the gap.
+torch's own on-device op chain to close the gap.  Also unpinned: the accumulation order of
+``torch.std_mean`` (last fp16 place of std / mean of the normal-quantile class) and the order of equal
+scores in ``torch.sort`` (block ranking; restated with a stable sort).
 """
 from __future__ import annotations
 
