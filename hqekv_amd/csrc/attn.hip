@@ -1105,7 +1105,7 @@ __global__ __launch_bounds__(CB_CH * CB_SLICES) void pv_combine_kernel(const flo
 #pragma unroll
     for (int k = 0; k < 4; ++k) v += t[k];
   }
-  v += xor_f(v, 32);  // the wave's two slices
+  v += xor_f(v, 32);  // the wave's two slices (once per thread)
   if ((threadIdx.x & 63) < CB_CH) sh[threadIdx.x >> 6][d] = v;
   __syncthreads();
   if (threadIdx.x < CB_CH && in) {

@@ -26,7 +26,18 @@ __device__ __forceinline__ uint32_t code_at(uint32_t w, int i) {
   return __builtin_amdgcn_ubfe(w, (uint32_t)(i * BITS), (uint32_t)BITS);
 }
 
-// butterfly exchange across the 64-lane wavefront
+// exchange with the lane 1 or 2 apart inside a quad: one DPP move, no trip through the LDS crossbar
+template <int M>
+__device__ __forceinline__ uint32_t quad_xor_u(uint32_t v) {
+  static_assert(M == 1 || M == 2, "quad permutes reach the lanes 1 and 2 apart");
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, M == 1 ? 0xB1 : 0x4E, 0xf, 0xf, true);
+}
+template <int M>
+__device__ __forceinline__ float quad_xor_f(float v) {
+  return __builtin_bit_cast(float, quad_xor_u<M>(__builtin_bit_cast(uint32_t, v)));
+}
+
+// butterfly exchange across the 64-lane wavefront (through the LDS crossbar: keep it off hot paths)
 __device__ __forceinline__ float xor_f(float v, int m) { return __shfl_xor(v, m, HQ_WAVE); }
 __device__ __forceinline__ uint32_t xor_u(uint32_t v, int m) {
   return (uint32_t)__shfl_xor((int)v, m, HQ_WAVE);

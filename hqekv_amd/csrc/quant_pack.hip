@@ -105,8 +105,8 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(
   half2_t hi2 = __builtin_elementwise_max(__builtin_elementwise_max(p[0], p[1]), __builtin_elementwise_max(p[2], p[3]));
   // (min, -max) in one register: one packed min per butterfly step serves both
   half2_t mm = {(half_t)__builtin_fminf((float)lo2[0], (float)lo2[1]), (half_t)(-__builtin_fmaxf((float)hi2[0], (float)hi2[1]))};
-  mm = __builtin_elementwise_min(mm, bits_h2(xor_u(h2_bits(mm), 1)));
-  mm = __builtin_elementwise_min(mm, bits_h2(xor_u(h2_bits(mm), 2)));
+  mm = __builtin_elementwise_min(mm, bits_h2(quad_xor_u<1>(h2_bits(mm))));
+  mm = __builtin_elementwise_min(mm, bits_h2(quad_xor_u<2>(h2_bits(mm))));
   const half_t mn_h = mm[0];
   const float mn = (float)mn_h, mx = -(float)mm[1];
 
@@ -141,13 +141,13 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(
     } else if (BITS == 1) {
       const uint32_t w = horner_pack<1, 4>(z);             // codes 0-3 in bits 0-3, codes 4-7 in bits 16-19
       const uint32_t b8 = (w & 0xfu) | ((w >> 12) & 0xf0u);  // this lane's 8 codes
-      const uint32_t b16 = b8 | (xor_u(b8, 1) << 8);        // even lanes: two lanes' codes in order
-      const uint32_t other = xor_u(b16, 2);
+      const uint32_t b16 = b8 | (quad_xor_u<1>(b8) << 8);        // even lanes: two lanes' codes in order
+      const uint32_t other = quad_xor_u<2>(b16);
       if (sub == 0) crow[0] = b16 | (other << 16);
     } else {
       const uint32_t w = horner_pack<2, 4>(z);             // codes 0-3 in byte 0, codes 4-7 in byte 2
       const uint32_t h = __builtin_amdgcn_perm(0u, w, 0x0c0c0200u);   // 16 bits: this lane's 8 codes
-      const uint32_t other = xor_u(h, 1);
+      const uint32_t other = quad_xor_u<1>(h);
       if ((sub & 1) == 0) crow[sub >> 1] = h | (other << 16);
     }
   }
@@ -282,8 +282,8 @@ __global__ __launch_bounds__(256) void normal1_rows_kernel(
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) sum += (float)v[i];
-  sum += xor_f(sum, 1);
-  sum += xor_f(sum, 2);
+  sum += quad_xor_f<1>(sum);
+  sum += quad_xor_f<2>(sum);
   const float mean_f = sum * (1.0f / 32.0f);
   float m2 = 0.f;
 #pragma unroll
@@ -291,14 +291,14 @@ __global__ __launch_bounds__(256) void normal1_rows_kernel(
     const float d = (float)v[i] - mean_f;
     m2 += d * d;
   }
-  m2 += xor_f(m2, 1);
-  m2 += xor_f(m2, 2);
+  m2 += quad_xor_f<1>(m2);
+  m2 += quad_xor_f<2>(m2);
   const Normal1Stats st = normal1_finish(sum, m2);
   uint32_t b8 = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) b8 |= normal1_code((half_t)((float)v[i] - (float)st.mean_h), st.thr) << i;
-  const uint32_t b16 = b8 | (xor_u(b8, 1) << 8);
-  const uint32_t other = xor_u(b16, 2);
+  const uint32_t b16 = b8 | (quad_xor_u<1>(b8) << 8);
+  const uint32_t other = quad_xor_u<2>(b16);
   if (sub == 0) {
     code[(int64_t)o * co + (int64_t)r * cr + g] = b16 | (other << 16);
     stdv[(int64_t)o * so + (int64_t)r * sr + g] = st.std_h;
