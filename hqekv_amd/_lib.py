@@ -27,7 +27,7 @@ LAYOUT_NORMAL1 = 2       # 1-bit segment in normal-quantile coding (scale = std,
 EXPORTS = (
     "hqekv_version", "hqekv_last_error",
     "hqekv_quant_pack_rows", "hqekv_quant_pack_k_tokenmajor", "hqekv_dequant_unpack_rows", "hqekv_pack_i32",
-    "hqekv_selftest_quant_division",
+    "hqekv_selftest_quant_division", "hqekv_selftest_wave_reduce",
     "hqekv_normal1_quant_pack_rows", "hqekv_normal1_quant_pack_k_tokenmajor", "hqekv_normal1_dequant_unpack_rows",
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
@@ -62,6 +62,7 @@ _PROTOS = {
     "hqekv_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "hqekv_pack_i32": (C.c_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "hqekv_selftest_quant_division": (C.c_int, [_vp, _vp]),
+    "hqekv_selftest_wave_reduce": (C.c_int, [_vp, _vp, _i64, _vp]),
     "hqekv_normal1_quant_pack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "hqekv_normal1_quant_pack_k_tokenmajor": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "hqekv_normal1_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),

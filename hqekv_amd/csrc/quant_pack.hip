@@ -589,6 +589,37 @@ extern "C" int hqekv_normal1_dequant_unpack_rows(const void *code, int64_t co, i
   return check_launch("dequant_rows_kernel");
 }
 
+// Every wave reduces its 64 inputs with the DPP / lane-row-swap reductions the attention kernels use and
+// with the plain shuffle butterfly; out holds (sum, max, butterfly sum, butterfly max) per wave.
+__global__ __launch_bounds__(256) void selftest_wave_reduce_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                                   int n_waves) {
+  const int w = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (w >= n_waves) return;  // whole waves leave together
+  const float v = in[(int64_t)w * 64 + lane];
+  const float s = wave_sum(v), m = wave_max(v);
+  float bs = v, bm = v;
+#pragma unroll
+  for (int k = 32; k >= 1; k >>= 1) {
+    bs += xor_f(bs, k);
+    bm = fmaxf(bm, xor_f(bm, k));
+  }
+  if (lane == 0) {
+    out[w * 4 + 0] = s;
+    out[w * 4 + 1] = m;
+    out[w * 4 + 2] = bs;
+    out[w * 4 + 3] = bm;
+  }
+}
+
+extern "C" int hqekv_selftest_wave_reduce(const void *in, void *out, int64_t n_waves, void *stream) {
+  if (n_waves < 0 || n_waves > 0x7fffffffLL) return fail(HQEKV_E_ARG, "selftest_wave_reduce: bad n_waves");
+  if (n_waves == 0) return HQEKV_OK;
+  if (!in || !out) return fail(HQEKV_E_ARG, "selftest_wave_reduce: null pointer");
+  hipLaunchKernelGGL(selftest_wave_reduce_kernel, dim3((unsigned)((n_waves + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                     (const float *)in, (float *)out, (int)n_waves);
+  return check_launch("selftest_wave_reduce_kernel");
+}
+
 extern "C" int hqekv_selftest_quant_division(void *counts, void *stream) {
   if (!counts) return fail(HQEKV_E_ARG, "selftest_quant_division: null pointer");
   if ((uintptr_t)counts & 7) return fail(HQEKV_E_ALIGN, "selftest_quant_division: counts must be 8-byte aligned");

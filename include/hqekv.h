@@ -113,6 +113,12 @@ int hqekv_normal1_dequant_unpack_rows(const void *code, int64_t code_outer_strid
  */
 int hqekv_selftest_quant_division(void *counts, void *stream);
 
+/* No counterpart in the reference: checks the wave-wide reductions the attention kernels are built on
+ * (DPP steps inside a row of 16 lanes, lane-row swaps across rows) on caller-supplied data.
+ * in: (n_waves, 64) fp32; out: (n_waves, 4) fp32 = sum, max, and the same two through plain shuffles.
+ */
+int hqekv_selftest_wave_reduce(const void *in, void *out, int64_t n_waves, void *stream);
+
 /* Replaces pack_along_last_dim (quant/pack_unpack.py:16-70): q is (n_rows, L) int32 codes,
  * code is (n_rows, L/pf) int32, both contiguous. */
 int hqekv_pack_i32(const void *q, void *code, int64_t n_rows, int64_t L, int bits, void *stream);

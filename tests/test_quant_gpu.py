@@ -255,3 +255,21 @@ def test_normal1_dequantiser_bit_exact_and_edges(dev):
     assert torch.equal(m.cpu().view(torch.int16), om.view(torch.int16))
     with pytest.raises(NotImplementedError):
         P.normal_group_quantize_pack_last_dim(x.to(dev), 32, 2)
+
+
+def test_wave_reductions_on_integer_data(dev):
+    """The DPP / lane-row-swap reductions of the attention kernels: exact on integer-valued inputs, for
+    every position of the maximum and with negative values, and equal to the plain shuffle butterfly."""
+    from hqekv_amd import _lib
+    g = torch.Generator().manual_seed(9)
+    n_waves = 4096 + 3
+    x = torch.randint(-1000, 1000, (n_waves, 64), generator=g).float()
+    x[:64] = -5.0
+    x[torch.arange(64), torch.arange(64)] = 7.0          # the maximum visits every lane
+    out = torch.empty(n_waves, 4, dtype=torch.float32, device=dev)
+    xd = x.to(dev)
+    _lib.check(_lib.load().hqekv_selftest_wave_reduce(xd.data_ptr(), out.data_ptr(), n_waves, _lib.stream_ptr(xd.device)),
+               "selftest_wave_reduce")
+    o = out.cpu()
+    assert torch.equal(o[:, 0], x.sum(1)) and torch.equal(o[:, 1], x.max(1)[0])
+    assert torch.equal(o[:, 2], o[:, 0]) and torch.equal(o[:, 3], o[:, 1])
