@@ -44,6 +44,18 @@ def test_argument_validation_without_a_gpu():
     assert rc == -1  # Hq % Hkv
     rc = lib.hqekv_qk_hybrid(None, 0, None, None, 1, 12, 4, 128, 10, None)
     assert rc == -4  # GQA group of 3 unsupported
+    rc = lib.hqekv_normal1_quant_pack_rows(None, 0, 0, None, 0, 0, None, None, 0, 0, 1, 1, 48, None)
+    assert rc == -1 and b"multiple of 32" in lib.hqekv_last_error()
+    rc = lib.hqekv_normal1_quant_pack_k_tokenmajor(None, 0, 0, None, 0, 0, None, None, 0, 0, 1, 64, 127, None)
+    assert rc == -1
+    rc = lib.hqekv_normal1_dequant_unpack_rows(None, 0, 0, None, None, 0, 0, None, 0, 0, 1, 1, 64, None)
+    assert rc == -1 and b"null" in lib.hqekv_last_error()
+    assert lib.hqekv_selftest_wave_reduce(None, None, 4, None) == -1
+    assert lib.hqekv_selftest_quant_division(None, None) == -1
+    # a segment table with an unknown bit width
+    segs = _lib.make_segs([dict(bits=3, n_tokens=32, data=None)])
+    segs[0].data = 16
+    assert lib.hqekv_qk_hybrid(segs, 1, None, None, 1, 4, 4, 128, 32, None) == -1
     with pytest.raises(ValueError):
         _lib.check(-1, "x")
     with pytest.raises(RuntimeError):
