@@ -11,7 +11,7 @@ import importlib
 import sys
 import types
 
-_MODULES = ("pack_unpack", "matmul", "quant_matmul_hq", "hqe_matmul", "hybrid_quant", "hqe_2")
+_MODULES = ("pack_unpack", "matmul", "quant_matmul_hq", "hqe_matmul", "hybrid_quant", "hqe_2", "hqe")
 
 
 def install(force: bool = False) -> None:

@@ -26,3 +26,13 @@ def qkv_matmul_hqe_2(q: torch.Tensor, past_key_value: Tuple, attention_mask, hea
         raise ValueError('invalid past_key_value')
     return decode_attention(q, past_key_value, None, real_len, zero_init=False,
                             low_uniform=quant_strategy == "uniform_group")
+
+
+def qkv_matmul_hqe(q: torch.Tensor, past_key_value: Tuple, attention_mask, head_dim: int,
+                   quant_strategy: str, block_size: int = 32, group_size: int = 32):
+    """Signature of quant/hqe_matmul.py:27-35: attention over a cache whose K is quantised per token
+    (the generation written by ``quant/hqe.py``).  The model files import the name
+    (model/llama_hqe.py:25) and call ``qkv_matmul_hqe_2`` only; it resolves here and is not built."""
+    raise NotImplementedError(
+        "qkv_matmul_hqe (per-token K, quant/hqe_matmul.py:27) belongs to the superseded cache generation; "
+        "use qkv_matmul_hqe_2")

@@ -72,8 +72,14 @@ def test_reference_import_names_resolve():
         compat.install(force=True)
         from pack_unpack import uniform_group_quantize_pack_last_dim  # noqa: F401
         from matmul import cuda_bmm_fA_qB_uniform_group, cuda_bmm_forward_qk_group_hq  # noqa: F401
-        from quant.hqe_matmul import qkv_matmul_hqe_2  # noqa: F401
+        # the three import lines of the model files (model/llama_hqe.py:23-25), verbatim
+        from quant.hqe import KV_cache_hqe
         from quant.hqe_2 import KV_cache_hqe_2  # noqa: F401
+        from quant.hqe_matmul import qkv_matmul_hqe, qkv_matmul_hqe_2  # noqa: F401
+        with pytest.raises(NotImplementedError):  # imported there, never called: the per-token-K generation
+            KV_cache_hqe((None,) * 42, 32, 0, None, None, None, None, "uniform_group")
+        with pytest.raises(NotImplementedError):
+            qkv_matmul_hqe(None, (None,) * 42, None, 128, "high_uniform_group_low_normal_group")
         from quant.quant_matmul_hq import qkv_matmul, qkv_matmul_hq  # noqa: F401
         from quant.hybrid_quant import KV_cache_compress, KV_cache_reconstruct  # noqa: F401
         from model.public_func import get_block_token_idx, last_attn_weights, make_sum_equal  # noqa: F401
