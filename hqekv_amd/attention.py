@@ -49,7 +49,10 @@ def _f16_k_item(k16: torch.Tensor, idx, keep: list) -> dict:
     return dict(bits=16, n_tokens=T, data=data, idx=idx, token_major=tm)
 
 
-def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True) -> Tuple[List[dict], int, int]:
+def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True,
+                 residual: bool = True) -> Tuple[List[dict], int, int]:
+    """K classes of the tuple in launch order; ``residual=False`` leaves out ``new_K`` (the only segment
+    that changes between two compressions)."""
     items = []
     nh_kv = D = None
     if pkv[K16] is not None:
@@ -69,7 +72,7 @@ def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = Tru
             layout = _lib.LAYOUT_NORMAL1 if (b == 1 and not low_uniform) else 0
             items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx, layout=layout))
     new_K = pkv[NEW_K]
-    if new_K is not None and new_K.shape[2] > 0:
+    if residual and new_K is not None and new_K.shape[2] > 0:
         nk = new_K.contiguous()
         keep.append(nk)
         nh_kv, D = nk.shape[1], nk.shape[3]
@@ -78,7 +81,8 @@ def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = Tru
     return items, nh_kv, D
 
 
-def value_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True) -> Tuple[List[dict], int, int]:
+def value_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = True,
+                   residual: bool = True) -> Tuple[List[dict], int, int]:
     items = []
     nh_kv = D = None
     if pkv[V16] is not None:
@@ -100,7 +104,7 @@ def value_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = T
             layout = _lib.LAYOUT_NORMAL1 if (b == 1 and not low_uniform) else 0
             items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx, layout=layout))
     new_V = pkv[NEW_V]
-    if new_V is not None and new_V.shape[2] > 0:
+    if residual and new_V is not None and new_V.shape[2] > 0:
         nv = new_V.contiguous()
         keep.append(nv)
         nh_kv, D = nv.shape[1], nv.shape[3]
@@ -167,13 +171,82 @@ def default_flags() -> int:
     return 0 if os.environ.get("HQEKV_UNFUSED", "0") == "1" else _lib.FUSE_SOFTMAX
 
 
+class SegmentMemo:
+    """One layer's segment tables between two compressions.  Fields 0..38 of the tuple (the classes) stay
+    the same tensor objects from one decode step to the next -- the caller only replaces ``new_K``,
+    ``new_V`` and the length -- so their table entries are built once and only the residual entry is
+    rewritten per step.  The memo holds the class tensors it points into; it is valid for a tuple whose
+    first 39 fields ARE the held objects, and rebuilt otherwise.  The workspace is kept as well (calls of
+    one layer are ordered on one stream)."""
+
+    def __init__(self):
+        self.held: Optional[tuple] = None
+        self.key = None
+        self.ws: Optional[torch.Tensor] = None
+
+    def lookup(self, pkv: tuple, dev, low_uniform: bool) -> bool:
+        held = self.held
+        if held is None or self.key != (dev, low_uniform):
+            return False
+        for a, b in zip(held, pkv):  # zip stops after the 39 held fields
+            if a is not b:
+                return False
+        return True
+
+    def build(self, pkv: tuple, dev, low_uniform: bool) -> None:
+        self.keep: list = []
+        k_items, hk, dk = key_segments(pkv, dev, 0, self.keep, low_uniform, residual=False)
+        v_items, hv, dv = value_segments(pkv, dev, 0, self.keep, low_uniform, residual=False)
+        if len(k_items) + 1 > _lib.MAX_SEGS or len(v_items) + 1 > _lib.MAX_SEGS:
+            raise ValueError("too many segments")
+        self.n_k, self.n_v = len(k_items), len(v_items)
+        self.k_arr = (_lib.Seg * (self.n_k + 1))()   # one spare entry each for the residual
+        self.v_arr = (_lib.Seg * (self.n_v + 1))()
+        for dst, src in ((self.k_arr, _lib.make_segs(k_items)), (self.v_arr, _lib.make_segs(v_items))):
+            for i in range(len(dst) - 1):
+                C.memmove(C.byref(dst[i]), C.byref(src[i]), C.sizeof(_lib.Seg))
+        self.Hkv = hk if hk is not None else hv
+        self.dims = (dk, dv)
+        self.held = tuple(pkv[:NEW_K])
+        self.key = (dev, low_uniform)
+
+    def tables(self, pkv: tuple, Tall: int, keep: list):
+        """-> (k_segs, n_k, v_segs, n_v, Hkv, (dk, dv)) with this step's residual filled in."""
+        n_k, n_v, Hkv, (dk, dv) = self.n_k, self.n_v, self.Hkv, self.dims
+        new_K, new_V = pkv[NEW_K], pkv[NEW_V]
+        if new_K is not None and new_K.shape[2] > 0:
+            nk = new_K.contiguous()
+            keep.append(nk)
+            s = self.k_arr[n_k]
+            s.bits, s.layout, s.n_tokens, s.pos_base = 16, _lib.LAYOUT_TOKEN_MAJOR, nk.shape[2], Tall - nk.shape[2]
+            s.data = nk.data_ptr()
+            n_k += 1
+            Hkv, dk = nk.shape[1], nk.shape[3]
+        if new_V is not None and new_V.shape[2] > 0:
+            nv = new_V.contiguous()
+            keep.append(nv)
+            s = self.v_arr[n_v]
+            s.bits, s.layout, s.n_tokens, s.pos_base = 16, 0, nv.shape[2], Tall - nv.shape[2]
+            s.data = nv.data_ptr()
+            n_v += 1
+            Hkv, dv = nv.shape[1], nv.shape[3]
+        return self.k_arr, n_k, self.v_arr, n_v, Hkv, (dk, dv)
+
+    def workspace(self, need: int, dev) -> torch.Tensor:
+        if self.ws is None or self.ws.numel() * 4 < need or self.ws.device != dev:
+            self.ws = torch.empty(max(need + need // 8, 256) // 4, dtype=torch.float32, device=dev)
+        return self.ws
+
+
 def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool, flags: Optional[int] = None,
-                     low_uniform: bool = True):
+                     low_uniform: bool = True, memo: Optional[SegmentMemo] = None):
     """q (B,Hq,1,D) fp16 -> (attn_weights (B,Hq,1,Tall) fp16 probabilities, attn_output (B,Hq,1,D) fp16).
 
     One q.K^T launch over all K classes and one p.V launch over all V classes with the softmax fused
     into them; or, with a mask / an incomplete cover of the positions / ``flags=0``, the general path
     (q.K^T, scale+mask+clamp+softmax, p.V, fixed-order combine).  Runs on torch's current stream.
+    ``memo``: a ``SegmentMemo`` the caller keeps per layer, so that steps between two compressions rebuild
+    only the residual's table entry.
     """
     _lib.require_gpu(q, "q")
     if q.dtype != torch.float16:
@@ -183,9 +256,15 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     B, Hq, _, D = q.shape
     dev = q.device
     keep: list = []
-    k_items, hk, dk = key_segments(pkv, dev, Tall, keep, low_uniform)
-    v_items, hv, dv = value_segments(pkv, dev, Tall, keep, low_uniform)
-    Hkv = hk if hk is not None else hv
+    if memo is not None:
+        if not memo.lookup(pkv, dev, low_uniform):
+            memo.build(pkv, dev, low_uniform)
+        k_segs, n_k, v_segs, n_v, Hkv, (dk, dv) = memo.tables(pkv, Tall, keep)
+    else:
+        k_items, hk, dk = key_segments(pkv, dev, Tall, keep, low_uniform)
+        v_items, hv, dv = value_segments(pkv, dev, Tall, keep, low_uniform)
+        Hkv = hk if hk is not None else hv
+        k_segs, v_segs, n_k, n_v = _lib.make_segs(k_items), _lib.make_segs(v_items), len(k_items), len(v_items)
     if Hkv is None:
         raise ValueError("invalid past_key_value")
     for d_ in (dk, dv):
@@ -194,12 +273,18 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     qc = q.contiguous()
     weights = (torch.zeros if zero_init else torch.empty)(B, Hq, 1, Tall, dtype=torch.float16, device=dev)
     out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev)
-    k_segs, v_segs = _lib.make_segs(k_items), _lib.make_segs(v_items)
     mptr, mstride = _mask_arg(mask, B, Hq, Tall, dev, keep)
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        ws = decode_workspace(k_segs, len(k_items), v_segs, len(v_items), B, Hq, Hkv, D, dev)
-        rc = _lib.load().hqekv_decode_attn(
-            k_segs, len(k_items), v_segs, len(v_items), qc.data_ptr(), mptr, mstride,
+        if memo is not None:
+            need = lib.hqekv_decode_workspace_bytes(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D)
+            if need < 0:
+                raise ValueError("invalid segment table")
+            ws = memo.workspace(need, dev)
+        else:
+            ws = decode_workspace(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D, dev)
+        rc = lib.hqekv_decode_attn(
+            k_segs, n_k, v_segs, n_v, qc.data_ptr(), mptr, mstride,
             weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4,
             default_flags() if flags is None else flags, _lib.stream_ptr(dev))
     _lib.check(rc, "decode_attention")

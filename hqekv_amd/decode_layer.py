@@ -20,6 +20,7 @@ from typing import Optional, Tuple
 
 import torch
 
+from .attention import SegmentMemo
 from .hqe_2 import KV_cache_hqe_2
 from .hqe_matmul import qkv_matmul_hqe_2
 from .public_func import get_block_token_idx, last_attn_weights, make_sum_equal
@@ -55,6 +56,7 @@ class HqeAttentionLayer:
         self.history_reserve_length = 0
         self.token_num = 0
         self.last_weights = last_attn_weights(last_length=last_length)
+        self._memo = SegmentMemo()   # segment tables of the classes, rebuilt after each compression
 
     def reset(self) -> None:
         """What the reference's ``generate`` does per layer before a new prompt [555-557]."""
@@ -63,6 +65,7 @@ class HqeAttentionLayer:
         self.token_num = 0
         self.ratio_e = self.ratio_e_0.clone()
         self.last_weights.reset()
+        self._memo = SegmentMemo()
 
     def set_max_length(self, max_length: int) -> None:
         """Prompt length + new tokens: the width of the importance ring [691-695]."""
@@ -98,7 +101,7 @@ class HqeAttentionLayer:
             new_V = torch.cat((past_key_value[-2], value_states), dim=2) if past_key_value[-2] is not None else value_states
             past_key_value = past_key_value[:-3] + (new_K, new_V, kv_seq_len)
             attn_weights, attn_output = qkv_matmul_hqe_2(query_states, past_key_value, attention_mask,
-                                                         self.head_dim, self.quant_strategy)
+                                                         self.head_dim, self.quant_strategy, memo=self._memo)
         else:
             attn_weights, attn_output = self._prefill(query_states, key_states, value_states, attention_mask)
             past_key_value = (None,) * 39 + (key_states, value_states, kv_seq_len)

@@ -14,8 +14,9 @@ from .quant_matmul_hq import _KNOWN
 
 
 def qkv_matmul_hqe_2(q: torch.Tensor, past_key_value: Tuple, attention_mask, head_dim: int,
-                     quant_strategy: str, block_size: int = 32, group_size: int = 32):
-    """-> (attn_weights (B,Hq,1,real_len) fp16, attn_output (B,Hq,1,D) fp16)."""
+                     quant_strategy: str, block_size: int = 32, group_size: int = 32, memo=None):
+    """-> (attn_weights (B,Hq,1,real_len) fp16, attn_output (B,Hq,1,D) fp16).
+    ``memo`` (not in the reference's signature, optional): an ``attention.SegmentMemo`` kept per layer."""
     if quant_strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
         # upstream accepts only these two here (quant/hqe_matmul.py:370-377)
         raise ValueError('invalid quant_strategy')
@@ -25,7 +26,7 @@ def qkv_matmul_hqe_2(q: torch.Tensor, past_key_value: Tuple, attention_mask, hea
     if real_len == 0:
         raise ValueError('invalid past_key_value')
     return decode_attention(q, past_key_value, None, real_len, zero_init=False,
-                            low_uniform=quant_strategy == "uniform_group")
+                            low_uniform=quant_strategy == "uniform_group", memo=memo)
 
 
 def qkv_matmul_hqe(q: torch.Tensor, past_key_value: Tuple, attention_mask, head_dim: int,

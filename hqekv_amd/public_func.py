@@ -111,7 +111,14 @@ class last_attn_weights:
             new_line = rows.sum(0).sum(0)
             self.weights[:new_line.shape[0], :new_line.shape[1]] = new_line
         else:                           # decode: one row into the ring
-            new_line = attn_weights.sum(0).sum(0)
-            self.weights[self.next_line:self.next_line + 1, :new_line.shape[1]] = new_line
+            # sum over the batch, then over the heads, each rounded to the ring's dtype like the reference's
+            # ``.sum(0).sum(0)``; with one batch row the first sum is the identity, and the second one
+            # writes its row of the ring directly
+            per_head = attn_weights[0] if attn_weights.shape[0] == 1 else attn_weights.sum(0)
+            new_line = self.weights[self.next_line:self.next_line + 1, :per_head.shape[-1]]
+            if new_line.dtype == per_head.dtype:
+                torch.sum(per_head, dim=0, out=new_line)
+            else:
+                new_line.copy_(per_head.sum(0))
         self.kv_seq_len = new_line.shape[1]
         self.next_line = (self.next_line + new_line.shape[0]) % self.last_length

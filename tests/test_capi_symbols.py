@@ -112,3 +112,25 @@ def test_host_helpers_match_oracle():
     # ring of the last 4 decode rows, each summed over 2 heads; columns seen by fewer rows divide by fewer
     imp2 = lw.calculate_token_importance()
     assert imp2.shape == (6,) and abs(float(imp2[0]) - 2 * (3 + 4 + 5 + 6) / 4) < 1e-6
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_importance_ring_matches_oracle(batch):
+    """Decode rows written straight into the ring (one reduction, no temporary) against the oracle's
+    ``.sum(0).sum(0)`` + slice assignment, fp16, growing length, more steps than the ring has rows."""
+    import torch
+    from hqekv_amd import public_func as P
+    from oracle import hqe_oracle as O
+    g = torch.Generator().manual_seed(5)
+    a, b = P.last_attn_weights(20), O.ImportanceRing(20, 300)
+    a.set_max_length(300)
+    prompt = torch.rand(batch, 8, 20, 200, generator=g).half()
+    a.update(prompt)
+    b.update(prompt)
+    for step in range(45):
+        w = torch.rand(batch, 8, 1, 201 + step, generator=g).half()
+        a.update(w)
+        b.update(w)
+        assert a.next_line == b.next_line and a.kv_seq_len == b.kv_seq_len
+    assert torch.equal(a.weights, b.weights)
+    assert torch.equal(a.calculate_token_importance(), b.importance())
