@@ -60,8 +60,46 @@ def _host_idx(t: torch.Tensor) -> np.ndarray:
     return h
 
 
+class _Staging:
+    """Page-locked staging area for the small index arrays a compression sends to the device: a copy out of
+    pageable memory is synchronous (tens of microseconds each, a dozen per compression), one out of
+    page-locked memory is queued like a kernel.  Slices are handed out in ring order; before the ring wraps
+    the stream that read the previous lap is waited for."""
+    WORDS = 1 << 20  # int64 entries (8 MiB)
+
+    def __init__(self):
+        self.buf = torch.empty(self.WORDS, dtype=torch.int64, pin_memory=True)
+        self.view = self.buf.numpy()
+        self.pos = 0
+        self.used_by = set()
+
+    def put(self, a: np.ndarray, dev) -> torch.Tensor:
+        n = a.size
+        if n > self.WORDS // 4:
+            return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(dev)
+        if self.pos + n > self.WORDS:
+            for d in self.used_by:
+                torch.cuda.current_stream(d).synchronize()
+            self.used_by.clear()
+            self.pos = 0
+        lo = self.pos
+        self.pos += n
+        self.view[lo:lo + n] = a
+        self.used_by.add(dev)
+        return self.buf[lo:lo + n].to(dev, non_blocking=True)
+
+
+_staging: Optional[_Staging] = None
+
+
 def _to_dev(a: np.ndarray, dev) -> torch.Tensor:
-    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(dev)
+    global _staging
+    dev = torch.device(dev)
+    if dev.type != "cuda":
+        return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(dev)
+    if _staging is None:
+        _staging = _Staging()
+    return _staging.put(a, dev)
 
 
 def _dev_idx(h: np.ndarray, dev) -> torch.Tensor:
@@ -207,7 +245,12 @@ def _v_append(dst: _Cls, x: torch.Tensor, idx_h: np.ndarray, bits: int, strategy
 def _targets(sorted_idx: torch.Tensor, bit_num: torch.Tensor) -> List[Optional[np.ndarray]]:
     """Slices (host) of the ranked token list for (16, 8, 4, 2, 1[, evict]); None where a share is empty."""
     cum = [0] + [int(v) for v in torch.cumsum(bit_num.to(torch.int64).cpu(), 0).tolist()]
-    sorted_h = sorted_idx.detach().to("cpu", torch.int64).numpy()
+    packed = getattr(sorted_idx, "_hq_block_order", None)
+    if packed is not None and packed[0].numel() * packed[1] == sorted_idx.numel():
+        order, bs = packed  # made by get_block_token_idx: whole blocks in ranked order
+        sorted_h = (order.detach().to("cpu", torch.int64).numpy()[:, None] * bs + np.arange(bs, dtype=np.int64)).reshape(-1)
+    else:
+        sorted_h = sorted_idx.detach().to("cpu", torch.int64).numpy()
     return [sorted_h[cum[i]:cum[i + 1]] if cum[i + 1] > cum[i] else None for i in range(len(cum) - 1)]
 
 

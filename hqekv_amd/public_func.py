@@ -50,7 +50,11 @@ def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tenso
     device sort."""
     _, order = torch.sort(get_block_importance(block_size, block_num, importance), descending=True, stable=True)
     ar = torch.arange(block_size, dtype=order.dtype, device=order.device)
-    return (order.reshape(-1, 1) * block_size + ar.reshape(1, -1)).flatten()
+    idx = (order.reshape(-1, 1) * block_size + ar.reshape(1, -1)).flatten()
+    # the block order rides along: the cache policy needs the ranking on the host and fetches these
+    # block_num entries instead of block_num * block_size
+    idx._hq_block_order = (order, block_size)
+    return idx
 
 
 def make_sum_equal(array: torch.Tensor, array_sum: int, start_idx: int = 4) -> torch.Tensor:
