@@ -241,6 +241,147 @@ def bench_quantize(args):
     print(json.dumps(out))
 
 
+
+# ------------------------------------------------------------------------------------------------ config 5
+# End-to-end greedy decode of a random-init Llama-3.1-8B (bf16 weights) on the HqeKV cache.  The model around
+# the attention path (embedding, RMSNorm, projections, rotary embedding, MLP, lm_head) is plain torch: it is
+# the load the path runs under, not part of it.
+
+class _RandomLlama:
+    HID, FFN, VOCAB, HQ, HKV, D, THETA, EPS = 4096, 14336, 128256, 32, 8, 128, 500000.0, 1e-5
+
+    def __init__(self, n_layers: int, dev, seed: int = 0):
+        g = torch.Generator(device=dev).manual_seed(seed)
+
+        def w(*shape):
+            return torch.empty(*shape, dtype=torch.bfloat16, device=dev).normal_(0.0, 0.02, generator=g)
+
+        self.dev, self.n_layers = dev, n_layers
+        self.embed, self.lm_head = w(self.VOCAB, self.HID), w(self.VOCAB, self.HID)
+        self.norm_f = torch.ones(self.HID, dtype=torch.bfloat16, device=dev)
+        self.layers = []
+        for _ in range(n_layers):
+            self.layers.append(dict(
+                n1=torch.ones(self.HID, dtype=torch.bfloat16, device=dev),
+                n2=torch.ones(self.HID, dtype=torch.bfloat16, device=dev),
+                qkv=w((self.HQ + 2 * self.HKV) * self.D, self.HID), o=w(self.HID, self.HQ * self.D),
+                gate_up=w(2 * self.FFN, self.HID), down=w(self.HID, self.FFN)))
+        self.inv_freq = 1.0 / (self.THETA ** (torch.arange(0, self.D, 2, device=dev, dtype=torch.float32) / self.D))
+
+    def rot(self, pos):
+        """(cos, sin) tables (1, T, 1, D) for positions pos (T,), HF 'rotate_half' convention."""
+        ang = pos.to(torch.float32)[:, None] * self.inv_freq[None, :]
+        cos, sin = ang.cos(), ang.sin()
+        return (torch.cat((cos, cos), -1)[None, :, None, :].to(torch.bfloat16),
+                torch.cat((sin, sin), -1)[None, :, None, :].to(torch.bfloat16))
+
+    def qkv(self, lw, x, rot):
+        """x (B, T, HID) -> q (B,Hq,T,D), k, v (B,Hkv,T,D) fp16, rotary applied to q and k in one go."""
+        F = torch.nn.functional
+        B, T, _ = x.shape
+        y = F.linear(F.rms_norm(x, (self.HID,), lw["n1"], self.EPS), lw["qkv"]).view(B, T, self.HQ + 2 * self.HKV, self.D)
+        qk, h = y[:, :, : self.HQ + self.HKV], self.D // 2
+        qk = (qk * rot[0] + torch.cat((-qk[..., h:], qk[..., :h]), -1) * rot[1]).transpose(1, 2).half()
+        return qk[:, : self.HQ], qk[:, self.HQ:], y[:, :, self.HQ + self.HKV:].transpose(1, 2).half()
+
+    def after_attention(self, lw, x, attn):
+        """x (B,T,HID) residual stream, attn (B,Hq,T,D) fp16 -> new residual stream."""
+        F = torch.nn.functional
+        B, T, _ = x.shape
+        x = x + F.linear(attn.transpose(1, 2).reshape(B, T, self.HQ * self.D).to(torch.bfloat16), lw["o"])
+        gu = F.linear(F.rms_norm(x, (self.HID,), lw["n2"], self.EPS), lw["gate_up"])
+        return x + F.linear(F.silu(gu[..., : self.FFN]) * gu[..., self.FFN:], lw["down"])
+
+    def logits(self, x):
+        F = torch.nn.functional
+        return F.linear(F.rms_norm(x, (self.HID,), self.norm_f, self.EPS), self.lm_head)
+
+
+def bench_end_to_end(args):
+    from hqekv_amd.decode_layer import HqeAttentionLayer
+    dev = torch.device("cuda:0")
+    B, T0, NEW, NL = args.e2e_batch, args.prompt_len, args.new_tokens, args.layers or 32
+    CH = 16384  # tokens per chunk of the prompt pass outside attention (bounds the MLP's intermediate)
+    m = _RandomLlama(NL, dev)
+    # shares of all tokens: evicted 20 %, 4-bit 48 %, 2-bit 32 % (+ 64 fp16 tokens): 2.56 bit on average
+    att = [HqeAttentionLayer(m.D, bit_0=0.20, bit_4=0.48, bit_2=0.32, bit_1=0.0) for _ in range(NL)]
+    for a in att:
+        a.set_max_length(T0 + NEW)
+    g = torch.Generator(device=dev).manual_seed(1239)
+    tokens = torch.randint(0, m.VOCAB, (B, T0), generator=g, device=dev)
+    sync = torch.cuda.synchronize
+
+    # ---- prompt pass, layer by layer over the whole prompt; each layer's cache is compressed right away
+    t0 = time.perf_counter()
+    x = m.embed[tokens]
+    pos = torch.arange(T0, device=dev)
+    caches, aux = [], None
+    for l, lw in enumerate(m.layers):
+        q = torch.empty(B, m.HQ, T0, m.D, dtype=torch.float16, device=dev)
+        k = torch.empty(B, m.HKV, T0, m.D, dtype=torch.float16, device=dev)
+        v = torch.empty(B, m.HKV, T0, m.D, dtype=torch.float16, device=dev)
+        for c0 in range(0, T0, CH):
+            qc, kc, vc = m.qkv(lw, x[:, c0:c0 + CH], m.rot(pos[c0:c0 + CH]))
+            q[:, :, c0:c0 + CH], k[:, :, c0:c0 + CH], v[:, :, c0:c0 + CH] = qc, kc, vc
+        del qc, kc, vc
+        out, _, pkv, aux = att[l](q, k, v, None, None, aux if l > 0 else None)
+        del q, k, v
+        for c0 in range(0, T0, CH):
+            x[:, c0:c0 + CH] = m.after_attention(lw, x[:, c0:c0 + CH], out[:, :, c0:c0 + CH])
+        del out
+        caches.append(pkv)
+        sync()
+        print(f"[c5] prompt pass layer {l + 1}/{NL} done, {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+    nxt = m.logits(x[:, -1:]).argmax(-1)  # (B, 1)
+    del x
+    sync()
+    prompt_s = time.perf_counter() - t0
+    from hqekv_amd.attention import value_length
+    kept = value_length(caches[0])
+
+    # ---- greedy decode
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(NL)]
+          for _ in range(NEW)]
+    step_ev = [torch.cuda.Event(enable_timing=True) for _ in range(NEW + 1)]
+    sync()
+    t0 = time.perf_counter()
+    step_ev[0].record()
+    for s in range(NEW):
+        x = m.embed[nxt]
+        rot = m.rot(torch.full((1,), T0 + s, device=dev))
+        aux = None
+        for l, lw in enumerate(m.layers):
+            q, k, v = m.qkv(lw, x, rot)
+            ev[s][l][0].record()
+            out, _, caches[l], aux = att[l](q, k, v, None, caches[l], aux if l > 0 else None)
+            ev[s][l][1].record()
+            x = m.after_attention(lw, x, out)
+        nxt = m.logits(x).argmax(-1)
+        step_ev[s + 1].record()
+    sync()
+    decode_s = time.perf_counter() - t0
+    attn_ms = [sum(a.elapsed_time(b) for a, b in row) for row in ev]
+    step_ms = [step_ev[i].elapsed_time(step_ev[i + 1]) for i in range(NEW)]
+    plain = [i for i in range(NEW) if (T0 + i + 1) % 32 != 0] or list(range(NEW))  # steps without a compression
+    out = {
+        "metric": "tokens/s, end-to-end greedy decode on the HqeKV cache (config 5)",
+        "value": round(B * NEW / decode_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": NEW, "warmup": 0,
+        "ms_per_step": round(decode_s / NEW * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 cache / bf16 weights", "data": "synthetic",
+        "config": {"workload": f"c5 end to end: random-init Llama-3.1-8B shape, {NL} layers, B={B}, prompt {T0} "
+                               f"uniform-random token ids, {NEW} greedy tokens", "kept_tokens_after_prompt": kept,
+                   "shares": "evicted 20 % / 4-bit 48 % / 2-bit 32 % / 64 tokens fp16 (2.56 bit average)"},
+        "prompt_pass_s": round(prompt_s, 2),
+        "attention_share_of_step_time": round(sum(attn_ms) / sum(step_ms), 4),
+        "attention_ms_per_token_step": round(sum(attn_ms) / NEW, 3),
+        "plain_steps": {"ms_per_token_step": round(sum(step_ms[i] for i in plain) / len(plain), 3),
+                        "attention_ms": round(sum(attn_ms[i] for i in plain) / len(plain), 3)},
+        "note": "attention = the whole cache-side layer call (hybrid q.K^T / p.V launches, ring update and, every "
+                "32 tokens, the compression), measured with HIP events on the stream; the rest is torch",
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -250,6 +391,11 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="distinct layer caches cycled through")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--end-to-end", action="store_true",
+                    help="workload c5 only: prompt pass + greedy decode of a random-init Llama-3.1-8B (takes minutes)")
+    ap.add_argument("--prompt-len", type=int, default=131072)
+    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--e2e-batch", type=int, default=4)
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 256 MiB device copy, the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -263,6 +409,12 @@ def main():
 
     if args.workload == "c3":
         bench_quantize(args)
+        return
+    if args.end_to_end:
+        if args.workload != "c5":
+            print("bench.py: --end-to-end belongs to --workload c5", file=sys.stderr)
+            sys.exit(2)
+        bench_end_to_end(args)
         return
 
     from hqekv_amd import synth
