@@ -218,6 +218,32 @@ def test_fused_path_is_deterministic_and_reusable(dev):
     _close(o0, orr.cpu(), "fused vs general attn_output")
 
 
+def test_segment_memo_gives_the_same_bits(dev):
+    """A caller that keeps a SegmentMemo per layer (class entries built once, only the residual entry per
+    step, workspace reused) gets bit-identical results to the memo-less call: while the residual grows
+    token by token, after the classes are replaced by another cache, and for a cache without a residual."""
+    from hqekv_amd.attention import SegmentMemo
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    memo = SegmentMemo()
+    g = torch.Generator().manual_seed(11)
+    for ci in (1, 6, 0):
+        case = CASES[ci]
+        q, cache = _case(**case)
+        c = list(synth.cache_to(cache, dev))
+        for step in range(4):
+            if step:  # the caller appends one token to the residual; the class tensors stay the same objects
+                nk = torch.randn(case["B"], case["Hkv"], 1, case["D"], generator=g).half().to(dev)
+                nv = torch.randn(case["B"], case["Hkv"], 1, case["D"], generator=g).half().to(dev)
+                c[39] = nk if c[39] is None else torch.cat((c[39], nk), 2)
+                c[40] = nv if c[40] is None else torch.cat((c[40], nv), 2)
+                c[41] = int(c[41]) + 1
+            qd = torch.randn(case["B"], case["Hq"], 1, case["D"], generator=g).half().to(dev)
+            w0, o0 = qkv_matmul_hqe_2(qd, tuple(c), None, case["D"], "uniform_group")
+            w1, o1 = qkv_matmul_hqe_2(qd, tuple(c), None, case["D"], "uniform_group", memo=memo)
+            assert torch.equal(w0, w1) and torch.equal(o0, o1), (ci, step)
+            assert memo.lookup(tuple(c), torch.device(dev), True)
+
+
 @pytest.mark.parametrize("flags", [1, 0], ids=["fused", "general"])
 def test_plan_replayed_from_a_hip_graph(dev, flags):
     """A captured decode step (no allocation, no memset inside) replayed several times with new queries,
