@@ -20,7 +20,7 @@ position arrays (numpy), so a compression waits for the device only to fetch the
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Optional
 
 import numpy as np
 import torch

@@ -10,7 +10,6 @@ from typing import Tuple
 import torch
 
 from .attention import decode_attention, value_length
-from .quant_matmul_hq import _KNOWN
 
 
 def qkv_matmul_hqe_2(q: torch.Tensor, past_key_value: Tuple, attention_mask, head_dim: int,

@@ -11,7 +11,7 @@ or CPU fallback.  Differences from the reference that callers can observe:
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Tuple
 
 import torch
 

@@ -35,7 +35,6 @@ scores in ``torch.sort`` (block ranking; restated with a stable sort).
 """
 from __future__ import annotations
 
-import math
 from typing import List, Optional, Sequence, Tuple
 
 import torch

@@ -1,7 +1,6 @@
 """Pins for the CPU oracle: known answers, closed forms, invariants and brute force chosen so that a
 dropped term, a wrong shift or a transposed operand fails at least one of them.  No GPU needed."""
 import json
-import math
 from pathlib import Path
 
 import pytest
