@@ -814,13 +814,14 @@ __device__ __forceinline__ void pv_fetch(const SegDev &sg, int64_t t0, int nt, i
     pr.pa = sg.idx[ta];
     pr.pb = sg.idx[tb2];
   }
-  if (QUANT) {  // n_tokens is a multiple of 32, so pairs are always complete
+  if (QUANT) {  // a V class may hold any number of tokens: the last pair of an odd count reads row a twice
     const uint2 *sc = reinterpret_cast<const uint2 *>(sg.scale + ((int64_t)bh * sg.n_tokens + ta) * NG);
     const uint2 *zr = reinterpret_cast<const uint2 *>(sg.zero + ((int64_t)bh * sg.n_tokens + ta) * NG);
+    const int second = (int)(tb2 - ta);
     pr.sa = sc[0];
-    pr.sb = sc[1];
+    pr.sb = sc[second];
     pr.za = zr[0];
-    pr.zb = zr[1];
+    pr.zb = zr[second];
   }
 #pragma unroll
   for (int h = 0; h < NREP; ++h) {
@@ -1133,7 +1134,8 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
     if (!s.data) return fail(HQEKV_E_ARG, "%s: segment %d has null data", who, k);
     if (s.bits != 16) {
       if (!s.scale || !s.zero) return fail(HQEKV_E_ARG, "%s: segment %d lacks scale/zero", who, k);
-      if (s.n_tokens % 32 != 0)
+      // K is grouped along the tokens (32 per scale); V along the channels, so a V class holds any count
+      if (is_k && s.n_tokens % 32 != 0)
         return fail(HQEKV_E_ARG, "%s: segment %d n_tokens=%lld not a multiple of 32", who, k, (long long)s.n_tokens);
     }
     if (!s.idx && (s.pos_base < 0 || s.pos_base + s.n_tokens > Tall))
@@ -1423,7 +1425,9 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
 }
 
 // ------------------------------------------------------------------ per-class GEMV on the same kernels
-static bool gemv_is_pv_shape(int64_t K, int64_t N) { return N == 128 && K % 32 == 0 && K > N; }
+// Both launches compute the same contraction; the p.V one reduces over many rows (tokens) with split-K and
+// takes any row count, the q.K^T one wants the rows (channels) in multiples of 32.
+static bool gemv_is_pv_shape(int64_t K, int64_t N) { return N == 128 && (K > N || K % 32 != 0); }
 
 extern "C" int64_t hqekv_gemv_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N, int bits) {
   (void)bits;

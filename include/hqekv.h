@@ -155,7 +155,7 @@ int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale
 typedef struct hqekv_seg {
   int32_t bits;          /* 16, 8, 4, 2 or 1                                           */
   int32_t layout;        /* HQEKV_LAYOUT_*: 0 = as listed at the top of this file       */
-  int64_t n_tokens;      /* multiple of 32 unless bits == 16                           */
+  int64_t n_tokens;      /* K side: multiple of 32 unless bits == 16; V side: any       */
   int64_t pos_base;      /* used when idx == NULL                                      */
   const void *data;      /* codes (int32) or fp16 values                               */
   const void *scale;     /* NULL when bits == 16                                       */

@@ -42,6 +42,23 @@ def test_pv_shape(dev, bit, T):
     _close(out, O.gemv_uniform_group(32, p, code, s, z, bit))
 
 
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
+@pytest.mark.parametrize("T", [1, 2, 31, 37, 129, 513, 2081])
+def test_pv_shape_any_token_count(dev, bit, T):
+    """V is grouped along the channels, so a V class may hold any number of tokens (a KIVI-style cache
+    quantises V one token at a time, model/llama_kivi.py:190-203): odd counts, counts below one group of
+    lanes, counts that end a chunk with a single token."""
+    from hqekv_amd.matmul import cuda_bmm_fA_qB_uniform_group
+    g = torch.Generator().manual_seed(250 + bit + T)
+    B, Hq, Hkv, D = 2, 8, 2, 128
+    v = torch.randn(B, Hkv, T, D, generator=g).half()
+    p = torch.softmax(torch.randn(B, Hq, 1, T, generator=g) * 3, -1).half()
+    code, s, z = O.uniform_group_quantize_pack_last_dim(v, 32, bit)
+    out = cuda_bmm_fA_qB_uniform_group(32, p.to(dev), code.to(dev), s.to(dev), z.to(dev), bit)
+    assert out.shape == (B, Hq, 1, D)
+    _close(out, O.gemv_uniform_group(32, p, code, s, z, bit))
+
+
 @pytest.mark.parametrize("n_rep", [1, 2, 4, 8])
 def test_gqa_group_sizes(dev, n_rep):
     from hqekv_amd.matmul import cuda_bmm_fA_qB_uniform_group
