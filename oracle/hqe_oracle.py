@@ -24,6 +24,9 @@ Pinned:
   DecodeLayerOracle / ImportanceRing            bookkeeping invariants over a prompt and 40 decode steps (every
                                                 token in one class, the residual or evicted; class sizes follow
                                                 the ratio schedule; two blocks stay fp16)
+  KiviLayerOracle                               closed-form lengths after every step (whole blocks of K, all
+                                                but the last R tokens of V quantised) and equality of its decode
+                                                step with plain attention over the reconstructed cache
 
 Parity unpinned (no reference fixture exists and only a run of the original GPU stack
 could pin it): the last-bit behaviour of ``fp16_tensor / python_int`` on the GPU, which
@@ -698,3 +701,87 @@ class DecodeLayerOracle:
         else:
             auxiliary_parameters = None
         return attn_output, attn_weights, past_key_value, auxiliary_parameters
+
+
+class KiviLayerOracle:
+    """The cache-side logic of the reference's KIVI-style attention (model/llama_kivi.py:96-266) without the
+    projections, the rotary embedding and ``o_proj``: every token is kept, K is quantised per channel in
+    blocks of ``residual_length`` tokens once that many fp16 tokens have gathered (:155-167,236-252), V per
+    token, one token at a time, as soon as more than ``residual_length`` fp16 tokens exist (:190-203,254-264).
+    Cache tuple (:266): (K codes (B,H,D,Tq/pf), K fp16 tail (B,H,r,D), K scale, K zero, V codes (B,H,Tv,D/pf),
+    V fp16 tail, V scale, V zero, kv_seq_len).  A decode step attends over the quantised part with the
+    per-class GEMV and over the fp16 tails with plain matmuls (:130-188); here both run as dequantise-then-
+    matmul, the reference's own definition of the GEMV's result (quant/cuda_hq_test.py:82,242)."""
+
+    def __init__(self, head_dim: int, k_bits: int = 2, v_bits: int = 2, group_size: int = 32,
+                 residual_length: int = 128, scalar_div: str = "recip"):
+        assert residual_length % group_size == 0
+        self.head_dim, self.k_bits, self.v_bits = head_dim, k_bits, v_bits
+        self.group_size, self.residual_length, self.scalar_div = group_size, residual_length, scalar_div
+
+    def _q(self, x, bits):
+        return uniform_group_quantize_pack_last_dim(x, self.group_size, bits, self.scalar_div)
+
+    def step(self, q, k, v, attention_mask=None, past_key_value=None, observed=None):
+        """-> (attn_output (B,Hq,L,D) fp16, attn_weights fp16, new 9-tuple).  ``observed``: probabilities of
+        another implementation for the same decode step; the output is then computed from THEM, which checks
+        that implementation's p.V stage on its own (a raw score that lands on the other side of an fp16
+        rounding boundary moves a peaked row's probabilities by up to half a percent, and the output with them)."""
+        n_rep = q.shape[1] // k.shape[1]
+        R, D = self.residual_length, self.head_dim
+        kv_seq_len = k.shape[-2] + (past_key_value[-1] if past_key_value is not None else 0)
+        if past_key_value is not None:
+            kq, k_full, ks, kz, vq, v_full, vs, vz, _ = past_key_value
+            att_q = gemv_uniform_group(self.group_size, q, kq, ks, kz, self.k_bits) if kq is not None else None
+            k_full = torch.cat([k_full, k], dim=2) if k_full is not None else k
+            att_f = torch.matmul(q.float(), repeat_kv(k_full, n_rep).transpose(2, 3).float()).half()
+            w = torch.cat([att_q, att_f], dim=-1) if att_q is not None else att_f
+            # ``/ sqrt(D)`` in fp16, the mask if any, fp32 softmax (:145-173); the clamp is the identity without a mask
+            w = _scale_clamp_softmax(w, D, attention_mask, self.scalar_div)
+            w_own = w
+            if observed is not None:
+                w = observed
+            if k_full.shape[-2] == R:
+                c, s, z = self._q(k_full.transpose(2, 3).contiguous(), self.k_bits)
+                k_full = None
+                kq = c if kq is None else torch.cat([kq, c], dim=3)
+                ks = s if ks is None else torch.cat([ks, s], dim=3)
+                kz = z if kz is None else torch.cat([kz, z], dim=3)
+            v_full = torch.cat([v_full, v], dim=2)
+            nf = v_full.shape[-2]
+            if vq is None:
+                out = torch.matmul(w.float(), repeat_kv(v_full, n_rep).float()).half()
+            else:
+                out = gemv_uniform_group(self.group_size, w[..., :-nf], vq, vs, vz, self.v_bits)
+                out = out + torch.matmul(w[..., -nf:].float(), repeat_kv(v_full, n_rep).float()).half()
+            if nf > R:
+                c, s, z = self._q(v_full[:, :, :1, :].contiguous(), self.v_bits)
+                v_full = v_full[:, :, 1:, :].contiguous()
+                vq = c if vq is None else torch.cat([vq, c], dim=2)
+                vs = s if vs is None else torch.cat([vs, s], dim=2)
+                vz = z if vz is None else torch.cat([vz, z], dim=2)
+        else:
+            T = k.shape[-2]
+            w = torch.matmul(q.float(), repeat_kv(k, n_rep).transpose(2, 3).float()).half()
+            w = (w.float() * (D ** -0.5)).half()
+            if attention_mask is not None:
+                w = w + attention_mask
+                w = torch.max(w, torch.tensor(torch.finfo(torch.float16).min, dtype=torch.float16))
+            w = torch.softmax(w.float(), dim=-1).half()
+            out = torch.matmul(w.float(), repeat_kv(v, n_rep).float()).half()
+            if T % R != 0:
+                if T < R:
+                    k_quant, k_full = None, k
+                else:
+                    k_quant, k_full = k[:, :, :-(T % R), :].contiguous(), k[:, :, -(T % R):, :].contiguous()
+            else:
+                k_quant, k_full = k, None
+            kq = ks = kz = None
+            if k_quant is not None:
+                kq, ks, kz = self._q(k_quant.transpose(2, 3).contiguous(), self.k_bits)
+            if T <= R:
+                vq, v_full, vs, vz = None, v, None, None
+            else:
+                v_full = v[:, :, -R:, :].contiguous()
+                vq, vs, vz = self._q(v[:, :, :-R, :].contiguous(), self.v_bits)
+        return out, (w_own if past_key_value is not None else w), (kq, k_full, ks, kz, vq, v_full, vs, vz, kv_seq_len)

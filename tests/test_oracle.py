@@ -307,3 +307,43 @@ def test_normal1_statistics_and_sign_rule():
     # a constant group stores code 0 everywhere
     z = torch.full((1, 1, 1, 32), 2.5, dtype=torch.float16)
     assert O.normal_group_quantize_pack_last_dim(z, 32, 1)[0].item() == 0
+
+
+def test_kivi_layer_bookkeeping_and_equivalence_to_plain_attention():
+    """The KIVI-style state machine (model/llama_kivi.py:96-266): closed-form lengths after every step, and
+    its decode step -- per-class GEMV + dense tails + concatenation -- equals plain attention over the
+    reconstructed cache (dequantised class followed by the fp16 tail)."""
+    R, D, B, Hq, Hkv = 64, 128, 1, 4, 2
+    lay = O.KiviLayerOracle(D, k_bits=4, v_bits=2, residual_length=R)
+    g = torch.Generator().manual_seed(3)
+
+    def qkv(L):
+        return [torch.randn(B, h, L, D, generator=g).half() for h in (Hq, Hkv, Hkv)]
+
+    T = 150
+    q, k, v = qkv(T)
+    _, _, pkv = lay.step(q, k, v, None, None)
+    for step in range(1, 80):
+        T += 1
+        q, k, v = qkv(1)
+        prev = pkv
+        out, w, pkv = lay.step(q, k, v, None, prev)
+        # K: whole blocks of R quantised, the rest fp16; V: everything but the last R tokens quantised
+        n_kq = 0 if pkv[0] is None else pkv[0].shape[3] * 8
+        n_kf = 0 if pkv[1] is None else pkv[1].shape[2]
+        assert (n_kq, n_kf) == (T // R * R, T % R) and pkv[8] == T
+        assert pkv[4].shape[2] == T - R and pkv[5].shape[2] == R
+        assert torch.equal(pkv[5][:, :, -1:], v) and (n_kf == 0 or torch.equal(pkv[1][:, :, -1:], k))
+        # the same step as plain attention over the reconstructed cache (dequantised class, then the tail)
+        kq, k_full, ks, kz, vq, v_full, vs, vz, _ = prev
+        k_full = k if k_full is None else torch.cat((k_full, k), 2)
+        v_full = torch.cat((v_full, v), 2)
+        k_all = k_full if kq is None else torch.cat(
+            (O.uniform_group_dequantize_unpack_last_dim(kq, ks, kz, 32, 4).transpose(2, 3), k_full), 2)
+        v_all = torch.cat((O.uniform_group_dequantize_unpack_last_dim(vq, vs, vz, 32, 2), v_full), 2)
+        assert k_all.shape[2] == v_all.shape[2] == T
+        sc = torch.matmul(q.float(), O.repeat_kv(k_all, Hq // Hkv).transpose(2, 3).float()).half()
+        w2 = torch.softmax((sc.float() * (torch.tensor(1.0) / torch.tensor(D ** 0.5))).half().float(), -1).half()
+        out2 = torch.matmul(w2.float(), O.repeat_kv(v_all, Hq // Hkv).float()).half()
+        assert w.shape == (B, Hq, 1, T) and torch.allclose(w.float(), w2.float(), rtol=1e-3, atol=1e-4)
+        assert torch.allclose(out.float(), out2.float(), rtol=1e-3, atol=1e-3)
