@@ -36,6 +36,31 @@ def _repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
     return x[:, :, None, :, :].expand(B, H, n_rep, T, D).reshape(B, H * n_rep, T, D)
 
 
+def class_token_counts(total_length: int, ratio_q: torch.Tensor, ratio_e: torch.Tensor):
+    """Tokens per target -- fp16, 8, 4, 2, 1 bit, evicted -- for a history of ``total_length`` tokens
+    (model/llama_hqe.py:216-224).  64 tokens' worth of blocks stay fp16 and nothing goes to 8 bit; the rest is
+    split by ``ratio_q`` (4, 2, 1 bit) and ``ratio_e`` (evicted), in float32 like the reference, rounded to
+    whole blocks and repaired to add up.  -> (shares (6,) float32, token counts (6,) int32)."""
+    blocks = total_length // BLOCK
+    shares = torch.zeros(6, dtype=torch.float32)
+    shares[0] = 64 / total_length
+    shares[2:5] = ratio_q
+    shares[5:] = ratio_e
+    shares[2:] = (1 - shares[0]) * shares[2:]
+    counts = make_sum_equal(torch.round(blocks * shares).to(torch.int), blocks)
+    counts *= BLOCK
+    return shares, counts
+
+
+def ratios_for_next_increment(history: int, ratio_e_0: torch.Tensor, ratio_q: torch.Tensor):
+    """The eviction share applies to the tokens the next compression adds, not to the history it re-ranks:
+    scale it by added / (history + added) and give the quantised classes the rest, in their old proportions
+    (model/llama_hqe.py:235-239).  -> (ratio_e, ratio_q)."""
+    added = (history + BLOCK) // BLOCK * BLOCK - history
+    ratio_e = (added * ratio_e_0) / (history + added)
+    return ratio_e, (1 - ratio_e) * ratio_q / ratio_q.sum()
+
+
 class HqeAttentionLayer:
     """State of one layer: un-quantised length, kept history length, eviction / quantisation ratios and the
     importance ring.  ``bit_0`` is the evicted share, ``bit_4``/``bit_2``/``bit_1`` the 4-, 2- and 1-bit
@@ -107,40 +132,32 @@ class HqeAttentionLayer:
             past_key_value = (None,) * 39 + (key_states, value_states, kv_seq_len)
 
         self.last_weights.update(attn_weights)
-        if self.current_length >= BLOCK:
-            residual_length = self.current_length % BLOCK
-            compress_length = self.current_length - residual_length
-            total_length = self.history_reserve_length + compress_length
-            block_num = total_length // BLOCK
-            token_importance = self.last_weights.calculate_token_importance()
-            if auxiliary_parameters is not None:
-                compress_ratio, K_bit_num, V_bit_num = auxiliary_parameters
-            else:
-                ratio_168 = torch.tensor([64 / total_length, 0], dtype=torch.float32)
-                compress_ratio = torch.cat((ratio_168, self.ratio_q, self.ratio_e))
-                compress_ratio[2:] = (1 - compress_ratio[0]) * compress_ratio[2:]
-                K_bit_num = torch.round(block_num * compress_ratio).to(torch.int)
-                K_bit_num = make_sum_equal(K_bit_num, block_num)
-                K_bit_num *= BLOCK
-                V_bit_num = K_bit_num.clone()
-            eviction_len = int(K_bit_num[-1])
-            sort_importance = token_importance[:total_length].clone()
-            # ranks the blocks AND divides sort_importance by 32 in place, as the reference does
-            K_token_idx = get_block_token_idx(BLOCK, block_num, sort_importance)
-            past_key_value = KV_cache_hqe_2(past_key_value, compress_length, self.history_reserve_length,
-                                            K_token_idx, K_bit_num, V_bit_num, sort_importance,
-                                            self.quant_strategy, self.last_weights, BLOCK, BLOCK, self.times_range)
-            self.history_reserve_length += compress_length - eviction_len
-            self.current_length -= compress_length
-            if auxiliary_parameters is None:
-                next_total_length = (self.history_reserve_length + BLOCK) // BLOCK * BLOCK
-                add_length = next_total_length - self.history_reserve_length
-                self.ratio_e = (add_length * self.ratio_e_0) / (self.history_reserve_length + add_length)
-                self.ratio_q = (1 - self.ratio_e) * self.ratio_q / self.ratio_q.sum()
-            auxiliary_parameters = (compress_ratio, K_bit_num, V_bit_num)
+        if self.current_length < BLOCK:
+            self.token_num += 1
+            return attn_output, attn_weights, past_key_value, None
+
+        # whole blocks of the un-quantised tokens join the history; the rest stays the fp16 residual
+        compress_length = self.current_length // BLOCK * BLOCK
+        total_length = self.history_reserve_length + compress_length
+        shared = auxiliary_parameters is not None          # layer 0 of this step already sized the classes
+        if shared:
+            shares, K_bit_num, V_bit_num = auxiliary_parameters
         else:
-            auxiliary_parameters = None
+            shares, K_bit_num = class_token_counts(total_length, self.ratio_q, self.ratio_e)
+            V_bit_num = K_bit_num.clone()
+        importance = self.last_weights.calculate_token_importance()[:total_length].clone()
+        # ranks the blocks AND divides `importance` by the block length in place, as the reference's helper
+        # does; the policy below is handed the divided values [226-231]
+        K_token_idx = get_block_token_idx(BLOCK, total_length // BLOCK, importance)
+        past_key_value = KV_cache_hqe_2(past_key_value, compress_length, self.history_reserve_length,
+                                        K_token_idx, K_bit_num, V_bit_num, importance,
+                                        self.quant_strategy, self.last_weights, BLOCK, BLOCK, self.times_range)
+        self.history_reserve_length += compress_length - int(K_bit_num[-1])
+        self.current_length -= compress_length
+        if not shared:
+            self.ratio_e, self.ratio_q = ratios_for_next_increment(self.history_reserve_length, self.ratio_e_0,
+                                                                   self.ratio_q)
         self.token_num += 1
-        return attn_output, attn_weights, past_key_value, auxiliary_parameters
+        return attn_output, attn_weights, past_key_value, (shares, K_bit_num, V_bit_num)
 
     __call__ = forward

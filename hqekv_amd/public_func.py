@@ -58,44 +58,32 @@ def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tenso
 
 
 def make_sum_equal(array: torch.Tensor, array_sum: int, start_idx: int = 4) -> torch.Tensor:
-    """Repair rounded block counts so they sum to ``array_sum``: a surplus is taken from index
-    ``start_idx`` walking down to 0, a deficit is added to ``start_idx``; later entries (the evicted
-    share) are never touched.  Works in place and returns the array, like the reference."""
-    sub = array.sum() - array_sum
-    for i in range(start_idx, -1, -1):
-        if array[i] - sub < 0:
-            sub -= array[i]
-            array[i] = 0
-        else:
-            array[i] -= sub
-            break
+    """Repair rounded block counts so that they add up to ``array_sum`` (the rule of the reference's
+    model/public_func.py:259-268): what is too much is taken away from entry ``start_idx``, then from the
+    entries below it, each down to zero at most; what is missing is added to entry ``start_idx``.  Entries
+    above ``start_idx`` (the evicted share) are never touched.  Works in place and returns ``array``."""
+    excess = int(array.sum()) - int(array_sum)
+    if excess < 0:
+        array[start_idx] -= excess
+        return array
+    i = start_idx
+    while excess > 0 and i >= 0:
+        take = min(excess, int(array[i]))
+        array[i] -= take
+        excess -= take
+        i -= 1
     return array
 
 
 class last_attn_weights:
-    """Ring of the last ``last_length`` attention rows (summed over batch and heads); the column mean of
-    the ring is the token importance the policy ranks blocks by."""
+    """The last ``last_length`` attention rows, each summed over batch and heads (model/public_func.py:208-257;
+    same attribute and method names: the model code and the cache policy reach into them).  ``weights`` is the
+    (last_length, max_length) store: the rows of a prompt fill it from the top, decode rows go round in a ring
+    from ``next_line``.  A token's importance is the mean of its column over the rows that have seen it."""
 
     def __init__(self, last_length: int = 20):
         self.last_length = last_length
-        self.max_length = 0
-        self.kv_seq_len = 0
-        self.next_line = 0
-        self.weights = None
-
-    def calculate_token_importance(self) -> torch.Tensor:
-        count = torch.arange(self.kv_seq_len, 0, -1, dtype=self.weights.dtype, device=self.weights.device)
-        count[:-self.last_length] = self.last_length
-        return self.weights[:, :self.kv_seq_len].sum(0) / count
-
-    def clear(self) -> None:
-        self.next_line = 0
-        self.weights.zero_()
-
-    def eviction(self, reserve_idx: torch.Tensor) -> None:
-        if self.weights is not None:
-            kept = self.weights[:, reserve_idx]
-            self.weights[:, :kept.shape[1]] = kept
+        self.reset()
 
     def reset(self) -> None:
         self.max_length = 0
@@ -106,23 +94,39 @@ class last_attn_weights:
     def set_max_length(self, max_length: int) -> None:
         self.max_length = max_length
 
-    def update(self, attn_weights: torch.Tensor) -> None:
+    def clear(self) -> None:
+        self.next_line = 0
+        self.weights.zero_()
+
+    def calculate_token_importance(self) -> torch.Tensor:
+        n, w = self.kv_seq_len, self.weights
+        # column j has been seen by min(last_length, n - j) rows: the newest tokens by fewer than all of them
+        seen = torch.clamp(n - torch.arange(n, device=w.device), max=self.last_length).to(w.dtype)
+        return w[:, :n].sum(0) / seen
+
+    def eviction(self, reserve_idx: torch.Tensor) -> None:
+        """Keep the columns ``reserve_idx`` (ascending positions of the survivors), packed to the left."""
         if self.weights is None:
-            self.weights = torch.zeros(self.last_length, self.max_length, dtype=attn_weights.dtype,
-                                       device=attn_weights.device)
-        if attn_weights.shape[2] > 1:   # prefill: keep the last rows
-            rows = attn_weights if attn_weights.shape[2] < self.last_length else attn_weights[:, :, -self.last_length:, :]
-            new_line = rows.sum(0).sum(0)
-            self.weights[:new_line.shape[0], :new_line.shape[1]] = new_line
-        else:                           # decode: one row into the ring
-            # sum over the batch, then over the heads, each rounded to the ring's dtype like the reference's
-            # ``.sum(0).sum(0)``; with one batch row the first sum is the identity, and the second one
-            # writes its row of the ring directly
+            return
+        kept = torch.index_select(self.weights, 1, reserve_idx)
+        self.weights.narrow(1, 0, kept.shape[1]).copy_(kept)
+
+    def update(self, attn_weights: torch.Tensor) -> None:
+        """attn_weights (B, H, L, T): a prompt (L > 1) stores its last rows, a decode step (L == 1) one ring row.
+        The sums run over the batch first and over the heads second, each rounded to the store's dtype."""
+        if self.weights is None:
+            self.weights = attn_weights.new_zeros(self.last_length, self.max_length)
+        L, T = attn_weights.shape[2], attn_weights.shape[3]
+        if L > 1:
+            rows = min(L, self.last_length)
+            self.weights[:rows, :T] = attn_weights[:, :, L - rows:, :].sum(0).sum(0)
+        else:
+            rows = 1
             per_head = attn_weights[0] if attn_weights.shape[0] == 1 else attn_weights.sum(0)
-            new_line = self.weights[self.next_line:self.next_line + 1, :per_head.shape[-1]]
-            if new_line.dtype == per_head.dtype:
-                torch.sum(per_head, dim=0, out=new_line)
+            line = self.weights[self.next_line:self.next_line + 1, :T]
+            if line.dtype == per_head.dtype:
+                torch.sum(per_head, dim=0, out=line)   # one reduction, written in place
             else:
-                new_line.copy_(per_head.sum(0))
-        self.kv_seq_len = new_line.shape[1]
-        self.next_line = (self.next_line + new_line.shape[0]) % self.last_length
+                line.copy_(per_head.sum(0))
+        self.kv_seq_len = T
+        self.next_line = (self.next_line + rows) % self.last_length

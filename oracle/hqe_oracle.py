@@ -356,18 +356,20 @@ def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tenso
 
 
 def make_sum_equal(array: torch.Tensor, array_sum: int, start_idx: int = 4) -> torch.Tensor:
-    """Repair rounded block counts so they sum to ``array_sum`` (model/public_func.py:259-268):
-    the surplus is taken from index ``start_idx`` walking down; a deficit is added to it."""
-    a = array.clone()
-    sub = int(a.sum()) - int(array_sum)
+    """Repair rounded block counts so they sum to ``array_sum`` (model/public_func.py:259-268): a surplus is
+    taken from index ``start_idx`` and then from the indices below it, none below zero; a deficit is added to
+    index ``start_idx``.  Returns a repaired copy."""
+    a = [int(x) for x in array.tolist()]
+    surplus = sum(a) - int(array_sum)
+    if surplus < 0:
+        a[start_idx] -= surplus
     for i in range(start_idx, -1, -1):
-        if int(a[i]) - sub < 0:
-            sub -= int(a[i])
-            a[i] = 0
-        else:
-            a[i] -= sub
+        if surplus <= 0:
             break
-    return a
+        cut = min(a[i], surplus)
+        a[i] -= cut
+        surplus -= cut
+    return torch.tensor(a, dtype=array.dtype)
 
 
 def rerank_after_eviction(idx_per_class: Sequence[Optional[torch.Tensor]]) -> List[Optional[torch.Tensor]]:
@@ -586,8 +588,10 @@ def reconstruct_cache(past_key_value: tuple, quant_strategy: str = "uniform_grou
 
 # --------------------------------------------------------------------------- the layer that calls the path
 class ImportanceRing:
-    """model/public_func.py:208-257: ring of the last ``last_length`` attention rows, summed over batch and
-    heads in the rows' own dtype; importance = column sum / number of rows that saw the column."""
+    """model/public_func.py:208-257: the last ``last_length`` attention rows, each summed over the batch and
+    then over the heads in the rows' own dtype; a prompt fills the store from the top with its last rows, a
+    decode step writes the row at ``next_line`` and moves on, modulo ``last_length``.
+    importance[j] = column sum / number of stored rows that have seen token j."""
 
     def __init__(self, last_length: int = 20, max_length: int = 0):
         self.last_length, self.max_length = last_length, max_length
@@ -598,20 +602,18 @@ class ImportanceRing:
     def update(self, attn_weights: torch.Tensor) -> None:
         if self.weights is None:
             self.weights = torch.zeros(self.last_length, self.max_length, dtype=attn_weights.dtype)
-        if attn_weights.shape[2] > 1:
-            rows = attn_weights if attn_weights.shape[2] < self.last_length else attn_weights[:, :, -self.last_length:, :]
-            line = rows.sum(0).sum(0)
-            self.weights[:line.shape[0], :line.shape[1]] = line
-        else:
-            line = attn_weights.sum(0).sum(0)
-            self.weights[self.next_line:self.next_line + 1, :line.shape[1]] = line
-        self.kv_seq_len = line.shape[1]
-        self.next_line = (self.next_line + line.shape[0]) % self.last_length
+        L, T = attn_weights.shape[2], attn_weights.shape[3]
+        rows = min(L, self.last_length) if L > 1 else 1
+        summed = attn_weights[:, :, L - rows:, :].sum(0).sum(0)            # (rows, T)
+        first = 0 if L > 1 else self.next_line
+        self.weights[first:first + rows, :T] = summed
+        self.kv_seq_len = T
+        self.next_line = (self.next_line + rows) % self.last_length
 
     def importance(self) -> torch.Tensor:
-        count = torch.arange(self.kv_seq_len, 0, -1, dtype=self.weights.dtype)
-        count[:-self.last_length] = self.last_length
-        return self.weights[:, :self.kv_seq_len].sum(0) / count
+        n = self.kv_seq_len
+        seen = torch.tensor([min(self.last_length, n - j) for j in range(n)], dtype=self.weights.dtype)
+        return self.weights[:, :n].sum(0) / seen
 
 
 class DecodeLayerOracle:
@@ -661,46 +663,45 @@ class DecodeLayerOracle:
             past_key_value = (None,) * 39 + (k, v, kv_seq_len)
 
         self.ring.update(attn_weights if observed is None else observed)
-        if self.current_length >= 32:
-            residual = self.current_length % 32
-            compress_length = self.current_length - residual
-            total = self.history_reserve_length + compress_length
-            block_num = total // 32
-            importance = self.ring.importance()
-            if auxiliary_parameters is not None:
-                compress_ratio, K_bit_num, V_bit_num = auxiliary_parameters
-            else:
-                ratio_168 = torch.tensor([64 / total, 0], dtype=torch.float32)
-                compress_ratio = torch.cat((ratio_168, self.ratio_q, self.ratio_e))
-                compress_ratio[2:] = (1 - compress_ratio[0]) * compress_ratio[2:]
-                K_bit_num = torch.round(block_num * compress_ratio).to(torch.int)
-                K_bit_num = make_sum_equal(K_bit_num, block_num)
-                K_bit_num *= 32
-                V_bit_num = K_bit_num.clone()
-            eviction_len = int(K_bit_num[-1])
-            sort_importance = importance[:total].clone()
-            K_token_idx = get_block_token_idx(32, block_num, sort_importance)
-            # the reference's ranking divides its argument by the block length in place
-            # (model/public_func.py:94-96), so the policy below receives importance / 32
-            sort_importance = sort_importance / 32
-            past_key_value, ring = compress_cache(past_key_value, compress_length, self.history_reserve_length,
-                                                  K_token_idx, K_bit_num, V_bit_num, sort_importance,
-                                                  times_range=self.times_range, scalar_div=self.scalar_div,
-                                                  weights_ring=self.ring.weights,
-                                                  quant_strategy=self.quant_strategy)
-            if ring is not None:
-                self.ring.weights = ring
-            self.history_reserve_length += compress_length - eviction_len
-            self.current_length -= compress_length
-            if auxiliary_parameters is None:
-                next_total = (self.history_reserve_length + 32) // 32 * 32
-                add_length = next_total - self.history_reserve_length
-                self.ratio_e = (add_length * self.ratio_e_0) / (self.history_reserve_length + add_length)
-                self.ratio_q = (1 - self.ratio_e) * self.ratio_q / self.ratio_q.sum()
-            auxiliary_parameters = (compress_ratio, K_bit_num, V_bit_num)
+        if self.current_length < 32:
+            return attn_output, attn_weights, past_key_value, None
+        compress_length = self.current_length - self.current_length % 32
+        total = self.history_reserve_length + compress_length
+        if auxiliary_parameters is not None:      # sized by layer 0 of the same step (:211-214)
+            compress_ratio, K_bit_num, V_bit_num = auxiliary_parameters
         else:
-            auxiliary_parameters = None
-        return attn_output, attn_weights, past_key_value, auxiliary_parameters
+            compress_ratio, K_bit_num = split_history(total, self.ratio_q, self.ratio_e)
+            V_bit_num = K_bit_num.clone()
+        importance = self.ring.importance()[:total]
+        K_token_idx = get_block_token_idx(32, total // 32, importance)
+        # the reference's ranking helper divides its argument by the block length in place
+        # (model/public_func.py:94-96), so its policy receives importance / 32 (model/llama_hqe.py:226-231)
+        past_key_value, ring = compress_cache(past_key_value, compress_length, self.history_reserve_length,
+                                              K_token_idx, K_bit_num, V_bit_num, importance / 32,
+                                              times_range=self.times_range, scalar_div=self.scalar_div,
+                                              weights_ring=self.ring.weights,
+                                              quant_strategy=self.quant_strategy)
+        if ring is not None:
+            self.ring.weights = ring
+        self.history_reserve_length += compress_length - int(K_bit_num[-1])
+        self.current_length -= compress_length
+        if auxiliary_parameters is None:
+            # (:235-239) the eviction share is meant for the tokens the next compression adds
+            add = (self.history_reserve_length + 32) // 32 * 32 - self.history_reserve_length
+            self.ratio_e = (add * self.ratio_e_0) / (self.history_reserve_length + add)
+            self.ratio_q = (1 - self.ratio_e) * self.ratio_q / self.ratio_q.sum()
+        return attn_output, attn_weights, past_key_value, (compress_ratio, K_bit_num, V_bit_num)
+
+
+def split_history(total: int, ratio_q: torch.Tensor, ratio_e: torch.Tensor):
+    """model/llama_hqe.py:216-224: float32 shares of (fp16, 8, 4, 2, 1 bit, evicted) -- 64 tokens fp16, no
+    8-bit class, the remainder by ``ratio_q`` and ``ratio_e`` -- turned into whole 32-token blocks by rounding
+    and ``make_sum_equal``.  -> (shares, tokens per target as int32)."""
+    fp16_share = torch.tensor([64 / total, 0], dtype=torch.float32)
+    shares = torch.cat((fp16_share, ratio_q, ratio_e))
+    shares[2:] = (1 - shares[0]) * shares[2:]
+    blocks = total // 32
+    return shares, make_sum_equal(torch.round(blocks * shares).to(torch.int), blocks) * 32
 
 
 class KiviLayerOracle:
