@@ -136,6 +136,65 @@ def test_fused_wrappers_match_oracle(dev):
     _close(out, ref, "attn_output")
 
 
+def test_shape_of_the_reference_kernel_script(dev):
+    """The one configuration the reference's own kernel script runs (quant/cuda_hq_test.py:340-355 with the
+    class bounds of :27 and :296-304): B=1, 32 query heads over 8 KV heads, 8192 quantised tokens + 1023 new
+    ones, inputs uniform in [0, 1), shuffled positions; fp16 [0,64), 4 bit [64,256), 2 bit [256,7168), 1 bit
+    normal-quantile [7168,8192), no 8-bit class.  Its criterion is ours: dequantise with the library's own
+    unpack, place by idx, matmul."""
+    from hqekv_amd.matmul import cuda_bmm_forward_qk_group_hq, cuda_bmm_forward_wv_group_hq
+    g = torch.Generator().manual_seed(77)
+    quant_len, new_len, D = 8192, 1023, 128
+    T = quant_len + new_len
+    q = torch.rand(1, 32, 1, D, generator=g).half()
+    k = torch.rand(1, 8, T, D, generator=g).half()
+    v = torch.rand(1, 8, T, D, generator=g).half()
+    idx = torch.randperm(quant_len, generator=g)
+    bounds = [0, 64, 256, 7168, quant_len]          # fp16 | 4 bit | 2 bit | 1 bit
+    sl = [slice(bounds[i], bounds[i + 1]) for i in range(4)]
+
+    def classes(x, is_k):
+        """-> per class (codes or fp16 data, scale/std, zero/mean) in the stored layout, and the dequantised rows"""
+        out, dq = [], torch.zeros_like(x)
+        for s_, bits in zip(sl, (16, 4, 2, 1)):
+            part = x[:, :, s_, :].contiguous()
+            src = part.transpose(2, 3).contiguous() if is_k else part
+            if bits == 16:
+                out.append((src, None, None))
+                rows = part
+            else:
+                if bits == 1:
+                    c, a, b = O.normal_group_quantize_pack_last_dim(src, 32, 1)
+                    r = O.normal_group_dequantize_unpack_last_dim(c, a, b, 32, 1)
+                else:
+                    c, a, b = O.uniform_group_quantize_pack_last_dim(src, 32, bits)
+                    r = O.uniform_group_dequantize_unpack_last_dim(c, a, b, 32, bits)
+                out.append((c, a, b))
+                rows = r.transpose(2, 3) if is_k else r
+            dq[:, :, idx[s_], :] = rows
+        dq[:, :, quant_len:, :] = x[:, :, quant_len:, :]
+        return out, dq
+
+    def to(x):
+        return None if x is None else x.to(dev)
+
+    (k16, k4, k2, k1), dq_k = classes(k, True)
+    i16, i4, i2, i1 = (to(idx[s_]) for s_ in sl)
+    scores = cuda_bmm_forward_qk_group_hq(
+        32, 8, to(q), to(k16[0]), i16, None, None, None, None, to(k4[0]), i4, to(k4[1]), to(k4[2]),
+        to(k2[0]), i2, to(k2[1]), to(k2[2]), to(k1[0]), i1, to(k1[1]), to(k1[2]), to(k[:, :, quant_len:, :].contiguous()))
+    ref = torch.matmul(q.float(), O.repeat_kv(dq_k, 4).transpose(2, 3).float())
+    assert scores.shape == (1, 32, 1, T)
+    torch.testing.assert_close(scores.float().cpu(), ref, rtol=1e-3, atol=2e-2)   # raw scores are O(30)
+
+    w = torch.softmax((ref / D ** 0.5), dim=-1).half()
+    (v16, v4, v2, v1), dq_v = classes(v, False)
+    out = cuda_bmm_forward_wv_group_hq(
+        32, 8, to(w), to(v16[0]), i16, None, None, None, None, to(v4[0]), i4, to(v4[1]), to(v4[2]),
+        to(v2[0]), i2, to(v2[1]), to(v2[2]), to(v1[0]), i1, to(v1[1]), to(v1[2]), to(v[:, :, quant_len:, :].contiguous()))
+    _close(out, torch.matmul(w.float(), O.repeat_kv(dq_v, 4).float()), "attn_output")
+
+
 def test_all_fp16_equals_dense_attention(dev):
     """Permutation invariance: with every class at fp16 and tokens shuffled between positions, the
     result must equal dense attention over the permuted sequence."""
