@@ -376,3 +376,76 @@ def test_linearity_in_v_at_scale(dev):
     expect = (dq * w[0, 0, 0, 0].float()).sum(2, keepdim=True)                     # (B,Hkv,1,D)
     expect = expect[:, :, None].expand(B, Hkv, 4, 1, D).reshape(B, 8, 1, D)
     torch.testing.assert_close(o.float(), expect, rtol=2e-3, atol=2e-3)
+
+
+def test_random_configurations(dev):
+    """200 seeded random configurations: batch, GQA ratio 1..8, context 32..3500, class shares (with and
+    without the 1-bit class, either 1-bit coding), residual lengths, shuffled positions, masks, fused and
+    general path.  Probabilities against the oracle; the output against the oracle's p.V of the SAME
+    probabilities (a raw score on an fp16 rounding boundary may round the other way in another summation
+    order and move a peaked row by half a percent, which the first check tolerates and the second one
+    would otherwise inherit)."""
+    import random
+    from hqekv_amd.attention import decode_attention
+    checked = 0
+    for case in range(200):
+        rnd = random.Random(1000 + case)
+        B = rnd.choice([1, 1, 2, 3])
+        Hkv = rnd.choice([1, 2, 4, 8])
+        Hq = Hkv * rnd.choice([1, 2, 4, 4, 8])
+        nblocks = rnd.choice([1, 2, 3, 8, 17, 40, 64, 100])
+        residual = rnd.choice([0, 0, 1, 5, 31, 32, 97, 200])
+        nfr = 6 if rnd.random() < 0.5 else 5
+        raw = [rnd.random() ** 2 if rnd.random() < 0.7 else 0.0 for _ in range(nfr)]
+        if sum(raw) == 0:
+            raw[2] = 1.0
+        fr = [x / sum(raw) for x in raw]
+        if sum(fr[:-1]) == 0 and residual == 0:   # everything evicted and no residual: nothing to attend over
+            fr = [0.0] * nfr
+            fr[1] = 1.0
+        T = nblocks * 32 + residual
+        permute = rnd.random() < 0.4
+        low_uniform = rnd.random() < 0.5
+        use_mask = rnd.random() < 0.2
+        flags = rnd.choice([None, None, 0])
+        what = f"case {case}: B={B} Hq={Hq} Hkv={Hkv} T={T} residual={residual} shares={[round(f, 2) for f in fr]} " \
+               f"shuffled={permute} low_uniform={low_uniform} mask={use_mask} flags={flags}"
+        try:
+            classes = synth.split_blocks(T - residual, fr, 7000 + case)
+        except AssertionError:   # shares that do not round to whole blocks
+            continue
+        q, K, V = synth.make_qkv(B, Hq, Hkv, T, 128, 5000 + case)
+        override = None
+        if permute:
+            pos, kept = synth.survivor_positions(classes, T - residual)
+            perm = torch.randperm(kept, generator=torch.Generator().manual_seed(case))
+            override, start = {}, 0
+            for b, p_ in pos.items():
+                override[b] = perm[start:start + p_.numel()]
+                start += p_.numel()
+
+        def quant(x, g, bits):
+            if bits == 1 and not low_uniform:
+                return O.normal_group_quantize_pack_last_dim(x, 32, 1)
+            return O.uniform_group_quantize_pack_last_dim(x, 32, bits)
+
+        cache = synth.build_cache(K, V, classes, residual, quant, override)
+        Tall = cache[41]
+        if Tall == 0:
+            continue
+        mask = None
+        if use_mask:
+            mask = torch.zeros(B, 1, 1, Tall, dtype=torch.float16)
+            mask[..., : max(1, Tall // 3)] = torch.finfo(torch.float16).min
+        strategy = "uniform_group" if low_uniform else "high_uniform_group_low_normal_group"
+        w_ref, _ = O.qkv_matmul(q, cache, mask, 128, strategy, use_mask=True, round_per_class=False)
+        w, o = decode_attention(q.to(dev), synth.cache_to(cache, dev), None if mask is None else mask.to(dev), Tall,
+                                zero_init=True, flags=flags, low_uniform=low_uniform)
+        w, o = w.cpu(), o.cpu()
+        assert torch.isfinite(o).all(), what
+        assert torch.allclose(w.float(), w_ref.float(), rtol=RTOL, atol=ATOL), what
+        _, v_dense = O.reconstruct_cache(cache, strategy)
+        o_stage = torch.matmul(w.float(), O.repeat_kv(v_dense, Hq // Hkv).float())
+        assert torch.allclose(o.float(), o_stage, rtol=RTOL, atol=ATOL), what
+        checked += 1
+    assert checked >= 150
