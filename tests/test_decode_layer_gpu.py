@@ -61,6 +61,8 @@ def _same_tuple(got, want, where, normal=False):
     (1, 8, 2, 300, 72, "uniform_group", 0.0),
     (2, 4, 4, 96, 40, "uniform_group", 0.0),
     (1, 8, 2, 300, 72, "high_uniform_group_low_normal_group", 0.25),   # the reference's shipped default
+    (1, 4, 2, 20, 70, "uniform_group", 0.0),                            # prompt shorter than one block
+    (2, 16, 4, 511, 40, "high_uniform_group_low_normal_group", 0.1),    # ragged prompt, GQA 4, two batch rows
 ])
 def test_layer_in_lockstep_with_oracle(dev, B, Hq, Hkv, T0, steps, strategy, bit_1):
     from hqekv_amd.decode_layer import HqeAttentionLayer
@@ -86,7 +88,7 @@ def test_layer_in_lockstep_with_oracle(dev, B, Hq, Hkv, T0, steps, strategy, bit
         where = f"step {step}"
         assert torch.allclose(w_obs.float(), w_o.float(), rtol=RTOL, atol=ATOL), where
         # the prompt's output comes from torch's fused attention (outside the quantised path): looser there
-        o_rtol, o_atol = (RTOL, ATOL) if step else (1e-2, 5e-3)
+        o_rtol, o_atol = (RTOL, ATOL) if step else (1e-2, 1e-2)
         assert torch.allclose(out_g.cpu().float(), out_o.float(), rtol=o_rtol, atol=o_atol), where
         assert (aux_g is None) == (aux_o is None), where
         if aux_g is not None:
