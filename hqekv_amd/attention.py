@@ -180,9 +180,14 @@ class SegmentMemo:
     one layer are ordered on one stream)."""
 
     def __init__(self):
-        self.held: Optional[tuple] = None
-        self.key = None
+        self.held: Optional[tuple] = None      # fields 0..38 of the tuple the tables were built from
+        self.key = None                        # (device, low_uniform) they were built for
         self.ws: Optional[torch.Tensor] = None
+        self.keep: list = []                   # converted / made-contiguous tensors the tables point into
+        self.k_arr = self.v_arr = None         # ctypes arrays of hqekv_seg with one spare entry each
+        self.n_k = self.n_v = 0
+        self.Hkv = None
+        self.dims = (None, None)
 
     def lookup(self, pkv: tuple, dev, low_uniform: bool) -> bool:
         held = self.held
@@ -194,7 +199,7 @@ class SegmentMemo:
         return True
 
     def build(self, pkv: tuple, dev, low_uniform: bool) -> None:
-        self.keep: list = []
+        self.keep = []
         k_items, hk, dk = key_segments(pkv, dev, 0, self.keep, low_uniform, residual=False)
         v_items, hv, dv = value_segments(pkv, dev, 0, self.keep, low_uniform, residual=False)
         if len(k_items) + 1 > _lib.MAX_SEGS or len(v_items) + 1 > _lib.MAX_SEGS:
