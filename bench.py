@@ -37,6 +37,45 @@ WORKLOADS = {
 }
 
 
+def kernel_source_sha16() -> str:
+    """Hash of the HIP sources the library is built from: recorded next to counter-derived figures so that a
+    figure measured on other kernels is recognised as stale."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "hqekv_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            h.update(open(os.path.join(csrc, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def recorded_traffic(workload: str, kernel: str):
+    """HBM bytes per launch of ``kernel`` from the committed rocprofv3 --pmc summary, or (None, why) when that
+    summary was taken on other kernel sources than the ones this run uses.  The counters need the profiler, so
+    the figure is a recorded one, never measured by the run that prints it."""
+    path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    try:
+        rec = json.load(open(path))
+    except (OSError, ValueError):
+        return None, "profiles/pmc_traffic.json missing"
+    now = kernel_source_sha16()
+    if rec.get("kernel_source_sha16") != now:
+        return None, f"profiles/pmc_traffic.json was recorded on kernel sources {rec.get('kernel_source_sha16')}, this run uses {now}"
+    val = rec.get(workload, {}).get(kernel)
+    return val, f"recorded: profiles/pmc_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on kernel sources {now})"
+
+
 def side_bytes(pkv, k_side: bool) -> int:
     """Algorithmic bytes of the K side (q.K^T launch) or V side (p.V launch) of one layer-step."""
     if k_side:
@@ -122,8 +161,8 @@ def cpu_baseline(name: str, n_iter: int = 5, gpu_layer0=None):
         ref = O.qkv_matmul(q, cache, None, cfg["D"], use_mask=False)
         if i:
             times.append(time.perf_counter() - t0)
-    return dict(value=statistics.median(times) * 1e6 * scale, unit="us/layer", cores=cores, kind="port",
-                sample=f"{sample}; median of {n_iter} after 1 warm-up; torch {torch.__version__} CPU ops"), (q, cache, ref)
+    return dict(value=statistics.median(times) * 1e6 * scale, unit="us/layer", cores=cores, cpu_model=cpu_model(),
+                kind="port", sample=f"{sample}; median of {n_iter} after 1 warm-up; torch {torch.__version__} CPU ops"), (q, cache, ref)
 
 
 def bench_quantize(args):
@@ -224,7 +263,7 @@ def bench_quantize(args):
             O.uniform_group_quantize_pack_last_dim(vs, 32, 2)
             if i:
                 times.append(time.perf_counter() - t0)
-        cpu = dict(value=statistics.median(times) * 1e6 * H, unit="us", cores=cores, kind="port",
+        cpu = dict(value=statistics.median(times) * 1e6 * H, unit="us", cores=cores, cpu_model=cpu_model(), kind="port",
                    sample=f"K + V of ONE of the {H} KV heads at 2 bit, time x{H}; median of 3 after 1 warm-up")
     dom = max(res[2]["k_us"], res[2]["v_us"])
     out = {"metric": "us per quantize-and-pack of 8192 new tokens (K + V, 2-bit) & GB/s", "value": res[2]["us_k_plus_v"],
@@ -498,13 +537,7 @@ def main():
     dom_us, dom_bytes = (qk_us, k_bytes) if qk_us >= pv_us else (pv_us, v_bytes)
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get(args.workload, {}).get(dominant)
-        except Exception:
-            traffic = None
+    traffic, traffic_source = recorded_traffic(args.workload, dominant)
 
     out = {
         "metric": METRIC,
@@ -530,7 +563,7 @@ def main():
                        "pv_hybrid_kernel": round(pv_us, 3), "pv_combine_kernel": round(cb_us, 3)},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "bytes_per_launch": dom_bytes, "avg_us": round(dom_us, 3)},
+                     "traffic_source": traffic_source, "bytes_per_launch": dom_bytes, "avg_us": round(dom_us, 3)},
     }
 
     if args.workload == "c5":

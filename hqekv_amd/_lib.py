@@ -20,6 +20,14 @@ FUSE_SOFTMAX = 1
 ONLY_QK = 0x100
 ONLY_PV = 0x200
 ONLY_COMBINE = 0x400
+QK_TILINGS = {"8waves": 1, "4waves": 2}   # HQEKV_QK_TILING_*: tilings a call may force
+
+
+def qk_tiling(n: int) -> int:
+    """Flag bits of HQEKV_QK_TILING(n)."""
+    return (int(n) & 0xF) << 4
+
+
 LAYOUT_TOKEN_MAJOR = 1   # fp16 K segment stored (B,Hkv,T,D)
 LAYOUT_NORMAL1 = 2       # 1-bit segment in normal-quantile coding (scale = std, zero = mean)
 
@@ -29,7 +37,7 @@ EXPORTS = (
     "hqekv_quant_pack_rows", "hqekv_quant_pack_k_tokenmajor", "hqekv_dequant_unpack_rows", "hqekv_pack_i32",
     "hqekv_selftest_quant_division", "hqekv_selftest_wave_reduce",
     "hqekv_normal1_quant_pack_rows", "hqekv_normal1_quant_pack_k_tokenmajor", "hqekv_normal1_dequant_unpack_rows",
-    "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group",
+    "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group", "hqekv_gemv_normal_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
     "hqekv_decode_workspace_bytes", "hqekv_decode_attn",
 )
@@ -68,6 +76,7 @@ _PROTOS = {
     "hqekv_normal1_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "hqekv_gemv_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64, _int]),
     "hqekv_gemv_uniform_group": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
+    "hqekv_gemv_normal_group": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
     "hqekv_qk_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "hqekv_scale_softmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, C.c_float, _vp]),
     "hqekv_pv_workspace_bytes": (_i64, [_SEGP, _int, _i64, _i64, _i64, _i64]),

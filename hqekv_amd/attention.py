@@ -12,6 +12,7 @@ import ctypes as C
 import os
 from typing import List, Optional, Tuple
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -126,6 +127,52 @@ def value_length(pkv: tuple) -> int:
     return n
 
 
+def idx_cover_once(idx_list, n: int) -> bool:
+    """True when the class position arrays, taken together, hold every position in [0, n) exactly once -- what
+    the softmax fused into the two GEMV launches relies on (a position nobody writes keeps whatever the score
+    buffer held, one written twice is counted twice).  Arrays that carry a host copy (the cache policy's) are
+    checked there; others on the device, which waits for it once: the verdict is remembered per set of tensors
+    until one of them is written to."""
+    idx_list = [t for t in idx_list if t is not None]
+    if sum(int(t.numel()) for t in idx_list) != n:
+        return False
+    if not idx_list:
+        return True
+    key = tuple((id(t), t._version) for t in idx_list) + (n,)
+    hit = getattr(idx_list[0], "_hq_cover", None)   # rides on the first array, like the cache policy's host copies
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    hosts = [getattr(t, "_hq_host", None) if getattr(t, "_hq_host_version", None) == t._version else None
+             for t in idx_list]
+    if all(h is not None for h in hosts):
+        c = np.concatenate(hosts)
+        ok = bool(c.size == n and (c >= 0).all() and (c < n).all() and (np.bincount(c, minlength=n) == 1).all())
+    else:
+        c = torch.cat([t.reshape(-1).to(torch.int64) for t in idx_list])
+        inside = (c >= 0) & (c < n)
+        ok = bool(inside.all() & (torch.bincount(c.clamp(0, n - 1), minlength=n) == 1).all())
+    idx_list[0]._hq_cover = (key, ok)
+    return ok
+
+
+def _class_idx(pkv: tuple, base0: int, bases) -> list:
+    """Position arrays of the populated classes of one side."""
+    out = [pkv[base0 + 1]] if pkv[base0] is not None else []
+    return out + [pkv[bases[b] + 1] for b in BITS if pkv[bases[b]] is not None]
+
+
+def classes_partition_positions(pkv: tuple) -> bool:
+    """Both sides' classes cover [0, kept) exactly once each, kept = tokens held by the V classes."""
+    v_idx = _class_idx(pkv, V16, V_BASE)
+    n = sum(int(t.numel()) for t in v_idx if t is not None)
+    if any(t is None for t in v_idx):
+        return False
+    k_idx = _class_idx(pkv, K16, K_BASE)
+    if any(t is None for t in k_idx):
+        return False
+    return idx_cover_once(k_idx, n) and idx_cover_once(v_idx, n)
+
+
 def _mask_arg(mask, B: int, Hq: int, Tall: int, dev, keep: list):
     """-> (pointer or None, row stride in elements) for an additive fp16 mask."""
     if mask is None:
@@ -159,7 +206,7 @@ def workspace_for(v_segs, n_v: int, B: int, Hq: int, Hkv: int, D: int, dev) -> t
 
 
 def decode_workspace(k_segs, n_k: int, v_segs, n_v: int, B: int, Hq: int, Hkv: int, D: int, dev) -> torch.Tensor:
-    """Workspace of a whole decode-attention call (partials, softmax statistics, arrival counters)."""
+    """Workspace of a whole decode-attention call (split-K partials and per-tile softmax statistics)."""
     need = _lib.load().hqekv_decode_workspace_bytes(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D)
     if need < 0:
         raise ValueError("invalid segment table")
@@ -188,6 +235,7 @@ class SegmentMemo:
         self.n_k = self.n_v = 0
         self.Hkv = None
         self.dims = (None, None)
+        self.partition = False                 # the classes' position arrays cover [0, kept) once per side
 
     def lookup(self, pkv: tuple, dev, low_uniform: bool) -> bool:
         held = self.held
@@ -214,6 +262,7 @@ class SegmentMemo:
         self.dims = (dk, dv)
         self.held = tuple(pkv[:NEW_K])
         self.key = (dev, low_uniform)
+        self.partition = classes_partition_positions(pkv)
 
     def tables(self, pkv: tuple, Tall: int, keep: list):
         """-> (k_segs, n_k, v_segs, n_v, Hkv, (dk, dv)) with this step's residual filled in."""
@@ -261,11 +310,18 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     B, Hq, _, D = q.shape
     dev = q.device
     keep: list = []
+    use_flags = default_flags() if flags is None else flags
     if memo is not None:
         if not memo.lookup(pkv, dev, low_uniform):
             memo.build(pkv, dev, low_uniform)
         k_segs, n_k, v_segs, n_v, Hkv, (dk, dv) = memo.tables(pkv, Tall, keep)
+        covered = memo.partition
     else:
+        covered = not (use_flags & _lib.FUSE_SOFTMAX) or mask is not None or classes_partition_positions(pkv)
+    if not covered:   # a position nobody writes must read as zero, and the fused softmax must not run
+        use_flags &= ~_lib.FUSE_SOFTMAX
+        zero_init = True
+    if memo is None:
         k_items, hk, dk = key_segments(pkv, dev, Tall, keep, low_uniform)
         v_items, hv, dv = value_segments(pkv, dev, Tall, keep, low_uniform)
         Hkv = hk if hk is not None else hv
@@ -291,7 +347,7 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
         rc = lib.hqekv_decode_attn(
             k_segs, n_k, v_segs, n_v, qc.data_ptr(), mptr, mstride,
             weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4,
-            default_flags() if flags is None else flags, _lib.stream_ptr(dev))
+            use_flags, _lib.stream_ptr(dev))
     _lib.check(rc, "decode_attention")
     return weights, out
 
@@ -323,6 +379,8 @@ class DecodePlan:
         with torch.cuda.device(self.dev):
             self.ws = decode_workspace(self.k_segs, self.n_k, self.v_segs, self.n_v, B, Hq, self.Hkv, D, self.dev)
         self.flags = default_flags() if flags is None else flags
+        if (self.flags & _lib.FUSE_SOFTMAX) and mask is None and not classes_partition_positions(pkv):
+            self.flags &= ~_lib.FUSE_SOFTMAX   # weights is zero-initialised above: uncovered positions stay 0
         self._lib = _lib.load()
         self.inv_sqrt_d = 1.0 / (D ** 0.5)
 

@@ -20,6 +20,7 @@ position arrays (numpy), so a compression waits for the device only to fetch the
 """
 from __future__ import annotations
 
+import threading
 from typing import Dict, List, Optional
 
 import numpy as np
@@ -55,7 +56,8 @@ def _host_idx(t: torch.Tensor) -> np.ndarray:
     """Host copy of a position tensor.  Tensors made by this module carry theirs along (no device
     round trip); for anyone else's the copy is fetched, which waits for the device."""
     h = getattr(t, "_hq_host", None)
-    if h is None or h.shape[0] != t.numel():
+    # the copy is trusted only while nobody has written to the tensor since it was attached
+    if h is None or h.shape[0] != t.numel() or getattr(t, "_hq_host_version", None) != t._version:
         h = t.detach().to("cpu", torch.int64).numpy()
     return h
 
@@ -63,30 +65,36 @@ def _host_idx(t: torch.Tensor) -> np.ndarray:
 class _Staging:
     """Page-locked staging area for the small index arrays a compression sends to the device: a copy out of
     pageable memory is synchronous (tens of microseconds each, a dozen per compression), one out of
-    page-locked memory is queued like a kernel.  Slices are handed out in ring order; before the ring wraps
-    the stream that read the previous lap is waited for."""
+    page-locked memory is queued like a kernel.  Slices are handed out in ring order; every copy leaves an
+    event on the stream that issued it, and before the ring wraps all events of the lap are waited for, so a
+    slice is never overwritten while a copy on any stream may still read it.  One lock serialises callers."""
     WORDS = 1 << 20  # int64 entries (8 MiB)
 
     def __init__(self):
         self.buf = torch.empty(self.WORDS, dtype=torch.int64, pin_memory=True)
         self.view = self.buf.numpy()
         self.pos = 0
-        self.used_by = set()
+        self.events: list = []
+        self.lock = threading.Lock()
 
     def put(self, a: np.ndarray, dev) -> torch.Tensor:
         n = a.size
         if n > self.WORDS // 4:
             return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int64)).to(dev)
-        if self.pos + n > self.WORDS:
-            for d in self.used_by:
-                torch.cuda.current_stream(d).synchronize()
-            self.used_by.clear()
-            self.pos = 0
-        lo = self.pos
-        self.pos += n
-        self.view[lo:lo + n] = a
-        self.used_by.add(dev)
-        return self.buf[lo:lo + n].to(dev, non_blocking=True)
+        with self.lock:
+            if self.pos + n > self.WORDS:
+                for ev in self.events:
+                    ev.synchronize()
+                self.events.clear()
+                self.pos = 0
+            lo = self.pos
+            self.pos += n
+            self.view[lo:lo + n] = a
+            out = self.buf[lo:lo + n].to(dev, non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record(torch.cuda.current_stream(dev))
+            self.events.append(ev)
+        return out
 
 
 _staging: Optional[_Staging] = None
@@ -105,6 +113,7 @@ def _to_dev(a: np.ndarray, dev) -> torch.Tensor:
 def _dev_idx(h: np.ndarray, dev) -> torch.Tensor:
     t = _to_dev(h, dev)
     t._hq_host = h   # never modified afterwards
+    t._hq_host_version = t._version
     return t
 
 
@@ -246,7 +255,8 @@ def _targets(sorted_idx: torch.Tensor, bit_num: torch.Tensor) -> List[Optional[n
     """Slices (host) of the ranked token list for (16, 8, 4, 2, 1[, evict]); None where a share is empty."""
     cum = [0] + [int(v) for v in torch.cumsum(bit_num.to(torch.int64).cpu(), 0).tolist()]
     packed = getattr(sorted_idx, "_hq_block_order", None)
-    if packed is not None and packed[0].numel() * packed[1] == sorted_idx.numel():
+    if packed is not None and packed[0].numel() * packed[1] == sorted_idx.numel() \
+            and getattr(sorted_idx, "_hq_block_order_version", None) == sorted_idx._version:
         order, bs = packed  # made by get_block_token_idx: whole blocks in ranked order
         sorted_h = (order.detach().to("cpu", torch.int64).numpy()[:, None] * bs + np.arange(bs, dtype=np.int64)).reshape(-1)
     else:

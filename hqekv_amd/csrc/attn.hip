@@ -1189,28 +1189,22 @@ static int check_heads(const char *who, int64_t B, int64_t Hq, int64_t Hkv, int6
   return HQEKV_OK;
 }
 
+// Which q.K^T tiling a call uses: 0 = by launch size, 1 = 8 waves per 512-token tile, 2 = 4 waves per tile.
+static int qk_tiling_of(int flags) { return (flags >> 4) & 0xf; }
+
 static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
-                     int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st) {
+                     int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling = 0) {
   if (tb.total_units == 0) return HQEKV_OK;
+  if (tiling < 0 || tiling > 2) return fail(HQEKV_E_ARG, "q.K^T tiling %d (known: 0 = by size, 1, 2)", tiling);
   const int nrep = (int)(Hq / Hkv);
   // few tiles: 8 waves per tile; many tiles (several workgroups queue up per CU): 4 waves per tile
-  static const char *force = getenv("HQEKV_QK_WAVES");
-  const int waves = force ? atoi(force) : ((int64_t)tb.total_units * B * Hkv <= 1024 ? 8 : 4);
-  static const char *force_tpw = getenv("HQEKV_QK_TPW");
-  const int64_t wgs = (int64_t)tb.total_units * B * Hkv;
-  (void)wgs;  // measured at B=8, 64k context: 1, 2 and 4 tiles per workgroup take 121, 121 and 128 us -- one it is
-  const int tpw = force_tpw ? (atoi(force_tpw) > 0 ? atoi(force_tpw) : 1) : 1;
-  SegTable tw = tb;  // grid.y in workgroups: ceil(tiles / tpw) per class
-  int64_t ny = 0;
-  for (int k = 0; k < HQEKV_MAX_SEGS; ++k) {
-    tw.begin[k] = k < tb.nseg ? (int32_t)ny : 0x7fffffff;
-    if (k < tb.nseg) ny += (tb.seg[k].n_units + tpw - 1) / tpw;
-  }
-  dim3 grid((unsigned)(B * Hkv), (unsigned)ny), block((unsigned)waves * 64);
+  const int waves = tiling == 1 ? 8 : tiling == 2 ? 4 : ((int64_t)tb.total_units * B * Hkv <= 1024 ? 8 : 4);
+  const int tpw = 1;  // tiles per workgroup (2 and 4 measured no faster at B=8, 64k context)
+  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units), block((unsigned)waves * 64);
   const int rh = waves == 4 ? (nrep < 4 ? nrep : 4) : (nrep < 2 ? nrep : 2);  // QkReduce::RH
   const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
 #define LAUNCH(N_, W_)                                                                                        \
-  hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_>), grid, block, shmem, st, tw, (const half_t *)q, (half_t *)scores, \
+  hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
                      (int)Hq, (int)Hkv, (int)D, Tall, fz, tpw)
 #define LAUNCH_W(N_) \
   if (waves == 8) LAUNCH(N_, 8); else LAUNCH(N_, 4)
@@ -1227,7 +1221,7 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
 
 // chunk length for the p.V split-K: aim for a few workgroups per CU, never below 64 tokens
 static int64_t pv_chunk_tokens(int64_t total_tokens, int64_t BHkv) {
-  static const int64_t target_wgs = getenv("HQEKV_PV_TARGET_WGS") ? atoll(getenv("HQEKV_PV_TARGET_WGS")) : 256 * 4;
+  const int64_t target_wgs = 256 * 4;
   int64_t chunks_per_bh = (target_wgs + BHkv - 1) / BHkv;
   if (chunks_per_bh < 1) chunks_per_bh = 1;
   int64_t c = (total_tokens + chunks_per_bh - 1) / chunks_per_bh;
@@ -1412,7 +1406,7 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
   const int only = flags & (HQEKV_ONLY_QK | HQEKV_ONLY_PV | HQEKV_ONLY_COMBINE);
   const bool only_qk = only == HQEKV_ONLY_QK;
   if (only == 0 || only_qk) {
-    rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st);
+    rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st, qk_tiling_of(flags));
     if (rc) return rc;
     if (!fuse) {
       rc = hqekv_scale_softmax(attn_weights, mask, mask_row_stride, B * Hq, Tall, 1.0f / (float)sqrt((double)D), stream);
@@ -1438,13 +1432,13 @@ extern "C" int64_t hqekv_gemv_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv
   return hqekv_pv_workspace_bytes(&s, 1, B, Hq, Hkv, N);
 }
 
-extern "C" int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale, const void *zero,
-                                        void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N,
-                                        int bits, void *workspace, int64_t workspace_bytes, void *stream) {
-  if (!(bits == 1 || bits == 2 || bits == 4 || bits == 8)) return fail(HQEKV_E_ARG, "gemv_uniform_group: bits=%d", bits);
-  if (K <= 0 || N <= 0 || N % 32 != 0) return fail(HQEKV_E_ARG, "gemv_uniform_group: need N %% 32 == 0, K > 0");
+static int gemv_group(const char *who, int layout, const void *fA, const void *code, const void *scale,
+                      const void *zero, void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N, int bits,
+                      void *workspace, int64_t workspace_bytes, void *stream) {
+  if (K <= 0 || N <= 0 || N % 32 != 0) return fail(HQEKV_E_ARG, "%s: need N %% 32 == 0, K > 0", who);
   hqekv_seg s{};
   s.bits = bits;
+  s.layout = layout;
   s.data = code;
   s.scale = scale;
   s.zero = zero;
@@ -1455,7 +1449,24 @@ extern "C" int hqekv_gemv_uniform_group(const void *fA, const void *code, const 
     return hqekv_pv_hybrid(&s, 1, fA, out, B, Hq, Hkv, N, K, workspace, workspace_bytes, stream);
   }
   // q.K^T: reduce over the K rows, N = tokens
-  if (K % 32 != 0) return fail(HQEKV_E_UNSUPPORTED, "gemv_uniform_group: K=%lld must be a multiple of 32", (long long)K);
+  if (K % 32 != 0) return fail(HQEKV_E_UNSUPPORTED, "%s: K=%lld must be a multiple of 32", who, (long long)K);
   s.n_tokens = N;
   return hqekv_qk_hybrid(&s, 1, fA, out, B, Hq, Hkv, K, N, stream);
+}
+
+extern "C" int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale, const void *zero,
+                                        void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N,
+                                        int bits, void *workspace, int64_t workspace_bytes, void *stream) {
+  if (!(bits == 1 || bits == 2 || bits == 4 || bits == 8)) return fail(HQEKV_E_ARG, "gemv_uniform_group: bits=%d", bits);
+  return gemv_group("gemv_uniform_group", 0, fA, code, scale, zero, out, B, Hq, Hkv, K, N, bits, workspace,
+                    workspace_bytes, stream);
+}
+
+extern "C" int hqekv_gemv_normal_group(const void *fA, const void *code, const void *stdv, const void *meanv,
+                                       void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N,
+                                       int bits, void *workspace, int64_t workspace_bytes, void *stream) {
+  if (bits != 1)
+    return fail(HQEKV_E_UNSUPPORTED, "gemv_normal_group: bits=%d (only the 1-bit normal-quantile class is built)", bits);
+  return gemv_group("gemv_normal_group", HQEKV_LAYOUT_NORMAL1, fA, code, stdv, meanv, out, B, Hq, Hkv, K, N, 1,
+                    workspace, workspace_bytes, stream);
 }

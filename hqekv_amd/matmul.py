@@ -1,7 +1,8 @@
 """Drop-in for the in-scope wrappers of the reference's ``quant/matmul.py``.
 
 Same names and positional orders as quant/matmul.py:263-299 (``cuda_bmm_fA_qB_uniform_group``),
-:736-760 (``cuda_bmm_fA_qB_wv_uniform_group``), :351-434 (``cuda_bmm_forward_qk_group_hq``) and
+:736-760 (``cuda_bmm_fA_qB_wv_uniform_group``), :72-95 / :147-170 (``cuda_bmm_fA_qB_normal_group`` and its
+p.V twin), :351-434 (``cuda_bmm_forward_qk_group_hq``) and
 :507-579 (``cuda_bmm_forward_wv_group_hq``).  The reference flattens and transposes every operand
 into a kernel-side layout before each launch; these wrappers hand the stored layouts to the
 kernels unchanged.  Only the first row of ``fA`` / ``in_vector`` is computed upstream
@@ -22,17 +23,12 @@ def _need_f16(t: torch.Tensor, name: str) -> torch.Tensor:
     return t.contiguous()
 
 
-def cuda_bmm_fA_qB_uniform_group(group_size: int, fA: torch.Tensor, qB: torch.Tensor,
-                                 scales: torch.Tensor, zeros: torch.Tensor, bits: int) -> torch.Tensor:
-    """C[b,hq,0,n] = sum_k fA[b,hq,0,k] * (scales[b,hkv,k,n/32] * code[b,hkv,k,n] + zeros[b,hkv,k,n/32]).
-
-    fA (B,nh_q,1,K) fp16; qB (B,nh_kv,K,N/pf) int32; scales/zeros (B,nh_kv,K,N/32) fp16 -> (B,nh_q,1,N) fp16.
-    q.K^T passes K = head_dim, N = tokens; p.V passes K = tokens, N = head_dim.
-    """
+def _gemv_group(entry: str, who: str, group_size: int, fA: torch.Tensor, qB: torch.Tensor, scales: torch.Tensor,
+                zeros: torch.Tensor, bits: int, allowed_bits) -> torch.Tensor:
     if group_size != 32:
         raise ValueError("group_size must be 32")
-    if bits not in (1, 2, 4, 8):
-        raise ValueError("bits must be 1, 2, 4 or 8")
+    if bits not in allowed_bits:
+        raise ValueError("bits must be " + ", ".join(map(str, allowed_bits)))
     fA = _need_f16(fA, "fA")
     B, nh_q, M, K = fA.shape
     if M != 1:
@@ -53,15 +49,42 @@ def cuda_bmm_fA_qB_uniform_group(group_size: int, fA: torch.Tensor, qB: torch.Te
     with torch.cuda.device(fA.device):
         need = lib.hqekv_gemv_workspace_bytes(B, nh_q, nh_kv, K, N, bits)
         ws = torch.empty(max(need, 16) // 4, dtype=torch.float32, device=fA.device)
-        rc = lib.hqekv_gemv_uniform_group(fA.data_ptr(), qB.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
-                                          out.data_ptr(), B, nh_q, nh_kv, K, N, bits, ws.data_ptr(),
-                                          ws.numel() * 4, _lib.stream_ptr(fA.device))
-    _lib.check(rc, "cuda_bmm_fA_qB_uniform_group")
+        rc = getattr(lib, entry)(fA.data_ptr(), qB.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                                 out.data_ptr(), B, nh_q, nh_kv, K, N, bits, ws.data_ptr(),
+                                 ws.numel() * 4, _lib.stream_ptr(fA.device))
+    _lib.check(rc, who)
     return out
+
+
+def cuda_bmm_fA_qB_uniform_group(group_size: int, fA: torch.Tensor, qB: torch.Tensor,
+                                 scales: torch.Tensor, zeros: torch.Tensor, bits: int) -> torch.Tensor:
+    """C[b,hq,0,n] = sum_k fA[b,hq,0,k] * (scales[b,hkv,k,n/32] * code[b,hkv,k,n] + zeros[b,hkv,k,n/32]).
+
+    fA (B,nh_q,1,K) fp16; qB (B,nh_kv,K,N/pf) int32; scales/zeros (B,nh_kv,K,N/32) fp16 -> (B,nh_q,1,N) fp16.
+    q.K^T passes K = head_dim, N = tokens; p.V passes K = tokens, N = head_dim.
+    """
+    return _gemv_group("hqekv_gemv_uniform_group", "cuda_bmm_fA_qB_uniform_group", group_size, fA, qB, scales,
+                       zeros, bits, (1, 2, 4, 8))
 
 
 # the reference keeps a second entry point for the split-K p.V kernel; the dispatch is internal here
 cuda_bmm_fA_qB_wv_uniform_group = cuda_bmm_fA_qB_uniform_group
+
+
+def cuda_bmm_fA_qB_normal_group(group_size: int, fA: torch.Tensor, qB: torch.Tensor,
+                                stds: torch.Tensor, means: torch.Tensor, bits: int) -> torch.Tensor:
+    """The same GEMV over normal-quantile codes (quant/matmul.py:72-95; what the attention glue calls for the
+    1-bit class under 'high_uniform_group_low_normal_group', quant/hqe_matmul.py:372,424):
+    C[b,hq,0,n] = sum_k fA[b,hq,0,k] * dequant(code[b,hkv,k,n]; stds[b,hkv,k,n/32], means[b,hkv,k,n/32]).
+    Only ``bits == 1`` (2-entry table -+0.6745) is built; the wider normal-quantile tables are not on the path."""
+    if bits in (2, 4, 8):
+        raise NotImplementedError("normal-quantile GEMV is built for the 1-bit class only")
+    return _gemv_group("hqekv_gemv_normal_group", "cuda_bmm_fA_qB_normal_group", group_size, fA, qB, stds, means,
+                       bits, (1,))
+
+
+# quant/matmul.py:147-170: the split-K p.V twin; one entry serves both shapes here
+cuda_bmm_fA_qB_wv_normal_group = cuda_bmm_fA_qB_normal_group
 
 
 def _hq_tuple(m16, m16_idx, m8, m8_idx, s8, z8, m4, m4_idx, s4, z4, m2, m2_idx, s2, z2,

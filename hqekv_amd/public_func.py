@@ -54,6 +54,7 @@ def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tenso
     # the block order rides along: the cache policy needs the ranking on the host and fetches these
     # block_num entries instead of block_num * block_size
     idx._hq_block_order = (order, block_size)
+    idx._hq_block_order_version = idx._version   # ignored once somebody writes into idx
     return idx
 
 

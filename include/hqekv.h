@@ -141,6 +141,20 @@ int hqekv_gemv_uniform_group(const void *fA, const void *code, const void *scale
                              void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N,
                              int bits, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The same GEMV over a class in normal-quantile coding.  Replaces gemv_forward_cuda_normalize_group and
+ * gemv_forward_cuda_wv_normalize_group (quant/csrc/gemv_cuda.h; launched from cuda_bmm_fA_qB_normal_group,
+ * quant/matmul.py:72-95, and cuda_bmm_fA_qB_wv_normal_group, :147-170), which the attention glue calls for the
+ * 1-bit class under 'high_uniform_group_low_normal_group' (quant/hqe_matmul.py:372,424):
+ *
+ *   out[b,hq,n] = sum_k fA[b,hq,k] * rnd16(rnd16(centre[code[b,hkv,k,n]] * std[b,hkv,k,n/32]) + mean[b,hkv,k,n/32])
+ *
+ * with the 2-entry table centre = -+fp16(0.6745) (quant/pack_unpack.py:6-14).  Shapes, dtypes and workspace
+ * as above (hqekv_gemv_workspace_bytes with the same sizes); `bits` must be 1, the only width the path uses.
+ */
+int hqekv_gemv_normal_group(const void *fA, const void *code, const void *stdv, const void *meanv,
+                            void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t K, int64_t N,
+                            int bits, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------ hybrid (all classes, one launch)
  * One segment = one precision class of one layer's cache.  `idx` maps element j of the class
  * to its position in the compacted sequence (int64, shared by all batch rows and heads,
@@ -209,8 +223,14 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
  * HQEKV_ONLY_QK / HQEKV_ONLY_PV / HQEKV_ONLY_COMBINE run one part of the call (q.K^T [+ softmax] / the p.V
  * kernel / the combine) so that each can be timed on its own; the later parts expect the earlier ones to
  * have run on the same buffers.
+ * HQEKV_QK_TILING(n): which q.K^T tiling the call uses, n = 0 (default) chooses by launch size; any other
+ * value forces one of the tilings listed below, whatever the size -- results agree to the stated tolerance
+ * (the summation order over head_dim differs), so tests and measurements can name a tiling per call.
  */
 #define HQEKV_FUSE_SOFTMAX 1
+#define HQEKV_QK_TILING(n) (((n) & 0xf) << 4)
+#define HQEKV_QK_TILING_8WAVES 1 /* 512-token tile, head_dim split over 8 waves (launches of <= 1024 tiles) */
+#define HQEKV_QK_TILING_4WAVES 2 /* 512-token tile, head_dim split over 4 waves (larger launches)           */
 #define HQEKV_ONLY_QK 0x100
 #define HQEKV_ONLY_PV 0x200
 #define HQEKV_ONLY_COMBINE 0x400

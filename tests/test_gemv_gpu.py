@@ -105,3 +105,35 @@ def test_gemv_errors(dev):
         cuda_bmm_fA_qB_uniform_group(32, q, code, s[..., :1], s[..., :1], 2)
     with pytest.raises(TypeError):
         cuda_bmm_fA_qB_uniform_group(32, q.float(), code, s, s, 2)
+
+
+@pytest.mark.parametrize("shape", ["qk", "pv"])
+@pytest.mark.parametrize("T", [32, 992, 2080])
+def test_normal_group_gemv(dev, shape, T):
+    """cuda_bmm_fA_qB_normal_group (quant/matmul.py:72-95) and its p.V twin over the 1-bit normal-quantile class
+    against the reference's criterion: dequantise with the library's own unpack (quant/pack_unpack.py:356-376),
+    repeat_kv, matmul.  The stored (std, mean) are the oracle's, so the comparison is of the GEMV alone."""
+    from hqekv_amd.matmul import cuda_bmm_fA_qB_normal_group, cuda_bmm_fA_qB_wv_normal_group
+    g = torch.Generator().manual_seed(300 + T)
+    B, Hq, Hkv, D = 2, 8, 2, 128
+    if shape == "qk":
+        x = torch.randn(B, Hkv, D, T, generator=g)
+        x[:, :, 3] *= 10
+        a = torch.randn(B, Hq, 1, D, generator=g).half()
+        fn = cuda_bmm_fA_qB_normal_group
+    else:
+        x = torch.randn(B, Hkv, T, D, generator=g)
+        a = torch.softmax(torch.randn(B, Hq, 1, T, generator=g) * 3, -1).half()
+        fn = cuda_bmm_fA_qB_wv_normal_group
+    code, std, mean = O.normal_group_quantize_pack_last_dim(x.half(), 32, 1)
+    out = fn(32, a.to(dev), code.to(dev), std.to(dev), mean.to(dev), 1)
+    dq = O.normal_group_dequantize_unpack_last_dim(code, std, mean, 32, 1)
+    ref = torch.matmul(a.float(), O.repeat_kv(dq, Hq // Hkv).float())
+    assert out.shape == ref.shape and out.dtype == torch.float16
+    _close(out, ref)
+    # the uniform reading of the same bytes is a different function: the entry points are told apart
+    from hqekv_amd.matmul import cuda_bmm_fA_qB_uniform_group
+    other = cuda_bmm_fA_qB_uniform_group(32, a.to(dev), code.to(dev), std.to(dev), mean.to(dev), 1)
+    assert not torch.allclose(other.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    with pytest.raises(NotImplementedError):
+        fn(32, a.to(dev), code.to(dev), std.to(dev), mean.to(dev), 2)

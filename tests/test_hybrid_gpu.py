@@ -237,6 +237,35 @@ def test_errors(dev):
         qkv_matmul(q, (None,) * 41 + (0,), None, 128, "uniform_group")
 
 
+def test_positions_that_are_no_partition_take_the_general_path(dev):
+    """The softmax fused into the GEMV launches needs every position written exactly once.  A cache whose K
+    positions name one position twice (and so leave another out) must not take that path: the call falls back
+    to the separate softmax over a zero-initialised buffer, so every probability is finite and rows sum to one."""
+    from hqekv_amd import _lib
+    from hqekv_amd.attention import DecodePlan, classes_partition_positions
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    case = CASES[0]
+    q, cache = _case(**case)
+    c = list(synth.cache_to(cache, dev))
+    assert classes_partition_positions(tuple(c))
+    bad = c[21].clone()
+    bad[5] = bad[6]
+    c[21] = bad
+    assert not classes_partition_positions(tuple(c))
+    w, o = qkv_matmul_hqe_2(q.to(dev), tuple(c), None, case["D"], "uniform_group")
+    assert torch.isfinite(w.float()).all() and torch.isfinite(o.float()).all()
+    torch.testing.assert_close(w.float().sum(-1).cpu(), torch.ones(case["B"], case["Hq"], 1), rtol=0, atol=5e-3)
+    plan = DecodePlan(q.to(dev), tuple(c), flags=_lib.FUSE_SOFTMAX)
+    assert not (plan.flags & _lib.FUSE_SOFTMAX)
+    w2, _ = plan.run(q.to(dev))
+    torch.testing.assert_close(w2.float().sum(-1).cpu(), torch.ones(case["B"], case["Hq"], 1), rtol=0, atol=5e-3)
+    # an in-place edit of a position array is noticed (the remembered verdict is tied to the tensor's version)
+    good = list(synth.cache_to(cache, dev))
+    assert classes_partition_positions(tuple(good))
+    good[21][5] = good[21][6]
+    assert not classes_partition_positions(tuple(good))
+
+
 @pytest.mark.parametrize("Tall", [1, 7, 8, 1000, 8191, 8200, 26225, 70001, 140003])
 @pytest.mark.parametrize("with_mask", [False, True])
 def test_scale_softmax_rows(dev, Tall, with_mask):

@@ -246,6 +246,52 @@ def test_token_range_closed_form():
     assert O.calculate_token_range(None, r) is None
 
 
+def test_class_sizes_worked_by_hand():
+    """model/llama_hqe.py:216-224 and :235-239 worked with pencil arithmetic (exact fractions, no case sits on a
+    rounding tie), asserted on the oracle AND on the product's formulas.
+
+    416 tokens = 13 blocks, shipped shares 4/2/1 bit = 0.25 each, evicted 0.25: fp16 share 64/416 = 2/13, the
+    rest 11/13 * 0.25 = 11/52 each; 13 * (2/13, 0, 11/52 x 4) = (2, 0, 2.75 x 4) -> rounded (2, 0, 3, 3, 3, 3) = 14,
+    one too many, taken from the 1-bit entry -> (2, 0, 3, 3, 2, 3) blocks = (64, 0, 96, 96, 64, 96) tokens.
+    1056 tokens = 33 blocks, shares 0.2 / 0.3 / 0.4, evicted 0.1: 31/33 of them -> 33 * share = (2, 0, 6.2, 9.3, 12.4,
+    3.1) -> (2, 0, 6, 9, 12, 3) = 32, one short, added to the 1-bit entry -> (2, 0, 6, 9, 13, 3) blocks.
+    96 tokens = 3 blocks, shares 0.7 / 0.7 / 0 / 0: 3 * (2/3, 0, 0.7/3, 0.7/3, 0, 0) = (2, 0, 0.7, 0.7, 0, 0) -> (2, 0, 1, 1,
+    0, 0) = 4, one too many; the 1-bit entry is empty, so the 2-bit entry gives it up -> (2, 0, 1, 0, 0, 0)."""
+    from hqekv_amd.decode_layer import class_token_counts, ratios_for_next_increment
+    t = lambda *v: torch.tensor(v, dtype=torch.float32)
+    cases = [
+        (416, t(0.25, 0.25, 0.25), t(0.25), [64, 0, 96, 96, 64, 96], [2 / 13, 0, 11 / 52, 11 / 52, 11 / 52, 11 / 52]),
+        (1056, t(0.2, 0.3, 0.4), t(0.1), [64, 0, 192, 288, 416, 96], [2 / 33, 0, 6.2 / 33, 9.3 / 33, 12.4 / 33, 3.1 / 33]),
+        (96, t(0.7, 0.7, 0.0), t(0.0), [64, 0, 32, 0, 0, 0], [2 / 3, 0, 0.7 / 3, 0.7 / 3, 0, 0]),
+    ]
+    for total, rq, re, counts, shares in cases:
+        for fn in (O.split_history, class_token_counts):
+            got_shares, got_counts = fn(total, rq.clone(), re.clone())
+            assert got_counts.tolist() == counts, (fn.__name__, total)
+            assert int(got_counts.sum()) == total
+            assert torch.allclose(got_shares, torch.tensor(shares, dtype=torch.float32), atol=1e-6)
+    # next increment: history 320 -> 32 tokens are added to reach 352; the evicted share becomes 32 * 0.25 / 352 = 1/44,
+    # the three quantised shares (equal) take (1 - 1/44) / 3 = 43/132 each
+    e, q = ratios_for_next_increment(320, t(0.25), t(0.25, 0.25, 0.25))
+    assert torch.allclose(e, t(1 / 44), atol=1e-7) and torch.allclose(q, t(43 / 132, 43 / 132, 43 / 132), atol=1e-7)
+    # history 330 (not on the block grid): 22 tokens reach 352; 22 * 0.25 / 352 = 1/64; shares 0.2/0.3/0.5 scaled by 63/64
+    e, q = ratios_for_next_increment(330, t(0.25), t(0.2, 0.3, 0.5))
+    assert torch.allclose(e, t(1 / 64), atol=1e-7)
+    assert torch.allclose(q, t(0.196875, 0.2953125, 0.4921875), atol=1e-7)
+    # the oracle's layer applies the same update after a compression: one prompt of 352 tokens with the shipped
+    # shares -> 11 blocks: (2, 0, 2.25 x 4 * ...) worked below
+    orc = O.DecodeLayerOracle(32, bit_0=0.25, bit_4=0.25, bit_2=0.25, bit_1=0.25, max_length=400)
+    g = torch.Generator().manual_seed(1)
+    q_, k_, v_ = (torch.randn(1, h, 352, 32, generator=g).half() for h in (2, 1, 1))
+    mask = torch.triu(torch.full((352, 352), torch.finfo(torch.float16).min, dtype=torch.float16), 1)[None, None]
+    _, _, pkv, aux = orc.step(q_, k_, v_, mask, None, None)
+    # 352 tokens = 11 blocks: fp16 64/352 = 2/11; rest 9/11 * 0.25 = 9/44 each; 11 * 9/44 = 2.25 -> (2, 0, 2, 2, 2, 2) = 10,
+    # one short -> 1-bit entry 3: (64, 0, 64, 64, 96, 64) tokens, 64 evicted, history 288
+    assert aux[1].tolist() == [64, 0, 64, 64, 96, 64] and orc.history_reserve_length == 288
+    # next: 288 + 32 = 320: evicted share 32 * 0.25 / 320 = 1/40, quantised (1 - 1/40) / 3 = 13/40 each
+    assert torch.allclose(orc.ratio_e, t(1 / 40), atol=1e-7) and torch.allclose(orc.ratio_q, t(0.325, 0.325, 0.325), atol=1e-7)
+
+
 def test_layer_state_machine_bookkeeping():
     """Prompt + decode steps through the oracle's layer: every token is in exactly one class or the
     residual or was evicted, probabilities sum to one, class sizes follow the ratios."""
@@ -264,6 +310,8 @@ def test_layer_state_machine_bookkeeping():
         if aux is not None:
             evicted += int(aux[1][-1])
             assert int(aux[1].sum()) % 32 == 0 and int(aux[1][0]) == 64 and int(aux[1][1]) == 0
+            # every token of the re-ranked history gets a class: the sizes add up to history + compressed tokens
+            assert int(aux[1].sum()) == orc.history_reserve_length + int(aux[1][-1])
         kept = sum(pkv[s].shape[2] for s in (O.V16, O.V_BASE[8], O.V_BASE[4], O.V_BASE[2], O.V_BASE[1]) if pkv[s] is not None)
         resid = 0 if pkv[O.NEW_V] is None else pkv[O.NEW_V].shape[2]
         assert kept == orc.history_reserve_length and resid == orc.current_length

@@ -231,6 +231,31 @@ def test_normal1_quantiser_against_oracle(dev, layout):
     assert torch.equal(O.unpack_codes(code, 1), want_codes)
 
 
+@pytest.mark.parametrize("layout", ["rows", "token_major"])
+def test_normal1_matches_torch_std_mean_on_device(dev, layout):
+    """The reference computes the 1-bit class's statistics with ``torch.std_mean`` on the GPU
+    (quant/pack_unpack.py:227).  Its accumulation order is not documented, so the kernel's std / mean are
+    compared here with torch's own result executed on this device, bit for bit; the mismatch rate is printed
+    and the codes must follow the element-wise rule for the values the kernel stored."""
+    from hqekv_amd import pack_unpack as P
+    x = (_data((2, 4, 128, 1024), 91) * 2 + 0.5)
+    data = (x if layout == "rows" else x.transpose(2, 3)).to(dev)
+    code, std, mean = P.normal_group_quantize_pack_last_dim(data, 32, 1)
+    B, nh, R, L = data.shape
+    g = data.contiguous().reshape(B * nh * R, L // 32, 32)
+    t_std, t_mean = torch.std_mean(g, dim=-1, keepdim=True)
+    t_std, t_mean = t_std.reshape(std.shape), t_mean.reshape(mean.shape)
+    bad_std = int((std.view(torch.int16) != t_std.view(torch.int16)).sum())
+    bad_mean = int((mean.view(torch.int16) != t_mean.view(torch.int16)).sum())
+    print(f"normal1 {layout}: {bad_std} of {std.numel()} std and {bad_mean} of {mean.numel()} mean values differ "
+          f"from torch.std_mean on the device")
+    step = lambda a, b: (a.view(torch.int16).to(torch.int32) - b.view(torch.int16).to(torch.int32)).abs().max()
+    assert int(step(std, t_std)) <= 1 and int(step(mean, t_mean)) <= 1
+    assert bad_std == 0 and bad_mean == 0
+    v = (g - mean.reshape(B * nh * R, L // 32, 1)) / std.reshape(B * nh * R, L // 32, 1)
+    assert torch.equal(P.unpack_along_last_dim(code, 1).to(torch.int32), (v > 0).to(torch.int32).reshape(B, nh, R, L))
+
+
 def test_normal1_dequantiser_bit_exact_and_edges(dev):
     from hqekv_amd import pack_unpack as P
     g = torch.Generator().manual_seed(5)
