@@ -428,6 +428,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--layers", type=int, default=None, help="distinct layer caches cycled through")
+    ap.add_argument("--qk-tiling", default="auto", choices=["auto", "8waves", "4waves", "wave512", "wave128"],
+                    help="force one q.K^T tiling instead of the choice by launch size")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--end-to-end", action="store_true",
@@ -468,7 +470,10 @@ def main():
         del src, dst
     n_layers = args.layers or {"c1": 64, "c2": 32, "c4": 4, "c5": 32}[args.workload]
     layers = build_layers(args.workload, n_layers, dev)
-    plans = [DecodePlan(q, cache) for q, cache in layers]
+    from hqekv_amd import _lib as _L
+    from hqekv_amd.attention import default_flags
+    plan_flags = default_flags() | _L.qk_tiling(_L.QK_TILINGS.get(args.qk_tiling, 0))
+    plans = [DecodePlan(q, cache, flags=plan_flags) for q, cache in layers]
     qs = [q.contiguous() for q, _ in layers]
     cfg = synth.CONFIGS[args.workload]
     pkv0 = layers[0][1]
@@ -555,6 +560,7 @@ def main():
         "config": {"workload": f"{args.workload}: {WORKLOADS[args.workload]}", "B": cfg["B"], "Hq": cfg["Hq"],
                    "Hkv": cfg["Hkv"], "head_dim": cfg["D"], "context": cfg["T"], "kept_tokens": pkv0[41],
                    "layers_cycled": n_layers, "launch": "eager" if graph is None else "hip-graph replay",
+                   "qk_tiling": args.qk_tiling,
                    "softmax": "fused into the two GEMV launches" if fused else "separate launch",
                    "algorithmic_bytes_per_step": alg_bytes},
         "achieved_GBps": round(alg_bytes / (us_per_step * 1e-6) / 1e9, 1),

@@ -20,7 +20,7 @@ FUSE_SOFTMAX = 1
 ONLY_QK = 0x100
 ONLY_PV = 0x200
 ONLY_COMBINE = 0x400
-QK_TILINGS = {"8waves": 1, "4waves": 2}   # HQEKV_QK_TILING_*: tilings a call may force
+QK_TILINGS = {"8waves": 1, "4waves": 2, "wave512": 3, "wave128": 4}   # HQEKV_QK_TILING_*: tilings a call may force
 
 
 def qk_tiling(n: int) -> int:

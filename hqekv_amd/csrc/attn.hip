@@ -22,6 +22,8 @@
 //            through fp32 partials summed in a fixed order.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 #pragma clang fp contract(off)  // the two fp16 roundings of the dequantiser must stay separate
@@ -204,9 +206,6 @@ constexpr int QK_TILE = 64 * QK_TPL;    // tokens per workgroup tile
 // the smaller blocks keep the kernel at 4 waves per SIMD; 4 with 4 waves per tile
 __host__ __device__ constexpr int qk_unr(int waves) { return waves == 8 ? 2 : 4; }
 
-__host__ __device__ inline int64_t qk_tile_tokens(int bits, int token_major) {
-  return (bits == 16 && token_major) ? 64 : QK_TILE;
-}
 
 // What a lane holds of one block of QK_UNR row pairs of a quantised class (32-bit members only: a struct
 // with 16-bit members is not kept in registers).
@@ -399,7 +398,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
   }
   if (D == 128) {
     const int lg = lane & 7, tsub = lane >> 3;
-#pragma unroll
+#pragma unroll 2
     for (int r = 0; r < TPW / 8; ++r) {
       const int64_t t = (int64_t)tile * 64 + wave * TPW + r * 8 + tsub;
       const bool valid = t < n;
@@ -657,6 +656,402 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
     case 4: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<4, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
     case 8: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<8, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
     default: run_tiles([&](uint32_t, uint32_t t0, Acc acc) { qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, stage_q, q2s, acc); });
+  }
+}
+
+// =============================================================================== q.K^T, one wave per tile
+// The tiling for launches with many tiles.  A workgroup is ONE wave that owns its tokens across all of
+// head_dim: a lane keeps 8 adjacent tokens and walks the channel rows two at a time, so the sum over d never
+// leaves the lane -- no partial rows parked in LDS, no workgroup barrier, no second pass over the scores.
+// Per tile the wave first requests its first block of code words, then stages the query ([row pair][head]
+// pairs) and the tile's scale/zero rows in LDS: the rows are fetched with wide loads (a tile's groups of one
+// row are contiguous) and stored pair-interleaved -- {(s_d, s_d+1), (z_d, z_d+1)} per (row pair, group) -- so
+// the inner loop reads both with one 8-byte LDS access and pairs nothing itself.
+// DS = 1: 64 token lanes, tile = 512 tokens, a lane walks all 64 row pairs (least fixed work per code).
+// DS = 4: 16 token lanes x 4 quarters of head_dim, tile = 128 tokens; the quarters sit 16 lanes apart and are
+//         summed with two lane-row swaps: four times the waves for launches that would not fill the chip.
+// head_dim is 128 here; the host sends other sizes to the tilings above.
+template <int DS>
+struct QwGeom {
+  static constexpr int TL = 64 / DS;       // token lanes
+  static constexpr int TILE = TL * QK_TPL; // tokens per tile
+  static constexpr int NG = TILE / 32;     // scale/zero groups per tile and row
+  static constexpr int RP = 64 / DS;       // row pairs a lane walks
+  static constexpr int GPI = NG >= 8 ? 8 : NG;  // groups one staging item covers (16 or 8 bytes per row)
+};
+__host__ __device__ constexpr int qw_tile(int ds) { return (64 / ds) * QK_TPL; }
+
+// sum over the four rows of 16 lanes, valid in lanes 0-15 afterwards (two lane-row swaps per value; the swaps
+// need idle issue slots around them that the compiler does not insert for inline asm)
+__device__ __forceinline__ void rows_sum8(float (&v)[8]) {
+  float o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = v[i];
+#define HQ_SWAP8(OP_)                                                                                         \
+  asm volatile("s_nop 7\n\t" OP_ " %0, %8\n\t" OP_ " %1, %9\n\t" OP_ " %2, %10\n\t" OP_ " %3, %11\n\t"         \
+               OP_ " %4, %12\n\t" OP_ " %5, %13\n\t" OP_ " %6, %14\n\t" OP_ " %7, %15\n\ts_nop 7"               \
+               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), \
+                 "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]))
+  HQ_SWAP8("v_permlane16_swap_b32");  // rows 0 and 2: o = the old rows 1 and 3
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = o[i] = v[i] + o[i];
+  HQ_SWAP8("v_permlane32_swap_b32");  // row 0: o = the old row 2
+#undef HQ_SWAP8
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] += o[i];
+}
+// reductions inside a row of 16 lanes (every lane of the row gets the result)
+__device__ __forceinline__ float row_max16(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  return fmaxf(v, dpp_f<0x140>(v));
+}
+__device__ __forceinline__ float row_sum16(float v) {
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  return v + dpp_f<0x140>(v);
+}
+
+__device__ __forceinline__ uint4 buf_u128(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+  const v4u v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_off, (int)row_off, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 buf_u64(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+  const v2u v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)row_off, 0);
+  return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t buf_u8(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
+  return (uint32_t)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(r, (int)lane_off, (int)row_off, 0);
+}
+
+// the 8 codes of one row a lane owns: a byte at 1 bit, 16 bits at 2 bits, a word at 4 bits, two words at 8 bits
+template <int BITS>
+struct QwRow {
+  uint32_t w[BITS == 8 ? 2 : 1];
+};
+template <int BITS>
+__device__ __forceinline__ QwRow<BITS> qw_load_row(rsrc_t rc, uint32_t lane_off, uint32_t row_off) {
+  QwRow<BITS> r;
+  if constexpr (BITS == 8) {
+    const uint2 v = buf_u64(rc, lane_off, row_off);
+    r.w[0] = v.x;
+    r.w[1] = v.y;
+  } else if constexpr (BITS == 4) {
+    r.w[0] = buf_u32(rc, lane_off, row_off);
+  } else if constexpr (BITS == 2) {
+    r.w[0] = buf_u16(rc, lane_off, row_off);
+  } else {
+    r.w[0] = buf_u8(rc, lane_off, row_off);
+  }
+  return r;
+}
+
+// Stage the scale/zero rows of one tile: sz[dp * NG + g] = {(s[2dp][g], s[2dp+1][g]), (z[2dp][g], z[2dp+1][g])}.
+// Groups past the end of the class read whatever follows (the next row, or zero past the slab): only lanes
+// whose tokens do not exist look at them.
+template <int DS, bool NORMAL>
+__device__ __forceinline__ void qw_stage_sz(const SegDev &sg, int tile, int bh, int lane, uint2 *sz) {
+  using G = QwGeom<DS>;
+  constexpr int NG = G::NG, GPI = G::GPI;
+  constexpr int ITEMS = 64 * NG / GPI;   // (row pair, part of the tile's groups)
+  const uint32_t gpr = (uint32_t)(sg.n_tokens >> 5);
+  const rsrc_t rs = make_rsrc(sg.scale + (int64_t)bh * 128 * gpr, 128u * gpr * 2u);
+  const rsrc_t rz = make_rsrc(sg.zero + (int64_t)bh * 128 * gpr, 128u * gpr * 2u);
+  const uint32_t g0 = (uint32_t)tile * NG;
+#pragma unroll 1   // one item's sixteen registers at a time: the accumulators are live across this
+  for (int k = 0; k < ITEMS / 64; ++k) {
+    const int it = lane + 64 * k;
+    const int dp = it / (NG / GPI), part = it % (NG / GPI);
+    const uint32_t off = ((uint32_t)(2 * dp) * gpr + g0 + (uint32_t)part * GPI) * 2u;
+    uint32_t sa[GPI / 2], sb[GPI / 2], za[GPI / 2], zb[GPI / 2];
+    const uint32_t gb = g0 + (uint32_t)part * GPI;   // first group of this item
+    if (gb + GPI > gpr) {
+      // the last tile of a class: the item's window hangs over the end of the row (and, in the last row, over
+      // the end of the slab, where a wide load is dropped whole).  Element loads with the group clamped.
+#pragma unroll
+      for (int j = 0; j < GPI / 2; ++j) {
+        const uint32_t ga = min(gb + 2 * j, gpr - 1), gc = min(gb + 2 * j + 1, gpr - 1);
+        const uint32_t ra = ((uint32_t)(2 * dp) * gpr + ga) * 2u, rb = ((uint32_t)(2 * dp) * gpr + gc) * 2u;
+        sa[j] = buf_u16(rs, ra, 0) | (buf_u16(rs, rb, 0) << 16);
+        sb[j] = buf_u16(rs, ra, gpr * 2u) | (buf_u16(rs, rb, gpr * 2u) << 16);
+        za[j] = buf_u16(rz, ra, 0) | (buf_u16(rz, rb, 0) << 16);
+        zb[j] = buf_u16(rz, ra, gpr * 2u) | (buf_u16(rz, rb, gpr * 2u) << 16);
+      }
+    } else if constexpr (GPI == 8) {
+      const uint4 a = buf_u128(rs, off, 0), b = buf_u128(rs, off, gpr * 2u);
+      const uint4 c = buf_u128(rz, off, 0), d = buf_u128(rz, off, gpr * 2u);
+      sa[0] = a.x; sa[1] = a.y; sa[2] = a.z; sa[3] = a.w;
+      sb[0] = b.x; sb[1] = b.y; sb[2] = b.z; sb[3] = b.w;
+      za[0] = c.x; za[1] = c.y; za[2] = c.z; za[3] = c.w;
+      zb[0] = d.x; zb[1] = d.y; zb[2] = d.z; zb[3] = d.w;
+    } else {
+      const uint2 a = buf_u64(rs, off, 0), b = buf_u64(rs, off, gpr * 2u);
+      const uint2 c = buf_u64(rz, off, 0), d = buf_u64(rz, off, gpr * 2u);
+      sa[0] = a.x; sa[1] = a.y;
+      sb[0] = b.x; sb[1] = b.y;
+      za[0] = c.x; za[1] = c.y;
+      zb[0] = d.x; zb[1] = d.y;
+    }
+    uint4 *dst = reinterpret_cast<uint4 *>(sz + dp * NG + part * GPI);
+#pragma unroll
+    for (int j = 0; j < GPI / 2; ++j) {
+      half2_t s_lo = half_pair<0>(sa[j], sb[j]), s_hi = half_pair<1>(sa[j], sb[j]);
+      if (NORMAL) {  // the spread a = rnd16(k * std) once per group instead of once per use
+        s_lo = normal1_spread(s_lo);
+        s_hi = normal1_spread(s_hi);
+      }
+      dst[j] = make_uint4(as_u32(s_lo), as_u32(half_pair<0>(za[j], zb[j])), as_u32(s_hi), as_u32(half_pair<1>(za[j], zb[j])));
+    }
+  }
+}
+
+template <int BITS, int NREP, int DS, bool NORMAL, typename Stage>
+__device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int lane, Stage &&stage,
+                                                    const half2_t *q2s, const uint2 *sz, float (&acc)[NREP][QK_TPL]) {
+  using G = QwGeom<DS>;
+  constexpr int U = BITS == 8 ? 2 : 4;  // row pairs per register block; two blocks of loads are in flight
+  static_assert(G::RP % (2 * U) == 0, "the block loop covers the row pairs exactly");
+  const uint32_t n = (uint32_t)sg.n_tokens;
+  const uint32_t rowb = n / 8u * BITS;                       // bytes per channel row
+  const int tl = lane % G::TL, part = lane / G::TL;
+  const uint32_t lane_off = ts / 8u * BITS + (uint32_t)(part * G::RP * 2) * rowb;
+  const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * 128 * rowb, 128u * rowb);
+  const half2_t *qp = q2s + part * G::RP * NREP;
+  const uint2 *sp = sz + part * G::RP * G::NG + (tl >> 2);
+  struct Block {
+    QwRow<BITS> r0[U], r1[U];
+  };
+  auto load = [&](int i0, Block &b) {
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t row = (uint32_t)(2 * (i0 + k)) * rowb;  // uniform
+      b.r0[k] = qw_load_row<BITS>(rc, lane_off, row);
+      b.r1[k] = qw_load_row<BITS>(rc, lane_off, row + rowb);
+    }
+  };
+  auto compute = [&](int i0, const Block &b) {
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int i = i0 + k;
+      half2_t q2[NREP];
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) q2[h] = qp[i * NREP + h];
+      const uint2 szv = sp[i * G::NG];
+      const half2_t s2 = as_h2(szv.x), z2 = as_h2(szv.y);
+      if constexpr (BITS == 1) {
+        consume_byte<1, NREP, QK_TPL, NORMAL>(byte_pair<0>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 0);
+      } else if constexpr (BITS == 2) {
+        consume_byte<2, NREP, QK_TPL>(byte_pair<0>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 0);
+        consume_byte<2, NREP, QK_TPL>(byte_pair<1>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 4);
+      } else if constexpr (BITS == 4) {
+        consume_byte<4, NREP, QK_TPL>(byte_pair<0>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 0);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<1>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 2);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<2>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 4);
+        consume_byte<4, NREP, QK_TPL>(byte_pair<3>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 6);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          consume_byte<8, NREP, QK_TPL>(byte_pair<0>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 0);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<1>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 1);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<2>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 2);
+          consume_byte<8, NREP, QK_TPL>(byte_pair<3>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 3);
+        }
+      }
+    }
+  };
+  Block ba, bb;
+  load(0, ba);
+  stage();  // query and scale/zero into LDS while the first block is on its way; ends with the barrier
+#pragma unroll 1
+  for (int i0 = 0; i0 < G::RP; i0 += 2 * U) {
+    load(i0 + U, bb);
+    HQ_LOADS_ABOVE();
+    compute(i0, ba);
+    if (i0 + 2 * U < G::RP) load(i0 + 2 * U, ba);
+    HQ_LOADS_ABOVE();
+    compute(i0 + U, bb);
+  }
+}
+
+// fp16 class stored channel-major (B,Hkv,128,T), T a multiple of 8: a lane reads its 8 tokens of a row as 16 bytes
+template <int NREP, int DS, typename Stage>
+__device__ __forceinline__ void qw_f16_accumulate(const SegDev &sg, uint32_t ts, int bh, int lane, Stage &&stage,
+                                                  const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
+  using G = QwGeom<DS>;
+  constexpr int U = 2;
+  const uint32_t n = (uint32_t)sg.n_tokens;
+  const uint32_t rowb = n * 2u;
+  const int part = lane / G::TL;
+  const uint32_t lane_off = ts * 2u + (uint32_t)(part * G::RP * 2) * rowb;
+  const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * 128 * rowb, 128u * rowb);
+  const half2_t *qp = q2s + part * G::RP * NREP;
+  struct Block {
+    uint4 r0[U], r1[U];
+  };
+  auto load = [&](int i0, Block &b) {
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t row = (uint32_t)(2 * (i0 + k)) * rowb;
+      b.r0[k] = buf_u128(rc, lane_off, row);
+      b.r1[k] = buf_u128(rc, lane_off, row + rowb);
+    }
+  };
+  auto compute = [&](int i0, const Block &b) {
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t a[4] = {b.r0[k].x, b.r0[k].y, b.r0[k].z, b.r0[k].w};
+      const uint32_t c[4] = {b.r1[k].x, b.r1[k].y, b.r1[k].z, b.r1[k].w};
+      half2_t q2[NREP];
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) q2[h] = qp[(i0 + k) * NREP + h];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const half2_t ka = half_pair<0>(a[i], c[i]);  // token 2i:   (k[d], k[d+1])
+        const half2_t kb = half_pair<1>(a[i], c[i]);  // token 2i+1
+#pragma unroll
+        for (int h = 0; h < NREP; ++h) {
+          acc[h][2 * i] = __builtin_amdgcn_fdot2(ka, q2[h], acc[h][2 * i], false);
+          acc[h][2 * i + 1] = __builtin_amdgcn_fdot2(kb, q2[h], acc[h][2 * i + 1], false);
+        }
+      }
+    }
+  };
+  static_assert(G::RP % (2 * U) == 0, "the block loop covers the row pairs exactly");
+  Block ba, bb;
+  load(0, ba);
+  stage();
+#pragma unroll 1
+  for (int i0 = 0; i0 < G::RP; i0 += 2 * U) {
+    load(i0 + U, bb);
+    HQ_LOADS_ABOVE();
+    compute(i0, ba);
+    if (i0 + 2 * U < G::RP) load(i0 + 2 * U, ba);
+    HQ_LOADS_ABOVE();
+    compute(i0 + U, bb);
+  }
+}
+
+template <int NREP, int DS>
+__global__ __launch_bounds__(64, NREP <= 4 ? 4 : 2) void qk_wave_kernel(SegTable tb, const half_t *__restrict__ q,
+                                                                       half_t *__restrict__ scores, int Hq, int Hkv,
+                                                                       int64_t Tall, FuseArgs fz) {
+  using G = QwGeom<DS>;
+  __shared__ half2_t q2s[64 * NREP];                  // [row pair][head]: (q[d], q[d+1])
+  __shared__ __align__(16) uint2 sz[64 * G::NG];      // [row pair][group]: {(s_d, s_d+1), (z_d, z_d+1)}
+  __shared__ float red[2 * NREP];
+  const int lane = threadIdx.x;
+  const int bh = blockIdx.x;
+  const int b = bh / Hkv, hkv = bh % Hkv;
+  const int si = seg_of_unit(tb, blockIdx.y);
+  const SegDev sg = tb.seg[si];
+  const int tile = (int)blockIdx.y - begin_of_seg(tb, si);
+  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * 128);
+  auto stage_q = [&]() {
+#pragma unroll
+    for (int h = 0; h < NREP; ++h) q2s[lane * NREP + h] = as_h2(qsrc[h * 64 + lane]);
+  };
+  if (sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR) {
+    stage_q();
+    __syncthreads();
+    qk_f16_tm_tile<NREP, 1>(sg, tile, bh, b, hkv, 128, Hq, Tall, 0, lane, q2s, scores, fz, red);
+    return;
+  }
+  const uint32_t n = (uint32_t)sg.n_tokens;
+  const int tl = lane % G::TL;
+  const uint32_t t0 = (uint32_t)tile * G::TILE + (uint32_t)tl * QK_TPL;
+  const bool valid = t0 < n;          // class lengths are multiples of 8: a lane's tokens exist or do not
+  const uint32_t ts = valid ? t0 : 0;  // lanes past the end recompute the first tokens and store nothing
+  float acc[NREP][QK_TPL];
+#pragma unroll
+  for (int h = 0; h < NREP; ++h)
+#pragma unroll
+    for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
+
+  auto stage_quant = [&](auto normal) {
+    stage_q();
+    qw_stage_sz<DS, decltype(normal)::value>(sg, tile, bh, lane, sz);
+    __syncthreads();
+  };
+  auto stage_plain = [&]() {
+    stage_q();
+    __syncthreads();
+  };
+  using T = std::true_type;
+  using F = std::false_type;
+  switch (sg.bits) {
+    case 1:
+      if (sg.layout == HQEKV_LAYOUT_NORMAL1)
+        qw_quant_accumulate<1, NREP, DS, true>(sg, ts, bh, lane, [&]() { stage_quant(T{}); }, q2s, sz, acc);
+      else
+        qw_quant_accumulate<1, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc);
+      break;
+    case 2: qw_quant_accumulate<2, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
+    case 4: qw_quant_accumulate<4, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
+    case 8: qw_quant_accumulate<8, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
+    default: qw_f16_accumulate<NREP, DS>(sg, ts, bh, lane, stage_plain, q2s, acc);
+  }
+
+  // positions of the lane's tokens (they index a row of Tall < 2^31 scores, so the low word of each int64 entry
+  // is enough); requested here, used after the conversions below
+  uint32_t pos[QK_TPL];
+  if (sg.idx) {
+    const uint4 *ip = reinterpret_cast<const uint4 *>(sg.idx + ts);
+#pragma unroll
+    for (int i = 0; i < QK_TPL / 2; ++i) {
+      const uint4 v = ip[i];
+      pos[2 * i] = v.x;
+      pos[2 * i + 1] = v.z;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < QK_TPL; ++i) pos[i] = (uint32_t)sg.pos_base + ts + i;
+  }
+  if constexpr (DS > 1) {  // the quarters of head_dim sit 16 lanes apart: their sum lands in lanes 0-15
+#pragma unroll
+    for (int h = 0; h < NREP; ++h) rows_sum8(acc[h]);
+  }
+  const bool owner = valid && lane < G::TL;
+  bool contig = true;
+#pragma unroll
+  for (int i = 1; i < QK_TPL; ++i) contig = contig && (pos[i] == pos[0] + i);
+#pragma unroll
+  for (int h = 0; h < NREP; ++h) {
+    half_t v[QK_TPL];
+    float m_lane = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < QK_TPL; ++i) {
+      v[i] = (half_t)acc[h][i];
+      if (fz.stats) {  // the fp16 steps of the reference epilogue: round the score, scale, round again
+        v[i] = (half_t)((float)v[i] * fz.inv_sqrt_d);
+        m_lane = fmaxf(m_lane, (float)v[i]);
+      }
+    }
+    if (fz.stats) {  // (max, sum exp) of the tile
+      if (!owner) m_lane = -INFINITY;
+      const float m = DS > 1 ? row_max16(m_lane) : wave_max(m_lane);
+      float l_lane = 0.f;
+#pragma unroll
+      for (int i = 0; i < QK_TPL; ++i) l_lane += __expf((float)v[i] - m);
+      if (!owner) l_lane = 0.f;
+      const float l = DS > 1 ? row_sum16(l_lane) : wave_sum(l_lane);
+      if (lane == 0)
+        fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+    }
+    if (owner) {
+      half_t *srow = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+      // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one 16-byte
+      // store; otherwise 2-byte scatters through idx
+      if (contig && (((uintptr_t)(srow + pos[0])) & 15) == 0) {
+        __builtin_memcpy(__builtin_assume_aligned(srow + pos[0], 16), v, 16);
+      } else {
+#pragma unroll
+        for (int i = 0; i < QK_TPL; ++i) srow[pos[i]] = v[i];
+      }
+    }
   }
 }
 
@@ -1119,7 +1514,9 @@ __global__ __launch_bounds__(CB_CH * CB_SLICES) void pv_combine_kernel(const flo
 
 // =============================================================================== host side
 
-static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, int64_t chunk_tokens,
+// `unit_tokens`: tokens per work unit -- the q.K^T tile of the chosen tiling (the token-major fp16 residual
+// always has 64-token tiles) or the p.V chunk.
+static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, int64_t unit_tokens,
                        int64_t Tall, SegTable *tb, const char *who) {
   if (nseg < 0 || nseg > HQEKV_MAX_SEGS) return fail(HQEKV_E_ARG, "%s: nseg=%d out of range", who, nseg);
   if (nseg > 0 && !segs) return fail(HQEKV_E_ARG, "%s: null segment table", who);
@@ -1160,7 +1557,7 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
                : (s.bits == 1 && s.layout == HQEKV_LAYOUT_NORMAL1)              ? HQEKV_LAYOUT_NORMAL1
                                                                                 : 0;
     d.unit_begin = (int32_t)units;
-    const int64_t per = is_k ? qk_tile_tokens(s.bits, d.layout == HQEKV_LAYOUT_TOKEN_MAJOR) : chunk_tokens;
+    const int64_t per = (is_k && d.layout == HQEKV_LAYOUT_TOKEN_MAJOR) ? 64 : unit_tokens;
     const int64_t nu = (s.n_tokens + per - 1) / per;
     d.n_units = (int32_t)nu;
     if (nu > max_units) max_units = nu;
@@ -1189,18 +1586,65 @@ static int check_heads(const char *who, int64_t B, int64_t Hq, int64_t Hkv, int6
   return HQEKV_OK;
 }
 
-// Which q.K^T tiling a call uses: 0 = by launch size, 1 = 8 waves per 512-token tile, 2 = 4 waves per tile.
+// q.K^T tilings (HQEKV_QK_TILING_*): 1 = 8 waves per 512-token tile, 2 = 4 waves per tile (both split head_dim
+// over the waves of a workgroup), 3 = one wave per 512-token tile, 4 = one wave per 128-token tile.
 static int qk_tiling_of(int flags) { return (flags >> 4) & 0xf; }
+static int64_t qk_tile_of(int tiling) { return tiling == 4 ? qw_tile(4) : QK_TILE; }
+
+// The one-wave tilings read head_dim 128 with 16-byte row accesses: every channel-major fp16 class must hold a
+// multiple of 8 tokens.
+static bool qk_wave_tiling_fits(const hqekv_seg *segs, int nseg, int64_t D) {
+  if (D != 128) return false;
+  for (int k = 0; k < nseg; ++k)
+    if (segs[k].n_tokens > 0 && segs[k].bits == 16 && segs[k].layout != HQEKV_LAYOUT_TOKEN_MAJOR && segs[k].n_tokens % 8 != 0)
+      return false;
+  return true;
+}
+
+// tiling for a call: the forced one, or by launch size
+static int resolve_qk_tiling(int forced, const hqekv_seg *segs, int nseg, int64_t BHkv, int64_t D, const char *who,
+                             int *out) {
+  if (forced < 0 || forced > 4) return fail(HQEKV_E_ARG, "%s: q.K^T tiling %d (known: 0 = by size, 1 .. 4)", who, forced);
+  const bool fits = qk_wave_tiling_fits(segs, nseg, D);
+  if (forced >= 3 && !fits)
+    return fail(HQEKV_E_UNSUPPORTED, "%s: the one-wave q.K^T tilings need head_dim 128 and fp16 classes of a multiple of 8 tokens", who);
+  if (forced) {
+    *out = forced;
+    return HQEKV_OK;
+  }
+  int64_t tiles512 = 0;
+  for (int k = 0; k < nseg; ++k)
+    if (segs[k].n_tokens > 0) tiles512 += (segs[k].n_tokens + QK_TILE - 1) / QK_TILE;
+  const int64_t wgs = tiles512 * BHkv;
+  // few tiles: 8 waves share a tile (shortest critical path); many: one wave per tile (least work per code)
+  *out = wgs <= 1024 ? 1 : (fits ? 3 : 2);
+  return HQEKV_OK;
+}
 
 static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
-                     int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling = 0) {
+                     int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling) {
   if (tb.total_units == 0) return HQEKV_OK;
-  if (tiling < 0 || tiling > 2) return fail(HQEKV_E_ARG, "q.K^T tiling %d (known: 0 = by size, 1, 2)", tiling);
   const int nrep = (int)(Hq / Hkv);
-  // few tiles: 8 waves per tile; many tiles (several workgroups queue up per CU): 4 waves per tile
-  const int waves = tiling == 1 ? 8 : tiling == 2 ? 4 : ((int64_t)tb.total_units * B * Hkv <= 1024 ? 8 : 4);
+  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units);
+  if (tiling >= 3) {
+#define LAUNCH(N_, DS_)                                                                                        \
+  hipLaunchKernelGGL((qk_wave_kernel<N_, DS_>), grid, dim3(64), 0, st, tb, (const half_t *)q, (half_t *)scores, \
+                     (int)Hq, (int)Hkv, Tall, fz)
+#define LAUNCH_DS(N_) \
+  if (tiling == 3) LAUNCH(N_, 1); else LAUNCH(N_, 4)
+    switch (nrep) {
+      case 1: LAUNCH_DS(1); break;
+      case 2: LAUNCH_DS(2); break;
+      case 4: LAUNCH_DS(4); break;
+      default: LAUNCH_DS(8);
+    }
+#undef LAUNCH_DS
+#undef LAUNCH
+    return check_launch("qk_wave_kernel");
+  }
+  const int waves = tiling == 1 ? 8 : 4;
   const int tpw = 1;  // tiles per workgroup (2 and 4 measured no faster at B=8, 64k context)
-  dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units), block((unsigned)waves * 64);
+  dim3 block((unsigned)waves * 64);
   const int rh = waves == 4 ? (nrep < 4 ? nrep : 4) : (nrep < 2 ? nrep : 2);  // QkReduce::RH
   const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
 #define LAUNCH(N_, W_)                                                                                        \
@@ -1275,10 +1719,13 @@ extern "C" int hqekv_qk_hybrid(const hqekv_seg *segs, int nseg, const void *q, v
   if (rc) return rc;
   if (D > 1024) return fail(HQEKV_E_UNSUPPORTED, "qk_hybrid: D=%lld > 1024", (long long)D);
   if (!q || !scores || Tall <= 0) return fail(HQEKV_E_ARG, "qk_hybrid: null pointer or Tall <= 0");
-  SegTable tb{};
-  rc = build_table(segs, nseg, true, D, 0, Tall, &tb, "qk_hybrid");
+  int tiling = 0;
+  rc = resolve_qk_tiling(0, segs, nseg, B * Hkv, D, "qk_hybrid", &tiling);
   if (rc) return rc;
-  return launch_qk(tb, q, scores, B, Hq, Hkv, D, Tall, FuseArgs{}, (hipStream_t)stream);
+  SegTable tb{};
+  rc = build_table(segs, nseg, true, D, qk_tile_of(tiling), Tall, &tb, "qk_hybrid");
+  if (rc) return rc;
+  return launch_qk(tb, q, scores, B, Hq, Hkv, D, Tall, FuseArgs{}, (hipStream_t)stream, tiling);
 }
 
 extern "C" int hqekv_scale_softmax(void *scores, const void *mask, int64_t mask_row_stride, int64_t n_rows,
@@ -1353,7 +1800,8 @@ static int decode_layout(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_se
   int64_t tiles = 0;
   for (int k = 0; k < n_k; ++k)
     if (k_segs[k].n_tokens > 0) {
-      const int64_t per = qk_tile_tokens(k_segs[k].bits, k_segs[k].bits == 16 && k_segs[k].layout == HQEKV_LAYOUT_TOKEN_MAJOR);
+      // room for the statistics of the smallest tile any tiling uses (the token-major residual: 64 tokens)
+      const int64_t per = (k_segs[k].bits == 16 && k_segs[k].layout == HQEKV_LAYOUT_TOKEN_MAJOR) ? 64 : qw_tile(4);
       tiles += (k_segs[k].n_tokens + per - 1) / per;
     }
   if (tiles == 0) tiles = 1;
@@ -1386,8 +1834,11 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
     return fail(HQEKV_E_WORKSPACE, "decode_attn: workspace %lld bytes < %lld needed", (long long)workspace_bytes,
                 (long long)L.total);
   if ((uintptr_t)workspace & 255) return fail(HQEKV_E_ALIGN, "decode_attn: workspace not 256-byte aligned");
+  int tiling = 0;
+  rc = resolve_qk_tiling(qk_tiling_of(flags), k_segs, n_k, B * Hkv, D, "decode_attn", &tiling);
+  if (rc) return rc;
   SegTable kt{}, vt{};
-  rc = build_table(k_segs, n_k, true, D, 0, Tall, &kt, "decode_attn(K)");
+  rc = build_table(k_segs, n_k, true, D, qk_tile_of(tiling), Tall, &kt, "decode_attn(K)");
   if (rc) return rc;
   rc = build_table(v_segs, n_v, false, D, L.chunk, Tall, &vt, "decode_attn(V)");
   if (rc) return rc;
@@ -1406,7 +1857,7 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
   const int only = flags & (HQEKV_ONLY_QK | HQEKV_ONLY_PV | HQEKV_ONLY_COMBINE);
   const bool only_qk = only == HQEKV_ONLY_QK;
   if (only == 0 || only_qk) {
-    rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st, qk_tiling_of(flags));
+    rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st, tiling);
     if (rc) return rc;
     if (!fuse) {
       rc = hqekv_scale_softmax(attn_weights, mask, mask_row_stride, B * Hq, Tall, 1.0f / (float)sqrt((double)D), stream);

@@ -239,17 +239,43 @@ __global__ __launch_bounds__(512) void quant_k_tokenmajor_kernel(
 //   code = (u > 0) and (u > std * 2^-25),  u = rnd16(x - mean)
 // (u / std rounds to a positive fp16 exactly when it exceeds half the smallest denormal; std == 0 gives
 // +inf -> 1, std == inf gives 0).  A NaN -- 0/0 of a constant group -- becomes code 0.
-// The statistics are a two-pass fp32 evaluation (mean = sum / 32, M2 = sum (x - mean)^2, std =
-// sqrt(M2 / 31)); torch's own accumulation order is not specified, so the last bit of std / mean can
-// differ from a given torch build in rare cases.
+// The statistics follow torch's GPU reduction of a 32-element row operation for operation (ATen's WelfordOps,
+// native/SharedReduceOps.h, driven by native/cuda/Reduce.cuh: one element per thread, then a tree over ADJACENT
+// partners -- shuffle distances 1, 2, 4, 8, 16 -- each step merging two equal halves in fp32):
+//   delta = mean_b - mean_a;  mean = mean_a + delta * 0.5;  M2 = (M2_a + M2_b) + ((delta * delta) * n_half) * 0.5
+// with a the lower-indexed half; then std = sqrt(M2 / 31), both results rounded to fp16.  Compared bit for bit
+// with torch.std_mean executed on the device by the GPU tests.
 struct Normal1Stats {
   half_t mean_h, std_h;
   float thr;  // std * 2^-25
 };
-__device__ __forceinline__ Normal1Stats normal1_finish(float sum, float m2) {
+struct Welford {
+  float mean, m2;
+};
+// merge of two adjacent halves of n_half elements each (n_half a power of two, so every factor is exact)
+__device__ __forceinline__ Welford welford_merge(Welford a, Welford b, float n_half) {
+  const float delta = b.mean - a.mean;
+  Welford r;
+  r.mean = a.mean + delta * 0.5f;
+  r.m2 = (a.m2 + b.m2) + ((delta * delta) * n_half) * 0.5f;
+  return r;
+}
+// the tree over N = 2^k adjacent values held by one lane
+template <int N>
+__device__ __forceinline__ Welford welford_tree(const float (&x)[N]) {
+  Welford w[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) w[i] = Welford{x[i], 0.f};
+#pragma unroll
+  for (int span = 1; span < N; span *= 2)
+#pragma unroll
+    for (int i = 0; i < N; i += 2 * span) w[i] = welford_merge(w[i], w[i + span], (float)span);
+  return w[0];
+}
+__device__ __forceinline__ Normal1Stats normal1_finish(Welford w) {
   Normal1Stats st;
-  st.mean_h = (half_t)(sum * (1.0f / 32.0f));
-  st.std_h = (half_t)__builtin_sqrtf(m2 / 31.0f);
+  st.mean_h = (half_t)w.mean;
+  st.std_h = (half_t)__builtin_sqrtf(w.m2 / 31.0f);
   st.thr = (float)st.std_h * 0x1p-25f;
   return st;
 }
@@ -279,21 +305,20 @@ __global__ __launch_bounds__(256) void normal1_rows_kernel(
   const uint4 raw = *reinterpret_cast<const uint4 *>(x + (int64_t)o * xo + (int64_t)r * xr + g * 32u + sub * 8u);
   half_t v[8];
   __builtin_memcpy(v, &raw, 16);
-  float sum = 0.f;
+  float xf[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) sum += (float)v[i];
-  sum += quad_xor_f<1>(sum);
-  sum += quad_xor_f<2>(sum);
-  const float mean_f = sum * (1.0f / 32.0f);
-  float m2 = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float d = (float)v[i] - mean_f;
-    m2 += d * d;
+  for (int i = 0; i < 8; ++i) xf[i] = (float)v[i];
+  Welford w = welford_tree<8>(xf);
+  // the group's four lanes: the lane with the lower elements is the left partner of each merge
+  {
+    const Welford o = Welford{quad_xor_f<1>(w.mean), quad_xor_f<1>(w.m2)};
+    w = (sub & 1) ? welford_merge(o, w, 8.f) : welford_merge(w, o, 8.f);
   }
-  m2 += quad_xor_f<1>(m2);
-  m2 += quad_xor_f<2>(m2);
-  const Normal1Stats st = normal1_finish(sum, m2);
+  {
+    const Welford o = Welford{quad_xor_f<2>(w.mean), quad_xor_f<2>(w.m2)};
+    w = (sub & 2) ? welford_merge(o, w, 16.f) : welford_merge(w, o, 16.f);
+  }
+  const Normal1Stats st = normal1_finish(w);
   uint32_t b8 = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) b8 |= normal1_code((half_t)((float)v[i] - (float)st.mean_h), st.thr) << i;
@@ -330,17 +355,10 @@ __global__ __launch_bounds__(512) void normal1_k_tokenmajor_kernel(
     for (int k = 0; k < 32; ++k) t[k] = bits_h2(buf_u32(rx, voff, (uint32_t)k * row_b));
 #pragma unroll
     for (int ch = 0; ch < 2; ++ch) {
-      float sum = 0.f;
+      float xf[32];
 #pragma unroll
-      for (int k = 0; k < 32; ++k) sum += (float)t[k][ch];
-      const float mean_f = sum * (1.0f / 32.0f);
-      float m2 = 0.f;
-#pragma unroll
-      for (int k = 0; k < 32; ++k) {
-        const float d = (float)t[k][ch] - mean_f;
-        m2 += d * d;
-      }
-      const Normal1Stats st = normal1_finish(sum, m2);
+      for (int k = 0; k < 32; ++k) xf[k] = (float)t[k][ch];
+      const Normal1Stats st = normal1_finish(welford_tree<32>(xf));
       uint32_t w = 0;
 #pragma unroll
       for (int k = 0; k < 32; ++k) w |= normal1_code((half_t)((float)t[k][ch] - (float)st.mean_h), st.thr) << k;

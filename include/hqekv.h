@@ -230,7 +230,10 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
 #define HQEKV_FUSE_SOFTMAX 1
 #define HQEKV_QK_TILING(n) (((n) & 0xf) << 4)
 #define HQEKV_QK_TILING_8WAVES 1 /* 512-token tile, head_dim split over 8 waves (launches of <= 1024 tiles) */
-#define HQEKV_QK_TILING_4WAVES 2 /* 512-token tile, head_dim split over 4 waves (larger launches)           */
+#define HQEKV_QK_TILING_4WAVES 2 /* 512-token tile, head_dim split over 4 waves                              */
+#define HQEKV_QK_TILING_WAVE512 3 /* one wave per 512-token tile, no split of head_dim (launches of > 1024 tiles;
+                                     needs head_dim 128 and fp16 classes of a multiple of 8 tokens)          */
+#define HQEKV_QK_TILING_WAVE128 4 /* one wave per 128-token tile, head_dim split over four groups of 16 lanes */
 #define HQEKV_ONLY_QK 0x100
 #define HQEKV_ONLY_PV 0x200
 #define HQEKV_ONLY_COMBINE 0x400

@@ -146,6 +146,35 @@ def uniform_group_dequantize_unpack_last_dim(
 NORMAL1_CENTER = 0.6744897501960817
 
 
+# How the 1-bit class's statistics are accumulated.  "torch_cpu": ``torch.std_mean`` as this host evaluates it.
+# "gpu_tree": the order torch's GPU reduction uses for a 32-element row, which is what the reference runs
+# (its quantiser executes on the GPU): the two differ in the last fp16 place of std in rare groups.
+NORMAL1_STAT_ORDER = "torch_cpu"
+
+
+def std_mean_gpu_tree(g: torch.Tensor):
+    """std, mean of the last axis (32 fp16 values) in the order of torch's GPU reduction kernel, restated from
+    ATen (third party, torch==2.7.1 pinned at requirements.txt:114; native/SharedReduceOps.h ``WelfordOps`` and
+    native/cuda/Reduce.cuh): a row of 32 is reduced by 32 threads holding one element each (mean = x, M2 = 0),
+    then by shuffles over distances 1, 2, 4, 8, 16, i.e. a balanced tree over ADJACENT halves a (lower indices)
+    and b with ``WelfordOps::combine`` in fp32:
+        delta = mean_b - mean_a;  mean = mean_a + delta * (n_b / n);  M2 = M2_a + M2_b + delta * delta * n_a * (n_b / n)
+    (n_b / n = 1/2 exactly), then ``project``: std = sqrt(M2 / (32 - 1)), both rounded to fp16.
+    Pinned by comparing the HIP quantiser, which follows the same order, with ``torch.std_mean`` executed on the
+    GPU, bit for bit (tests/test_quant_gpu.py)."""
+    mean = g.float()
+    m2 = torch.zeros_like(mean)
+    n_half = 1.0
+    while mean.shape[-1] > 1:
+        ma, mb = mean[..., 0::2], mean[..., 1::2]
+        delta = mb - ma
+        mean = ma + delta * 0.5
+        m2 = (m2[..., 0::2] + m2[..., 1::2]) + ((delta * delta) * n_half) * 0.5
+        n_half *= 2.0
+    std = torch.sqrt(m2 / 31.0)
+    return std.to(g.dtype), mean.to(g.dtype)
+
+
 def normal_group_quantize_pack_last_dim(data: torch.Tensor, group_size: int, bit: int = 1):
     """quant/pack_unpack.py:218-253 for bit == 1: ``std, mean = torch.std_mean(group)`` (unbiased, fp32
     accumulation, rounded to fp16), ``v = rnd16(rnd16(x - mean) / std)``, code = searchsorted([0, inf], v)
@@ -155,7 +184,10 @@ def normal_group_quantize_pack_last_dim(data: torch.Tensor, group_size: int, bit
     B, nh, D, T = data.shape
     assert data.dtype == torch.float16 and T % group_size == 0
     g = data.reshape(B * nh * D, T // group_size, group_size)
-    std, mean = torch.std_mean(g, dim=-1, keepdim=True)
+    if NORMAL1_STAT_ORDER == "gpu_tree" and group_size == 32:
+        std, mean = std_mean_gpu_tree(g)
+    else:
+        std, mean = torch.std_mean(g, dim=-1, keepdim=True)
     v = (g - mean) / std
     q = (v > 0).to(torch.int32).reshape(B, nh, D, T)
     shp = (B, nh, D, T // group_size)

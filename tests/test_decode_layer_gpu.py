@@ -33,16 +33,6 @@ def _causal_mask(T):
 def _same_tuple(got, want, where, normal=False):
     assert len(got) == len(want) == 42
     for i, (a, b) in enumerate(zip(got, want)):
-        if normal and i in (28, 30, 31, 32, 34, 35) and a is not None and b is not None:
-            # normal-quantile 1-bit class: std / mean may differ in the last fp16 place in rare groups
-            # (torch.std_mean's accumulation order is not pinned), and with them the odd code next to the mean
-            a = a.cpu()
-            assert a.shape == b.shape and a.dtype == b.dtype, (where, i)
-            if a.dtype == torch.float16:
-                assert torch.allclose(a.float(), b.float(), rtol=2e-3, atol=1e-6), (where, i)
-            else:
-                assert float((a != b).float().mean()) < 0.02, (where, i)
-            continue
         if i == 41:
             assert int(a) == int(b), (where, i)
             continue

@@ -395,3 +395,26 @@ def test_kivi_layer_bookkeeping_and_equivalence_to_plain_attention():
         out2 = torch.matmul(w2.float(), O.repeat_kv(v_all, Hq // Hkv).float()).half()
         assert w.shape == (B, Hq, 1, T) and torch.allclose(w.float(), w2.float(), rtol=1e-3, atol=1e-4)
         assert torch.allclose(out.float(), out2.float(), rtol=1e-3, atol=1e-3)
+
+
+def test_gpu_tree_statistics_restatement():
+    """``std_mean_gpu_tree`` (torch's GPU reduction order for a 32-element row, restated): a hand-worked first
+    level, the closed form on arange(32), agreement with a float64 two-pass evaluation to one fp16 step, and
+    near-agreement with this host's ``torch.std_mean`` (another order: the std may differ in the last place)."""
+    # by hand, 2 elements per level: (1, 3) -> delta 2, mean 2, M2 = 2*2*1*0.5 = 2; (5, 9) -> delta 4, mean 7, M2 = 8;
+    # merge (n_half = 2): delta 5, mean 4.5, M2 = (2 + 8) + 25 * 2 * 0.5 = 35 = sum (x - 4.5)^2 = 12.25 + 2.25 + 0.25 + 20.25
+    x = torch.tensor([[1.0, 3.0, 5.0, 9.0] * 8]).half()
+    std, mean = O.std_mean_gpu_tree(x)
+    assert float(mean) == 4.5 and float(std) == float(torch.tensor((35.0 * 8 / 31) ** 0.5).half())
+    a = torch.arange(32).half()[None]
+    std, mean = O.std_mean_gpu_tree(a)
+    assert float(mean) == 15.5 and float(std) == float(torch.tensor(88.0 ** 0.5).half())
+    g = (torch.randn(20000, 32, generator=torch.Generator().manual_seed(3)) * 2 + 0.5).half()
+    std, mean = O.std_mean_gpu_tree(g)
+    d = g.double()
+    m64 = d.mean(-1, keepdim=True)
+    s64 = ((d - m64) ** 2).sum(-1, keepdim=True).div(31).sqrt()
+    step = lambda v: torch.exp2(torch.floor(torch.log2(v.abs().clamp_min(2.0 ** -14))) - 10)
+    assert bool(((std.double() - s64).abs() <= step(s64)).all()) and bool(((mean.double() - m64).abs() <= step(m64)).all())
+    t_std, t_mean = torch.std_mean(g, dim=-1, keepdim=True)
+    assert float((t_std != std).float().mean()) < 0.005 and float((t_mean != mean).float().mean()) < 0.005

@@ -48,23 +48,8 @@ def test_hqe2_policy_bit_exact_over_three_compressions(dev, strategy):
     got, _, _ = PC.run(prod, to_dev=lambda x: x.to(dev),
                        rank_blocks=lambda bs, bn, imp: get_block_token_idx(bs, bn, imp.to(dev)).cpu())
     want, _, _ = PC.run(orac)
-    normal = strategy != "uniform_group"
     for step, (g, w) in enumerate(zip(got, want)):
         for slot in range(42):
-            if normal and slot in (28, 30, 31, 32, 34, 35) and g[slot] is not None:
-                # std / mean of the normal-quantile class: torch.std_mean's accumulation order is not pinned,
-                # so the last fp16 place (and with it the odd code next to the mean) may differ in rare groups
-                a, b = g[slot].cpu(), w[slot]
-                assert a.shape == b.shape and a.dtype == b.dtype
-                if a.dtype == torch.int32:
-                    diff = (a ^ b).to(torch.int64) & 0xFFFFFFFF
-                    flipped = sum(int(((diff >> k) & 1).sum()) for k in range(32))
-                    assert flipped <= 0.002 * a.numel() * 32, (step, slot, flipped)
-                else:
-                    d = (a.float() - b.float()).abs()
-                    step16 = torch.exp2(torch.floor(torch.log2(b.float().abs().clamp_min(2.0 ** -14))) - 10)
-                    assert bool((d <= step16).all()) and float((d > 0).float().mean()) < 0.01, (step, slot)
-                continue
             _same(g[slot], w[slot], f"step {step} slot {slot}")
     _same(lw.weights, ring["cpu"], "ring of recent attention rows after eviction")
 

@@ -210,25 +210,24 @@ def _ulp16(x):
 
 @pytest.mark.parametrize("layout", ["rows", "token_major"])
 def test_normal1_quantiser_against_oracle(dev, layout):
-    """std / mean: the accumulation order of torch.std_mean is not pinned, so they may differ from the CPU
-    oracle in the last fp16 place in rare groups (asserted: <= 1 step, < 0.5 % of the groups); the codes must
-    be exactly what the reference's element-wise rule gives for the std / mean the kernel stored."""
+    """Codes, std and mean bit-identical to the oracle, whose statistics follow the tree order of torch's GPU
+    reduction (the order the kernels use).  Against ``torch.std_mean`` as THIS host's CPU evaluates it the std may
+    differ in the last fp16 place in rare groups (another accumulation order): asserted <= 1 step, < 0.5 %."""
     from hqekv_amd import pack_unpack as P
     x = (_data((2, 2, 64, 256), 77) * 2 + 0.5)
     data = x if layout == "rows" else x.transpose(2, 3)
     code, std, mean = P.normal_group_quantize_pack_last_dim(data.to(dev), 32, 1)
     oc, os_, om = O.normal_group_quantize_pack_last_dim(data.contiguous(), 32, 1)
     code, std, mean = code.cpu(), std.cpu(), mean.cpu()
-    assert code.shape == oc.shape and std.shape == os_.shape and code.dtype == torch.int32
-    for got, want in ((std, os_), (mean, om)):
+    assert torch.equal(code, oc)
+    assert torch.equal(std.view(torch.int16), os_.view(torch.int16)) and torch.equal(mean.view(torch.int16), om.view(torch.int16))
+    B, nh, R, L = data.shape
+    g = data.contiguous().reshape(B * nh * R, L // 32, 32)
+    c_std, c_mean = torch.std_mean(g, dim=-1)
+    for got, want in ((std, c_std.reshape(std.shape)), (mean, c_mean.reshape(mean.shape))):
         d = (got.float() - want.float()).abs()
         assert bool((d <= _ulp16(want.float())).all())
         assert float((d > 0).float().mean()) < 0.005
-    B, nh, R, L = data.shape
-    g = data.contiguous().reshape(B * nh * R, L // 32, 32)
-    v = (g - mean.reshape(B * nh * R, L // 32, 1)) / std.reshape(B * nh * R, L // 32, 1)
-    want_codes = (v > 0).to(torch.int32).reshape(B, nh, R, L)
-    assert torch.equal(O.unpack_codes(code, 1), want_codes)
 
 
 @pytest.mark.parametrize("layout", ["rows", "token_major"])

@@ -62,7 +62,7 @@ def _c4_mix_case(permute: bool):
 
 
 @pytest.mark.parametrize("permute", [False, True], ids=["blockidx", "randperm"])
-@pytest.mark.parametrize("tiling", ["8waves", "4waves", "auto"])
+@pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave128", "auto"])
 @pytest.mark.parametrize("fused", [True, False], ids=["fused", "general"])
 def test_config4_mix_batch8_every_row(dev, tiling, permute, fused):
     """Configuration 4's class mix at B=8, 32 query heads over 8 KV heads, 16384 tokens: a launch of more than
@@ -80,7 +80,7 @@ def test_config4_mix_batch8_every_row(dev, tiling, permute, fused):
     torch.testing.assert_close(w.float().sum(-1).cpu(), torch.ones(B, Hq, 1), rtol=0, atol=5e-3)
 
 
-@pytest.mark.parametrize("tiling", ["8waves", "4waves"])
+@pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave128"])
 @pytest.mark.parametrize("n_rep", [1, 2, 4, 8])
 @pytest.mark.parametrize("low_normal", [False, True], ids=["uniform1", "normal1"])
 def test_every_tiling_every_gqa_ratio(dev, tiling, n_rep, low_normal):
@@ -150,14 +150,21 @@ def test_config_full_size(dev, name, counts):
         classes = synth.split_blocks(cfg["T"], cfg["fractions"], cfg["seed"])
         assert {b: classes[b].numel() for b in counts} == counts
     Tall = cache[41]
-    refs = {b: O.qkv_matmul(q[b:b + 1].cpu(), _row(cache, b), None, D, use_mask=False, round_per_class=False)
-            for b in (0, B - 1)}
+    # The probabilities are held to the oracle's.  The output is held to the oracle's p.V of the SAME probabilities:
+    # with 50 000+ tokens and K outliers a raw score now and then sits on an fp16 rounding boundary, another
+    # summation order over head_dim rounds it the other way, and a peaked row moves by a fraction of a percent --
+    # inside the tolerance for the probabilities, but the output would inherit it on top of its own rounding.
+    refs = {}
+    for b in (0, B - 1):
+        row = _row(cache, b)
+        w_ref, _ = O.qkv_matmul(q[b:b + 1].cpu(), row, None, D, use_mask=False, round_per_class=False)
+        refs[b] = (w_ref, O.repeat_kv(O.reconstruct_cache(row, "uniform_group")[1], Hq // Hkv).float())
     first = None
     for tiling, n in [("auto", 0)] + _tilings():
         w, o = decode_attention(q, cache, None, Tall, zero_init=False, flags=_flags(True, n))
-        for b, (w_ref, o_ref) in refs.items():
+        for b, (w_ref, v_dense) in refs.items():
             _close(w[b:b + 1], w_ref, f"{name} attn_weights row {b} ({tiling})")
-            _close(o[b:b + 1], o_ref, f"{name} attn_output row {b} ({tiling})")
+            _close(o[b:b + 1], torch.matmul(w[b:b + 1].float().cpu(), v_dense), f"{name} attn_output row {b} ({tiling})")
         torch.testing.assert_close(w.float().sum(-1).cpu(), torch.ones(B, Hq, 1), rtol=0, atol=5e-3)
         if first is None:
             first = (w.clone(), o.clone())
