@@ -39,7 +39,7 @@ EXPORTS = (
     "hqekv_normal1_quant_pack_rows", "hqekv_normal1_quant_pack_k_tokenmajor", "hqekv_normal1_dequant_unpack_rows",
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group", "hqekv_gemv_normal_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
-    "hqekv_decode_workspace_bytes", "hqekv_decode_attn",
+    "hqekv_decode_workspace_bytes", "hqekv_decode_attn", "hqekv_decode_attn_static",
 )
 
 
@@ -83,7 +83,9 @@ _PROTOS = {
     "hqekv_pv_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "hqekv_decode_workspace_bytes": (_i64, [_SEGP, _int, _SEGP, _int, _i64, _i64, _i64, _i64]),
     "hqekv_decode_attn": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _int, _vp]),
+    "hqekv_decode_attn_static": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
 }
+STATIC_SCRATCH_BYTES = 8 << 20   # HQEKV_STATIC_SCRATCH_BYTES
 
 
 def lib_path() -> Path:

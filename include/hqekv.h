@@ -245,6 +245,20 @@ int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs,
                       int64_t D, int64_t Tall, void *workspace, int64_t workspace_bytes, int flags,
                       void *stream);
 
+/* No counterpart in the reference: hqekv_decode_attn for callers that cannot allocate (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc).  Same arguments minus the workspace: the split-K
+ * partials and softmax statistics go to a fixed buffer of HQEKV_STATIC_SCRATCH_BYTES inside the library's device
+ * image, one copy per GPU, held until the process ends; its address is looked up on the first call on a device.
+ * The call allocates and frees nothing.  A call whose hqekv_decode_workspace_bytes() exceeds the buffer returns
+ * HQEKV_E_WORKSPACE (use hqekv_decode_attn then).  All calls on one GPU share the buffer: calls that overlap in
+ * time on one GPU (two streams, two threads) race; calls ordered on one stream are fine.
+ */
+#define HQEKV_STATIC_SCRATCH_BYTES (8u << 20)
+int hqekv_decode_attn_static(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
+                             const void *q, const void *mask, int64_t mask_row_stride,
+                             void *attn_weights, void *attn_out, int64_t B, int64_t Hq, int64_t Hkv,
+                             int64_t D, int64_t Tall, int flags, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
