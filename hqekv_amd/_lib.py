@@ -40,6 +40,7 @@ EXPORTS = (
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group", "hqekv_gemv_normal_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
     "hqekv_decode_workspace_bytes", "hqekv_decode_attn", "hqekv_decode_attn_static",
+    "hqekv_cache_migrate",
 )
 
 
@@ -57,10 +58,25 @@ class Seg(C.Structure):
     ]
 
 
+class CacheClass(C.Structure):
+    """Mirror of ``struct hqekv_cache_class``."""
+    _fields_ = [
+        ("bits", C.c_int32),
+        ("layout", C.c_int32),
+        ("n_tokens", C.c_int64),
+        ("slab_tokens", C.c_int64),
+        ("data", C.c_void_p),
+        ("scale", C.c_void_p),
+        ("zero", C.c_void_p),
+        ("idx", C.c_void_p),
+    ]
+
+
 _lib: Optional[C.CDLL] = None
 
 _i64, _int, _vp = C.c_int64, C.c_int, C.c_void_p
 _SEGP = C.POINTER(Seg)
+_CCP = C.POINTER(CacheClass)
 
 _PROTOS = {
     "hqekv_version": (C.c_int, []),
@@ -84,6 +100,7 @@ _PROTOS = {
     "hqekv_decode_workspace_bytes": (_i64, [_SEGP, _int, _SEGP, _int, _i64, _i64, _i64, _i64]),
     "hqekv_decode_attn": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _int, _vp]),
     "hqekv_decode_attn_static": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
+    "hqekv_cache_migrate": (C.c_int, [_int, _CCP, _int, _CCP, _int, _vp, _i64, _i64, _vp]),
 }
 STATIC_SCRATCH_BYTES = 8 << 20   # HQEKV_STATIC_SCRATCH_BYTES
 

@@ -142,9 +142,14 @@ def idx_cover_once(idx_list, n: int) -> bool:
     hit = getattr(idx_list[0], "_hq_cover", None)   # rides on the first array, like the cache policy's host copies
     if hit is not None and hit[0] == key:
         return hit[1]
-    hosts = [getattr(t, "_hq_host", None) if getattr(t, "_hq_host_version", None) == t._version else None
-             for t in idx_list]
-    if all(h is not None for h in hosts):
+    trusted = [getattr(t, "_hq_host_version", None) == t._version for t in idx_list]
+    blocks = [getattr(t, "_hq_blocks", None) if ok_ else None for t, ok_ in zip(idx_list, trusted)]
+    hosts = [getattr(t, "_hq_host", None) if ok_ else None for t, ok_ in zip(idx_list, trusted)]
+    if n % 32 == 0 and all(b is not None and b.shape[0] * 32 == t.numel() for b, t in zip(blocks, idx_list)):
+        c = np.concatenate(blocks)   # whole aligned 32-token blocks: check the block numbers
+        nb = n // 32
+        ok = bool(c.size == nb and (c >= 0).all() and (c < nb).all() and (np.bincount(c, minlength=nb) == 1).all())
+    elif all(h is not None for h in hosts):
         c = np.concatenate(hosts)
         ok = bool(c.size == n and (c >= 0).all() and (c < n).all() and (np.bincount(c, minlength=n) == 1).all())
     else:

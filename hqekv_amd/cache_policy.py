@@ -13,13 +13,18 @@ in source order; a quantised source is dequantised (two fp16 roundings) and re-q
 whole 32-token groups.  After an eviction every surviving index is replaced by its rank among the
 survivors (quant/hqe_2.py:661-670).
 
-The reference re-copies whole class tensors with boolean masks; here a move gathers only the moved
-columns / rows with ``index_select`` and quantises them with one fused kernel (K straight from the
-token-major residual, no transpose copy).  Which token goes where is worked out on host copies of the
-position arrays (numpy), so a compression waits for the device only to fetch the two block rankings.
+Two engines produce the same bytes.  ``gather`` (the default wherever it applies): everything the reference
+moves is a whole block of 32 tokens and every block ends in exactly one place, so the host works out, per
+block, where each class's blocks come from (numpy over a few thousand entries), and ONE kernel launch per side
+(``hqekv_cache_migrate``) rebuilds all classes from the old ones and the new tokens -- survivors copied, demoted
+blocks dequantised and re-quantised, new blocks quantised, evicted blocks left out, positions re-ranked; the
+device is waited for once, to fetch the two block rankings.  ``steps``: the general engine for selections that
+are not made of whole aligned blocks (token-level V selections): the reference's sequence of moves with
+``index_select`` gathers and one quantiser call per move.
 """
 from __future__ import annotations
 
+import os
 import threading
 from typing import Dict, List, Optional
 
@@ -54,12 +59,32 @@ class _Cls:
 
 def _host_idx(t: torch.Tensor) -> np.ndarray:
     """Host copy of a position tensor.  Tensors made by this module carry theirs along (no device
-    round trip); for anyone else's the copy is fetched, which waits for the device."""
-    h = getattr(t, "_hq_host", None)
-    # the copy is trusted only while nobody has written to the tensor since it was attached
-    if h is None or h.shape[0] != t.numel() or getattr(t, "_hq_host_version", None) != t._version:
-        h = t.detach().to("cpu", torch.int64).numpy()
-    return h
+    round trip) -- token by token, or as the first positions of their 32-token blocks; for anyone else's the
+    copy is fetched, which waits for the device."""
+    trusted = getattr(t, "_hq_host_version", None) == t._version  # nobody wrote to the tensor since
+    h = getattr(t, "_hq_host", None) if trusted else None
+    if h is not None and h.shape[0] == t.numel():
+        return h
+    blocks = getattr(t, "_hq_blocks", None) if trusted else None
+    if blocks is not None and blocks.shape[0] * BLOCK == t.numel():
+        h = (blocks.astype(np.int64)[:, None] * BLOCK + np.arange(BLOCK, dtype=np.int64)).reshape(-1)
+        t._hq_host = h
+        return h
+    return t.detach().to("cpu", torch.int64).numpy()
+
+
+def _host_blocks(t: torch.Tensor) -> Optional[np.ndarray]:
+    """Block numbers (first position / 32) of a position tensor made of whole aligned blocks, else None."""
+    if getattr(t, "_hq_host_version", None) == t._version:
+        blocks = getattr(t, "_hq_blocks", None)
+        if blocks is not None and blocks.shape[0] * BLOCK == t.numel():
+            return blocks
+    if t.numel() % BLOCK:
+        return None
+    h = _host_idx(t).reshape(-1, BLOCK)
+    if h.size and (bool((h[:, 0] % BLOCK).any()) or not bool((h == h[:, :1] + np.arange(BLOCK)).all())):
+        return None
+    return (h[:, 0] // BLOCK).astype(np.int64)
 
 
 class _Staging:
@@ -349,10 +374,242 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[np
     return new, new_idx
 
 
+# ----------------------------------------------------------------------------------------------- gather engine
+# Everything below works on whole 32-token blocks.  A side's state is, per class, the block numbers (first position
+# / 32) of its blocks in stored order; a compression turns it into the same thing for the new classes plus, per new
+# block, where its bytes come from.
+
+_SRC_NEW = 5   # source slot of the new fp16 tokens (slots 0..4: the old fp16, 8, 4, 2, 1-bit classes)
+
+
+def _block_labels(sorted_idx: torch.Tensor, bit_num, total_blocks: int, order_h: Optional[np.ndarray]) -> Optional[np.ndarray]:
+    """label[b] = index of the target (fp16, 8, 4, 2, 1[, evict]) block b is ranked into, or None when the ranking
+    or the counts are not made of whole blocks covering every block once."""
+    counts = [int(v) for v in (bit_num.tolist() if torch.is_tensor(bit_num) else bit_num)]
+    if any(c % BLOCK or c < 0 for c in counts) or sum(counts) != total_blocks * BLOCK:
+        return None
+    if order_h is None:
+        order_h = _host_blocks(sorted_idx)
+    if order_h is None or order_h.shape[0] != total_blocks:
+        return None
+    label = np.full(total_blocks, -1, dtype=np.int8)
+    start = 0
+    for ti, c in enumerate(counts):
+        nb = c // BLOCK
+        label[order_h[start:start + nb]] = ti
+        start += nb
+    if (label < 0).any():   # a block ranked twice and another one never
+        return None
+    return label
+
+
+def _plan_side(old_blocks: Dict[int, Optional[np.ndarray]], hist_blocks: int, n_new_blocks: int, label: np.ndarray,
+               evicting: bool):
+    """-> (per class: (source slots, source blocks, old positions of the blocks), alive blocks ascending or None).
+
+    Normative order inside a class (quant/hqe_2.py:552-659): the members that stay, in their order; then the new
+    tokens ranked into it; then what comes down from the fp16, 8, 4 and 2-bit classes, each in source order.  A
+    block only ever moves to a lower precision; a block ranked into a higher one stays where it is."""
+    new_pos = np.arange(hist_blocks, hist_blocks + n_new_blocks, dtype=np.int64)
+    new_lab = label[new_pos]
+    final = {}
+    for ti, bits in enumerate(CLASS_BITS):
+        slots, srcs, poss = [], [], []
+        own = old_blocks.get(bits)
+        if own is not None and own.size:
+            lab = label[own]
+            stay = np.flatnonzero(lab <= ti)          # evict is the highest label; higher precision = lower label
+            slots.append(np.full(stay.size, ti, dtype=np.int64)); srcs.append(stay); poss.append(own[stay])
+        sel = np.flatnonzero(new_lab == ti)
+        slots.append(np.full(sel.size, _SRC_NEW, dtype=np.int64)); srcs.append(sel); poss.append(new_pos[sel])
+        for si in range(ti):                          # sources of higher precision, in the order 16, 8, 4, 2
+            src = old_blocks.get(CLASS_BITS[si])
+            if src is None or not src.size:
+                continue
+            sel = np.flatnonzero(label[src] == ti)
+            slots.append(np.full(sel.size, si, dtype=np.int64)); srcs.append(sel); poss.append(src[sel])
+        final[bits] = (np.concatenate(slots), np.concatenate(srcs), np.concatenate(poss))
+    alive = None
+    if evicting:
+        alive = np.flatnonzero(label != 5)
+    return final, alive
+
+
+def _carve(nbytes_list, dev):
+    """One allocation for all tensors of a side, each piece 256-byte aligned."""
+    offs, total = [], 0
+    for n in nbytes_list:
+        offs.append(total)
+        total += (n + 255) // 256 * 256
+    return torch.empty(max(total, 256), dtype=torch.uint8, device=dev), offs
+
+
+def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, final, rank_of: Optional[np.ndarray],
+                 strategy: str) -> Dict[int, _Cls]:
+    """Allocate the new classes of one side and fill them with one launch of the migration kernel."""
+    from . import _lib
+    B, H, n_new, D = new.shape
+    dev = new.device
+    low_layout = _lib.LAYOUT_NORMAL1 if strategy == LOW_NORMAL else 0
+    # ---- sources
+    src = (_lib.CacheClass * (_SRC_NEW + 1))()
+    keep = []
+    for si, bits in enumerate(CLASS_BITS):
+        c = side[bits]
+        if c.data is None:
+            continue
+        data = c.data if c.data.is_contiguous() else c.data.contiguous()
+        keep.append(data)
+        n = data.shape[3] * (1 if bits == 16 else 32 // bits) if is_k else data.shape[2]
+        src[si].bits, src[si].n_tokens, src[si].data = bits, n, data.data_ptr()
+        src[si].layout = low_layout if bits == 1 else 0
+        if bits != 16:
+            sc, zr = c.scale.contiguous(), c.zero.contiguous()
+            keep += [sc, zr]
+            src[si].scale, src[si].zero = sc.data_ptr(), zr.data_ptr()
+    # the new tokens are the head of a longer (B, H, T, D) tensor when a residual follows them: read in place
+    slab = n_new
+    if new.is_contiguous():
+        newc = new
+    elif new.stride(3) == 1 and new.stride(2) == D and new.stride(1) % D == 0 and new.stride(0) == H * new.stride(1):
+        newc, slab = new, new.stride(1) // D
+    else:
+        newc = new.contiguous()
+    keep.append(newc)
+    src[_SRC_NEW].bits, src[_SRC_NEW].n_tokens, src[_SRC_NEW].data = 16, n_new, newc.data_ptr()
+    src[_SRC_NEW].slab_tokens = slab
+    src[_SRC_NEW].layout = _lib.LAYOUT_TOKEN_MAJOR if is_k else 0
+    # ---- destinations: sizes, one allocation, views
+    pieces, sizes = [], []
+    for bits in CLASS_BITS:
+        n = final[bits][0].size * BLOCK
+        if n == 0:
+            continue
+        if bits == 16:
+            shapes = [((B, H, D, n) if is_k else (B, H, n, D), torch.float16)]
+        else:
+            pf = 32 // bits
+            if is_k:
+                shapes = [((B, H, D, n // pf), torch.int32), ((B, H, D, n // BLOCK), torch.float16), ((B, H, D, n // BLOCK), torch.float16)]
+            else:
+                shapes = [((B, H, n, D // pf), torch.int32), ((B, H, n, D // BLOCK), torch.float16), ((B, H, n, D // BLOCK), torch.float16)]
+        shapes.append(((n,), torch.int64))
+        for shp, dt in shapes:
+            pieces.append((bits, shp, dt))
+            sizes.append(int(np.prod(shp)) * torch.empty(0, dtype=dt).element_size())
+    out = {b: _Cls() for b in CLASS_BITS}
+    if not pieces:
+        return out
+    buf, offs = _carve(sizes, dev)
+    views: Dict[int, list] = {}
+    for (bits, shp, dt), off, nb in zip(pieces, offs, sizes):
+        views.setdefault(bits, []).append(buf[off:off + nb].view(dt).view(shp))
+    dst = (_lib.CacheClass * len(CLASS_BITS))()
+    n_dst = 0
+    plan_src, plan_pos = [], []
+    for bits in CLASS_BITS:
+        if bits not in views:
+            continue
+        slots, srcs, poss = final[bits]
+        v = views[bits]
+        d = dst[n_dst]
+        d.bits, d.n_tokens, d.data = bits, slots.size * BLOCK, v[0].data_ptr()
+        d.layout = low_layout if bits == 1 else 0
+        if bits != 16:
+            d.scale, d.zero = v[1].data_ptr(), v[2].data_ptr()
+        d.idx = v[-1].data_ptr()
+        n_dst += 1
+        pos = poss if rank_of is None else rank_of[poss]
+        plan_src.append((slots << 24) | srcs)
+        plan_pos.append(pos)
+        idx_t = v[-1]
+        idx_t._hq_blocks = pos.astype(np.int64)
+        idx_t._hq_host_version = idx_t._version
+        out[bits] = _Cls(v[0], idx_t, v[1] if bits != 16 else None, v[2] if bits != 16 else None)
+    plan_h = np.concatenate(plan_src + plan_pos + [np.zeros(1, dtype=np.int64)]).astype(np.int32)
+    plan = _to_dev(plan_h[:plan_h.size // 2 * 2].view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
+    with torch.cuda.device(dev):
+        rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src, _SRC_NEW + 1, dst, n_dst, plan.data_ptr(), B * H, D,
+                                             _lib.stream_ptr(dev))
+    _lib.check(rc, "cache_migrate")
+    # the kernel wrote the position arrays after the version stamps above were taken from fresh views: nothing in
+    # torch's bookkeeping changed, the host copies describe exactly what the kernel wrote
+    return out
+
+
+def _compress_gather(pkv: tuple, new_K, new_V, res_K, res_V, history: int, compress_length: int, K_sorted_idx,
+                     K_bit_num, V_bit_num, V_norm, V_sorted_idx, last_weights, strategy: str, n_targets: int):
+    """The whole compression as two gathers; -> new tuple, or None when the inputs are not made of whole blocks."""
+    if strategy not in ("uniform_group", LOW_NORMAL) or new_K.device.type != "cuda":
+        return None
+    if not torch.is_tensor(K_bit_num) or not torch.is_tensor(V_bit_num) or K_bit_num.is_cuda or V_bit_num.is_cuda:
+        return None
+    total_blocks = (history + compress_length) // BLOCK
+    hist_blocks, n_new_blocks = history // BLOCK, compress_length // BLOCK
+    k_side, v_side = _read_side(pkv, K_SLOT), _read_side(pkv, V_SLOT)
+    old = {}
+    for name, side in (("k", k_side), ("v", v_side)):
+        blocks = {}
+        kept = 0
+        for bits in CLASS_BITS:
+            c = side[bits]
+            if c.data is None:
+                continue
+            if c.idx is None:
+                return None
+            b = _host_blocks(c.idx)
+            if b is None:
+                return None
+            blocks[bits] = b
+            kept += b.size
+        if kept != hist_blocks:
+            return None
+        old[name] = blocks
+    # the two block rankings come down in one transfer when both carry theirs
+    k_ord = getattr(K_sorted_idx, "_hq_block_order", None)
+    v_ord = getattr(V_sorted_idx, "_hq_block_order", None)
+    k_order_h = v_order_h = None
+    if (k_ord is not None and v_ord is not None and k_ord[0].numel() == total_blocks == v_ord[0].numel()
+            and getattr(K_sorted_idx, "_hq_block_order_version", None) == K_sorted_idx._version
+            and k_ord[0].device == v_ord[0].device):
+        both = torch.stack((k_ord[0], v_ord[0])).to("cpu", torch.int64).numpy()
+        k_order_h, v_order_h = both[0], both[1]
+    elif v_ord is not None and v_ord[0].numel() == total_blocks:
+        v_order_h = v_ord[0].to("cpu", torch.int64).numpy()
+    k_label = _block_labels(K_sorted_idx, K_bit_num, total_blocks, k_order_h)
+    v_label = _block_labels(V_sorted_idx, V_bit_num, total_blocks, v_order_h)
+    if k_label is None or v_label is None:
+        return None
+    dev = new_V.device
+    sides = {}
+    for name, is_k, side, new, label in (("k", True, k_side, new_K, k_label), ("v", False, v_side, new_V, v_label)):
+        evicting = n_targets > 5 and bool((label == 5).any())
+        final, alive = _plan_side(old[name], hist_blocks, n_new_blocks, label, evicting)
+        rank_of = None
+        if alive is not None:
+            rank_of = np.full(total_blocks, -1, dtype=np.int64)
+            rank_of[alive] = np.arange(alive.size)
+        sides[name] = _gather_side(is_k, side, new, final, rank_of, strategy)
+        if name == "v" and alive is not None:
+            keep_tok = (alive[:, None] * BLOCK + np.arange(BLOCK, dtype=np.int64)).reshape(-1)
+            keep_t = _to_dev(keep_tok, dev)
+            V_norm = V_norm[keep_t]
+            if last_weights is not None:
+                last_weights.eviction(keep_t)
+    t = list(pkv)
+    _write_side(t, sides["k"], K_SLOT, dev)
+    _write_side(t, sides["v"], V_SLOT, dev)
+    t[38], t[39], t[40] = V_norm, res_K, res_V
+    return tuple(t)
+
+
 def compress(past_key_value: tuple, compress_length: int, history_length, K_sorted_idx: torch.Tensor,
              K_bit_num: torch.Tensor, V_bit_num: torch.Tensor, token_importance: torch.Tensor,
              quant_strategy: str, *, last_weights=None, block_size: int = 32, group_size: int = 32,
-             times_range: bool = True, n_targets: int = 6, V_token_range: Optional[torch.Tensor] = None) -> tuple:
+             times_range: bool = True, n_targets: int = 6, V_token_range: Optional[torch.Tensor] = None,
+             engine: Optional[str] = None) -> tuple:
+    """``engine``: None / "auto" = the one-launch-per-side gather when the selection is made of whole aligned blocks,
+    else the step-by-step engine; "steps" forces the latter, "gather" raises when it does not apply (tests)."""
     if quant_strategy not in _STRATEGIES:
         raise ValueError('invalid quant_strategy')
     if block_size != BLOCK or group_size != BLOCK:
@@ -377,6 +634,16 @@ def compress(past_key_value: tuple, compress_length: int, history_length, K_sort
     V_sorted_idx = get_block_token_idx(BLOCK, block_num, V_score)
 
     dev = new_V.device
+    engine = engine or os.environ.get("HQEKV_POLICY_ENGINE", "auto")
+    if engine not in ("auto", "gather", "steps"):
+        raise ValueError("engine must be 'auto', 'gather' or 'steps'")
+    if engine != "steps":
+        done = _compress_gather(pkv, new_K, new_V, res_K, res_V, history, compress_length, K_sorted_idx, K_bit_num,
+                                V_bit_num, V_norm, V_sorted_idx, last_weights, quant_strategy, n_targets)
+        if done is not None:
+            return done
+        if engine == "gather":
+            raise ValueError("the gather engine needs classes, rankings and counts made of whole aligned 32-token blocks")
     k_side, v_side = _read_side(pkv, K_SLOT, host=True), _read_side(pkv, V_SLOT, host=True)
     _migrate(k_side, new_K, _targets(K_sorted_idx, K_bit_num), history, True, quant_strategy)
 

@@ -1,0 +1,292 @@
+// Cache maintenance on the device: one launch rebuilds every precision class of one side (K or V) of a layer's
+// cache from the old classes and the new fp16 tokens, following a block-level plan the host worked out.
+//
+// What the reference does per compression (quant/hqe_2.py:552-836) is a sequence of boolean-mask gathers,
+// dequantise / re-quantise calls and torch.cat re-copies, one group of launches per (source, target) pair.  All of
+// it moves whole blocks of 32 tokens, and every block ends in exactly one place, so the whole compression is a
+// gather: destination block u of class c comes from block v of source s.  A unit of work is one quantisation
+// group of one block -- K: (block, channel), the 32 tokens of a channel; V: (token, 32 channels) -- held by one
+// lane as 32 fp16 values:
+//   same width            copy of the packed words, scale and zero (a survivor keeps its bytes)
+//   fp16 -> b bits        the quantiser of quant/pack_unpack.py:156-193 (or :218-253 for the 1-bit normal class)
+//   a bits -> b < a bits  dequantise with the reference's two fp16 roundings (quant/pack_unpack.py:331-332), then
+//                         quantise: what K_high_2_low / V_high_2_low do (quant/hqe_2.py:88-170)
+//   fp16 -> fp16          copy (new K arrives token-major and is stored channel-major)
+// Evicted blocks are simply in nobody's plan.  The arithmetic is the one of the stand-alone kernels (quant_math.h),
+// so the bytes equal those of the step-by-step path.
+#include "common.h"
+#include "quant_math.h"
+
+#pragma clang fp contract(off)
+
+namespace hq {
+
+struct MigClass {
+  void *data;
+  half_t *scale;
+  half_t *zero;
+  int64_t *idx;
+  int64_t n_tokens;
+  int64_t slab_tokens;  // tokens between (b, h) slabs of a token-major fp16 source (>= n_tokens)
+  int32_t bits;
+  int32_t layout;
+};
+
+struct MigArgs {
+  MigClass src[HQEKV_MAX_SEGS];
+  MigClass dst[HQEKV_MAX_SEGS];
+  int32_t dst_begin[HQEKV_MAX_SEGS + 1];  // first plan entry of every destination class; [n_dst] = total
+  int32_t n_dst;
+  const int32_t *plan_src;  // (source slot << 24) | source block, per destination block
+  const int32_t *plan_pos;  // new position of the block's first token / 32
+};
+
+// where one lane's group lives: fp16 values (with the element stride) or packed words + scale + zero
+struct GroupRef {
+  half_t *f16;
+  int64_t stride;
+  uint32_t *words;
+  half_t *s, *z;
+};
+
+template <bool IS_K>
+__device__ __forceinline__ GroupRef group_ref(const MigClass &c, int64_t bh, int64_t block, int lane, int D) {
+  GroupRef r{};
+  const int64_t n = c.n_tokens;
+  if (IS_K) {
+    const int d = lane;  // channel
+    if (c.bits == 16) {
+      if (c.layout == HQEKV_LAYOUT_TOKEN_MAJOR) {  // (B,H,T,D)
+        r.f16 = (half_t *)c.data + ((bh * c.slab_tokens + block * 32) * D + d);
+        r.stride = D;
+      } else {  // (B,H,D,T)
+        r.f16 = (half_t *)c.data + ((bh * D + d) * n + block * 32);
+        r.stride = 1;
+      }
+    } else {
+      const int64_t g = (bh * D + d) * (n >> 5) + block;
+      r.words = (uint32_t *)c.data + g * c.bits;  // 32 codes of b bits = b words
+      r.s = c.scale + g;
+      r.z = c.zero + g;
+    }
+  } else {
+    const int ng = D >> 5;
+    const int k = lane / ng, cg = lane % ng;  // token of the block, channel group
+    if (c.bits == 16) {
+      const int64_t t = bh * c.slab_tokens + block * 32 + k;
+      r.f16 = (half_t *)c.data + (t * D + cg * 32);
+      r.stride = 1;
+    } else {
+      const int64_t g = (bh * n + block * 32 + k) * ng + cg;
+      r.words = (uint32_t *)c.data + g * c.bits;
+      r.s = c.scale + g;
+      r.z = c.zero + g;
+    }
+  }
+  return r;
+}
+
+// 32 fp16 values as 16 registers: xp[j] = (x[2j], x[2j+1])
+__device__ __forceinline__ void load_f16(const GroupRef &r, uint32_t (&xp)[16]) {
+  if (r.stride == 1) {
+    const uint4 *p = reinterpret_cast<const uint4 *>(r.f16);  // block starts are 64-byte aligned
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint4 v = p[i];
+      xp[4 * i] = v.x;
+      xp[4 * i + 1] = v.y;
+      xp[4 * i + 2] = v.z;
+      xp[4 * i + 3] = v.w;
+    }
+  } else {
+    const unsigned short *p = reinterpret_cast<const unsigned short *>(r.f16);
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      xp[j] = (uint32_t)p[(2 * j) * r.stride] | ((uint32_t)p[(2 * j + 1) * r.stride] << 16);
+  }
+}
+__device__ __forceinline__ void store_f16(const GroupRef &r, const uint32_t (&xp)[16]) {
+  uint4 *p = reinterpret_cast<uint4 *>(r.f16);  // fp16 classes are stored with unit stride
+#pragma unroll
+  for (int i = 0; i < 4; ++i) p[i] = make_uint4(xp[4 * i], xp[4 * i + 1], xp[4 * i + 2], xp[4 * i + 3]);
+}
+
+// out = rnd16(rnd16(c * scale) + zero); NORMAL: rnd16(rnd16(+-k * std) + mean)
+template <int BITS, bool NORMAL>
+__device__ __forceinline__ void dequant_group(const GroupRef &r, uint32_t (&xp)[16]) {
+  constexpr int PF = 32 / BITS;
+  uint32_t w[BITS];
+#pragma unroll
+  for (int i = 0; i < BITS; ++i) w[i] = r.words[i];
+  const float s = (float)*r.s, z = (float)*r.z;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    half2_t v;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int k = 2 * j + e;
+      const float c = (float)code_at<BITS>(w[k / PF], k % PF);
+      const half_t m = NORMAL ? (half_t)((c != 0.f ? 0.67431640625f : -0.67431640625f) * s) : (half_t)(c * s);
+      v[e] = (half_t)((float)m + z);
+    }
+    xp[j] = h2_bits(v);
+  }
+}
+
+template <int BITS>
+__device__ __forceinline__ void quant_group(const GroupRef &r, const uint32_t (&xp)[16]) {
+  constexpr int PF = 32 / BITS;
+  constexpr int HALF = PF / 2;
+  constexpr float INV_QMAX = 1.0f / (float)((1 << BITS) - 1);
+  half2_t lo2 = bits_h2(xp[0]), hi2 = lo2;
+#pragma unroll
+  for (int j = 1; j < 16; ++j) {
+    lo2 = __builtin_elementwise_min(lo2, bits_h2(xp[j]));
+    hi2 = __builtin_elementwise_max(hi2, bits_h2(xp[j]));
+  }
+  const half_t mn_h = (half_t)__builtin_fminf((float)lo2[0], (float)lo2[1]);
+  const float mn = (float)mn_h, mx = __builtin_fmaxf((float)hi2[0], (float)hi2[1]);
+  const half_t d = (half_t)(mx - mn);
+  const half_t sc = (half_t)((float)d * INV_QMAX);
+  const float rcp = group_recip((float)sc);
+  const half2_t mn2 = {mn_h, mn_h};
+  float u[32];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const half2_t c = bits_h2(xp[j]) - mn2;
+    u[2 * j] = (float)c[0];
+    u[2 * j + 1] = (float)c[1];
+  }
+#pragma unroll
+  for (int wj = 0; wj < BITS; ++wj) {
+    uint32_t zz[HALF];
+#pragma unroll
+    for (int i = 0; i < HALF; ++i) zz[i] = code_pair_biased<BITS>(u[wj * PF + i], rcp, u[wj * PF + i + HALF], rcp);
+    r.words[wj] = horner_pack<BITS, HALF>(zz);
+  }
+  *r.s = sc;
+  *r.z = mn_h;
+}
+
+// the 1-bit normal-quantile quantiser: statistics in the order of torch's GPU reduction, code = [x > mean]
+__device__ __forceinline__ void quant_group_normal1(const GroupRef &r, const uint32_t (&xp)[16]) {
+  float xf[32];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const half2_t v = bits_h2(xp[j]);
+    xf[2 * j] = (float)v[0];
+    xf[2 * j + 1] = (float)v[1];
+  }
+  const Normal1Stats st = normal1_finish(welford_tree<32>(xf));
+  uint32_t w = 0;
+#pragma unroll
+  for (int k = 0; k < 32; ++k) w |= normal1_code((half_t)(xf[k] - (float)st.mean_h), st.thr) << k;
+  r.words[0] = w;
+  *r.s = st.std_h;
+  *r.z = st.mean_h;
+}
+
+template <bool IS_K>
+__global__ __launch_bounds__(128) void cache_migrate_kernel(MigArgs a, int D) {
+  const int u = blockIdx.x;
+  const int64_t bh = blockIdx.y;
+  int ci = 0;
+#pragma unroll
+  for (int k = 1; k < HQEKV_MAX_SEGS; ++k) ci += (k < a.n_dst && u >= a.dst_begin[k]) ? 1 : 0;
+  const MigClass dc = a.dst[ci];
+  const int64_t db = u - a.dst_begin[ci];  // block inside the destination class
+  const int32_t code = a.plan_src[u];
+  const MigClass sc = a.src[code >> 24];
+  const int64_t sb = code & 0xffffff;
+  if (bh == 0 && threadIdx.x < 32 && dc.idx) dc.idx[db * 32 + threadIdx.x] = (int64_t)a.plan_pos[u] * 32 + threadIdx.x;
+  const int lanes = IS_K ? D : D;  // K: one lane per channel; V: 32 tokens x D/32 groups
+  for (int lane = threadIdx.x; lane < lanes; lane += blockDim.x) {
+    const GroupRef sr = group_ref<IS_K>(sc, bh, sb, lane, D);
+    const GroupRef dr = group_ref<IS_K>(dc, bh, db, lane, D);
+    if (sc.bits != 16 && sc.bits == dc.bits) {  // a survivor of a quantised class keeps its bytes
+      for (int i = 0; i < sc.bits; ++i) dr.words[i] = sr.words[i];
+      *dr.s = *sr.s;
+      *dr.z = *sr.z;
+      continue;
+    }
+    uint32_t xp[16];
+    const bool sn = sc.layout == HQEKV_LAYOUT_NORMAL1;
+    switch (sc.bits) {
+      case 16: load_f16(sr, xp); break;
+      case 8: dequant_group<8, false>(sr, xp); break;
+      case 4: dequant_group<4, false>(sr, xp); break;
+      case 2: dequant_group<2, false>(sr, xp); break;
+      default:
+        if (sn) dequant_group<1, true>(sr, xp);
+        else dequant_group<1, false>(sr, xp);
+    }
+    switch (dc.bits) {
+      case 16: store_f16(dr, xp); break;
+      case 8: quant_group<8>(dr, xp); break;
+      case 4: quant_group<4>(dr, xp); break;
+      case 2: quant_group<2>(dr, xp); break;
+      default:
+        if (dc.layout == HQEKV_LAYOUT_NORMAL1) quant_group_normal1(dr, xp);
+        else quant_group<1>(dr, xp);
+    }
+  }
+}
+
+static int check_class(const hqekv_cache_class &c, bool is_src, int k, int64_t D) {
+  const char *side = is_src ? "source" : "destination";
+  if (c.n_tokens < 0 || c.n_tokens % 32 != 0)
+    return fail(HQEKV_E_ARG, "cache_migrate: %s %d holds %lld tokens (whole blocks of 32 only)", side, k, (long long)c.n_tokens);
+  if (c.n_tokens == 0) return HQEKV_OK;
+  if (!(c.bits == 16 || c.bits == 8 || c.bits == 4 || c.bits == 2 || c.bits == 1))
+    return fail(HQEKV_E_ARG, "cache_migrate: %s %d bits=%d", side, k, c.bits);
+  if (!c.data || (c.bits != 16 && (!c.scale || !c.zero)))
+    return fail(HQEKV_E_ARG, "cache_migrate: %s %d lacks data / scale / zero", side, k);
+  if ((uintptr_t)c.data & (c.bits == 16 ? 15 : 3)) return fail(HQEKV_E_ALIGN, "cache_migrate: %s %d data misaligned", side, k);
+  if (c.n_tokens * D >= (1LL << 40)) return fail(HQEKV_E_UNSUPPORTED, "cache_migrate: %s %d too large", side, k);
+  return HQEKV_OK;
+}
+
+}  // namespace hq
+
+using namespace hq;
+
+extern "C" int hqekv_cache_migrate(int is_k, const hqekv_cache_class *src, int n_src, const hqekv_cache_class *dst,
+                                   int n_dst, const int32_t *plan, int64_t BH, int64_t D, void *stream) {
+  if (n_src < 0 || n_src > HQEKV_MAX_SEGS || n_dst < 0 || n_dst > HQEKV_MAX_SEGS || (n_src && !src) || (n_dst && !dst))
+    return fail(HQEKV_E_ARG, "cache_migrate: bad class tables");
+  if (BH <= 0 || BH > 65535 || D <= 0 || D % 32 != 0 || D > 1024)
+    return fail(HQEKV_E_ARG, "cache_migrate: need 0 < B*H <= 65535 and head_dim a multiple of 32 up to 1024");
+  MigArgs a{};
+  int64_t total = 0;
+  for (int k = 0; k < n_src; ++k) {
+    const int rc = check_class(src[k], true, k, D);
+    if (rc) return rc;
+    // fp16 sources are read 32 values at a time: channel-major rows and token-major rows start 16-byte aligned
+    const int64_t slab = src[k].slab_tokens > 0 ? src[k].slab_tokens : src[k].n_tokens;
+    if (slab < src[k].n_tokens || (slab != src[k].n_tokens && !(src[k].bits == 16 && (!is_k || src[k].layout == HQEKV_LAYOUT_TOKEN_MAJOR))))
+      return fail(HQEKV_E_ARG, "cache_migrate: source %d: slab_tokens applies to token-major fp16 sources and must be >= n_tokens", k);
+    a.src[k] = MigClass{src[k].data, (half_t *)src[k].scale, (half_t *)src[k].zero, nullptr, src[k].n_tokens, slab, src[k].bits, src[k].layout};
+  }
+  for (int k = 0; k < n_dst; ++k) {
+    const int rc = check_class(dst[k], false, k, D);
+    if (rc) return rc;
+    if (dst[k].bits == 16 && dst[k].layout == HQEKV_LAYOUT_TOKEN_MAJOR && is_k)
+      return fail(HQEKV_E_UNSUPPORTED, "cache_migrate: the fp16 K class is stored channel-major");
+    if (dst[k].slab_tokens != 0 && dst[k].slab_tokens != dst[k].n_tokens)
+      return fail(HQEKV_E_ARG, "cache_migrate: destination %d must be stored densely", k);
+    a.dst[k] = MigClass{dst[k].data, (half_t *)dst[k].scale, (half_t *)dst[k].zero, dst[k].idx, dst[k].n_tokens, dst[k].n_tokens, dst[k].bits, dst[k].layout};
+    a.dst_begin[k] = (int32_t)total;
+    total += dst[k].n_tokens / 32;
+  }
+  for (int k = n_dst; k <= HQEKV_MAX_SEGS; ++k) a.dst_begin[k] = (int32_t)total;
+  if (total == 0) return HQEKV_OK;
+  if (total >= (1 << 24)) return fail(HQEKV_E_UNSUPPORTED, "cache_migrate: %lld blocks (limit 2^24)", (long long)total);
+  if (!plan) return fail(HQEKV_E_ARG, "cache_migrate: null plan");
+  a.n_dst = n_dst;
+  a.plan_src = plan;
+  a.plan_pos = plan + total;
+  const dim3 grid((unsigned)total, (unsigned)BH), block(128);
+  if (is_k) hipLaunchKernelGGL(cache_migrate_kernel<true>, grid, block, 0, (hipStream_t)stream, a, (int)D);
+  else hipLaunchKernelGGL(cache_migrate_kernel<false>, grid, block, 0, (hipStream_t)stream, a, (int)D);
+  return check_launch("cache_migrate_kernel");
+}

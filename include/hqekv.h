@@ -245,6 +245,36 @@ int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs,
                       int64_t D, int64_t Tall, void *workspace, int64_t workspace_bytes, int flags,
                       void *stream);
 
+/* ------------------------------------------------------------------ cache maintenance (one launch per side)
+ * Replaces the per-(source, target) gathers, dequantise / re-quantise calls and torch.cat re-copies of one
+ * compression -- V_high_2_eviction / K_high_2_eviction (quant/hqe_2.py:44-86), quant_new_K (:16-42), K_high_2_low
+ * (:88-130), V_high_2_low (:132-170) and their call sequence in KV_cache_hqe_2 (:552-836; KV_cache_compress,
+ * quant/hybrid_quant.py:318-612, is the same without eviction) -- by ONE gather over whole 32-token blocks.
+ *
+ * `src` lists the old classes of one side plus the new fp16 tokens, `dst` the classes after the compression (all
+ * freshly allocated by the caller, exact size).  Layouts as listed at the top of this file; a K source with bits == 16
+ * and layout HQEKV_LAYOUT_TOKEN_MAJOR is (B,H,T,D) (the new tokens), HQEKV_LAYOUT_NORMAL1 marks 1-bit classes in
+ * normal-quantile coding.  `plan` (device, int32) holds, for every destination block in the order of `dst`,
+ * first (source slot << 24) | source block, then -- after all of those -- the block's new first position / 32;
+ * the kernel also writes the destination classes' idx arrays from it (idx may be NULL).  A block that is in no
+ * destination is dropped (evicted).  Same width: the packed bytes are copied; fp16 -> b bits: quantised; a -> b < a
+ * bits: dequantised with the two fp16 roundings, then quantised; never the other way round.
+ * is_k != 0: classes are (B,H,D,*) with groups of 32 tokens per channel; else (B,H,T,*) with groups of 32 channels.
+ */
+typedef struct hqekv_cache_class {
+  int32_t bits;      /* 16, 8, 4, 2 or 1                       */
+  int32_t layout;    /* HQEKV_LAYOUT_*                         */
+  int64_t n_tokens;  /* multiple of 32; 0 = empty slot         */
+  int64_t slab_tokens; /* tokens between two (b, h) slabs in memory when the class is a window of a longer
+                          token-major tensor (the new tokens without the residual behind them); 0 = n_tokens */
+  void *data;
+  void *scale;       /* NULL when bits == 16                   */
+  void *zero;
+  int64_t *idx;      /* destination only: (n_tokens) or NULL   */
+} hqekv_cache_class;
+int hqekv_cache_migrate(int is_k, const hqekv_cache_class *src, int n_src, const hqekv_cache_class *dst,
+                        int n_dst, const int32_t *plan, int64_t BH, int64_t D, void *stream);
+
 /* No counterpart in the reference: hqekv_decode_attn for callers that cannot allocate (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  Same arguments minus the workspace: the split-K
  * partials and softmax statistics go to a fixed buffer of HQEKV_STATIC_SCRATCH_BYTES inside the library's device

@@ -97,3 +97,45 @@ def test_policy_errors(dev):
         KV_cache_hqe_2(pkv, 48, 0, ks, six, six, imp, "uniform_group")
     with pytest.raises(ValueError):
         KV_cache_hqe_2((None,) * 41 + (0,), 64, 0, ks, six, six, imp, "uniform_group")
+
+
+@pytest.mark.parametrize("strategy", ["uniform_group", "high_uniform_group_low_normal_group"])
+def test_gather_engine_equals_step_engine(dev, strategy):
+    """The one-launch-per-side gather (block-level plan on the host, hqekv_cache_migrate on the device) and the
+    step-by-step engine (the reference's sequence of moves) leave bit-identical tuples behind after each of three
+    compressions with demotions and evictions; the gather really ran (engine='gather' raises when it cannot)."""
+    from hqekv_amd import cache_policy
+    from hqekv_amd.public_func import get_block_token_idx
+
+    def runner(engine):
+        def f(pkv, cl, hist, ks, kb, vb, imp):
+            return cache_policy.compress(pkv, cl, hist, ks, kb, vb, imp, strategy, n_targets=6, engine=engine)
+        return PC.run(f, to_dev=lambda x: x.to(dev), rank_blocks=lambda bs, bn, imp: get_block_token_idx(bs, bn, imp.to(dev)))[0]
+
+    fast, slow = runner("gather"), runner("steps")
+    for step, (a, b) in enumerate(zip(fast, slow)):
+        for slot in range(42):
+            x, y = a[slot], b[slot]
+            _same(x, None if y is None else (y.cpu() if torch.is_tensor(y) else y), f"step {step} slot {slot}")
+
+
+def test_gather_engine_declines_selections_that_split_blocks(dev):
+    """V selections need not be made of whole blocks at this interface (a caller may hand in any ranking): the
+    gather engine then declines and the step-by-step engine does the compression; forcing the gather raises."""
+    from hqekv_amd import cache_policy
+    g = torch.Generator().manual_seed(31)
+    K = torch.randn(1, 2, 128, 128, generator=g).half()
+    V = torch.randn(1, 2, 128, 128, generator=g).half()
+    imp = torch.rand(128, generator=g)
+    ks = O.get_block_token_idx(32, 4, imp.clone())
+    ragged = torch.cat((ks[1:], ks[:1]))            # the same tokens, cut one token off the block grid
+    counts = torch.tensor([32, 32, 32, 32, 0], dtype=torch.int32)
+    pkv = tuple(x.to(dev) if torch.is_tensor(x) else x for x in O.empty_cache(K, V, 128))
+    with pytest.raises(ValueError, match="whole aligned"):
+        cache_policy.compress(pkv, 128, 0, ragged.to(dev), counts, counts.clone(), imp.to(dev), "uniform_group",
+                              n_targets=5, engine="gather")
+    # the same call without forcing: the step-by-step engine takes it, bit-identical to the oracle
+    got = cache_policy.compress(pkv, 128, 0, ragged.to(dev), counts, counts.clone(), imp.to(dev), "uniform_group", n_targets=5)
+    want, _ = O.compress_cache(O.empty_cache(K, V, 128), 128, 0, ragged, counts, counts.clone(), imp)
+    for slot in range(42):
+        _same(got[slot], want[slot], f"slot {slot}")
