@@ -403,50 +403,51 @@ def _block_labels(sorted_idx: torch.Tensor, bit_num, total_blocks: int, order_h:
     return label
 
 
-def _plan_side(old_blocks: Dict[int, Optional[np.ndarray]], hist_blocks: int, n_new_blocks: int, label: np.ndarray,
-               evicting: bool):
-    """-> (per class: (source slots, source blocks, old positions of the blocks), alive blocks ascending or None).
+def _plan_side(old_blocks: Dict[int, np.ndarray], hist_blocks: int, n_new_blocks: int, label: np.ndarray):
+    """-> (blocks per new class (5,), source slot / source block / old position of every new block, all classes
+    back to back in class order).
 
     Normative order inside a class (quant/hqe_2.py:552-659): the members that stay, in their order; then the new
     tokens ranked into it; then what comes down from the fp16, 8, 4 and 2-bit classes, each in source order.  A
-    block only ever moves to a lower precision; a block ranked into a higher one stays where it is."""
-    new_pos = np.arange(hist_blocks, hist_blocks + n_new_blocks, dtype=np.int64)
-    new_lab = label[new_pos]
-    final = {}
-    for ti, bits in enumerate(CLASS_BITS):
-        slots, srcs, poss = [], [], []
-        own = old_blocks.get(bits)
-        if own is not None and own.size:
-            lab = label[own]
-            stay = np.flatnonzero(lab <= ti)          # evict is the highest label; higher precision = lower label
-            slots.append(np.full(stay.size, ti, dtype=np.int64)); srcs.append(stay); poss.append(own[stay])
-        sel = np.flatnonzero(new_lab == ti)
-        slots.append(np.full(sel.size, _SRC_NEW, dtype=np.int64)); srcs.append(sel); poss.append(new_pos[sel])
-        for si in range(ti):                          # sources of higher precision, in the order 16, 8, 4, 2
-            src = old_blocks.get(CLASS_BITS[si])
-            if src is None or not src.size:
-                continue
-            sel = np.flatnonzero(label[src] == ti)
-            slots.append(np.full(sel.size, si, dtype=np.int64)); srcs.append(sel); poss.append(src[sel])
-        final[bits] = (np.concatenate(slots), np.concatenate(srcs), np.concatenate(poss))
-    alive = None
-    if evicting:
-        alive = np.flatnonzero(label != 5)
-    return final, alive
+    block only ever moves to a lower precision; a block ranked into a higher one stays where it is.  With the
+    classes numbered 0..4 from fp16 down, evicted = 5 and a new block's own class taken as -1, a block lands in
+    max(own class, ranked class); one three-key sort over all blocks (class, origin, place in the source) lays
+    every class out in that order."""
+    total = hist_blocks + n_new_blocks
+    cls_of = np.empty(total, dtype=np.int64)     # class a block is in now (5: the new tokens)
+    idx_in = np.empty(total, dtype=np.int64)     # its place inside that class
+    for ci, bits in enumerate(CLASS_BITS):
+        b = old_blocks.get(bits)
+        if b is not None and b.size:
+            cls_of[b] = ci
+            idx_in[b] = np.arange(b.size)
+    cls_of[hist_blocks:] = _SRC_NEW
+    idx_in[hist_blocks:] = np.arange(n_new_blocks)
+    own = np.where(cls_of == _SRC_NEW, -1, cls_of)
+    dest = np.maximum(own, label)
+    origin = np.where(own == dest, 0, own + 2)   # stays: 0; new: 1; moved down from class c: c + 2
+    order = np.lexsort((idx_in, origin, dest))
+    counts = np.bincount(dest, minlength=6)
+    order = order[:total - counts[5]]            # the evicted blocks sort last
+    return counts[:5], cls_of[order], idx_in[order], order
 
 
-def _carve(nbytes_list, dev):
-    """One allocation for all tensors of a side, each piece 256-byte aligned."""
-    offs, total = [], 0
-    for n in nbytes_list:
-        offs.append(total)
-        total += (n + 255) // 256 * 256
-    return torch.empty(max(total, 256), dtype=torch.uint8, device=dev), offs
+_CLASS_SHAPES_K = {b: (lambda B, H, D, n, b=b: [(B, H, D, n)] if b == 16 else [(B, H, D, n * b // 32), (B, H, D, n // 32), (B, H, D, n // 32)]) for b in CLASS_BITS}
+_CLASS_SHAPES_V = {b: (lambda B, H, D, n, b=b: [(B, H, n, D)] if b == 16 else [(B, H, n, D * b // 32), (B, H, n, D // 32), (B, H, n, D // 32)]) for b in CLASS_BITS}
 
 
-def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, final, rank_of: Optional[np.ndarray],
+def _numel(shape) -> int:
+    n = 1
+    for v in shape:
+        n *= v
+    return n
+
+
+def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, counts, slots, srcs, pos,
                  strategy: str) -> Dict[int, _Cls]:
-    """Allocate the new classes of one side and fill them with one launch of the migration kernel."""
+    """Allocate the new classes of one side (one buffer per element type, the tensors are views of it) and fill
+    them with one launch of the migration kernel.  ``slots`` / ``srcs`` / ``pos``: source slot, source block and
+    new block number of every new block, the classes back to back."""
     from . import _lib
     B, H, n_new, D = new.shape
     dev = new.device
@@ -460,13 +461,15 @@ def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, final, ra
             continue
         data = c.data if c.data.is_contiguous() else c.data.contiguous()
         keep.append(data)
-        n = data.shape[3] * (1 if bits == 16 else 32 // bits) if is_k else data.shape[2]
-        src[si].bits, src[si].n_tokens, src[si].data = bits, n, data.data_ptr()
-        src[si].layout = low_layout if bits == 1 else 0
+        e = src[si]
+        e.bits, e.data = bits, data.data_ptr()
+        e.n_tokens = (data.shape[3] * (1 if bits == 16 else 32 // bits)) if is_k else data.shape[2]
         if bits != 16:
             sc, zr = c.scale.contiguous(), c.zero.contiguous()
             keep += [sc, zr]
-            src[si].scale, src[si].zero = sc.data_ptr(), zr.data_ptr()
+            e.scale, e.zero = sc.data_ptr(), zr.data_ptr()
+            if bits == 1:
+                e.layout = low_layout
     # the new tokens are the head of a longer (B, H, T, D) tensor when a residual follows them: read in place
     slab = n_new
     if new.is_contiguous():
@@ -476,64 +479,72 @@ def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, final, ra
     else:
         newc = new.contiguous()
     keep.append(newc)
-    src[_SRC_NEW].bits, src[_SRC_NEW].n_tokens, src[_SRC_NEW].data = 16, n_new, newc.data_ptr()
-    src[_SRC_NEW].slab_tokens = slab
-    src[_SRC_NEW].layout = _lib.LAYOUT_TOKEN_MAJOR if is_k else 0
-    # ---- destinations: sizes, one allocation, views
-    pieces, sizes = [], []
-    for bits in CLASS_BITS:
-        n = final[bits][0].size * BLOCK
+    e = src[_SRC_NEW]
+    e.bits, e.n_tokens, e.data, e.slab_tokens = 16, n_new, newc.data_ptr(), slab
+    e.layout = _lib.LAYOUT_TOKEN_MAJOR if is_k else 0
+    # ---- destinations: element counts per type, three allocations, views
+    shapes_of = _CLASS_SHAPES_K if is_k else _CLASS_SHAPES_V
+    todo, n16, n32, n64 = [], 0, 0, 0
+    for ci, bits in enumerate(CLASS_BITS):
+        n = int(counts[ci]) * BLOCK
         if n == 0:
             continue
+        shp = shapes_of[bits](B, H, D, n)
         if bits == 16:
-            shapes = [((B, H, D, n) if is_k else (B, H, n, D), torch.float16)]
+            todo.append((bits, n, shp, (n16,), n64))
+            n16 += (_numel(shp[0]) + 127) // 128 * 128
         else:
-            pf = 32 // bits
-            if is_k:
-                shapes = [((B, H, D, n // pf), torch.int32), ((B, H, D, n // BLOCK), torch.float16), ((B, H, D, n // BLOCK), torch.float16)]
-            else:
-                shapes = [((B, H, n, D // pf), torch.int32), ((B, H, n, D // BLOCK), torch.float16), ((B, H, n, D // BLOCK), torch.float16)]
-        shapes.append(((n,), torch.int64))
-        for shp, dt in shapes:
-            pieces.append((bits, shp, dt))
-            sizes.append(int(np.prod(shp)) * torch.empty(0, dtype=dt).element_size())
+            o_s = n16
+            n16 += (_numel(shp[1]) + 127) // 128 * 128
+            o_z = n16
+            n16 += (_numel(shp[2]) + 127) // 128 * 128
+            todo.append((bits, n, shp, (n32, o_s, o_z), n64))
+            n32 += (_numel(shp[0]) + 63) // 64 * 64
+        n64 += (n + 31) // 32 * 32
     out = {b: _Cls() for b in CLASS_BITS}
-    if not pieces:
+    if not todo:
         return out
-    buf, offs = _carve(sizes, dev)
-    views: Dict[int, list] = {}
-    for (bits, shp, dt), off, nb in zip(pieces, offs, sizes):
-        views.setdefault(bits, []).append(buf[off:off + nb].view(dt).view(shp))
+    buf16 = torch.empty(max(n16, 1), dtype=torch.float16, device=dev)
+    buf32 = torch.empty(max(n32, 1), dtype=torch.int32, device=dev)
+    buf64 = torch.empty(n64, dtype=torch.int64, device=dev)
+
+    def view(buf, shape, off):
+        st, acc = [], 1
+        for v in reversed(shape):
+            st.append(acc)
+            acc *= v
+        return buf.as_strided(shape, st[::-1], off)
+
     dst = (_lib.CacheClass * len(CLASS_BITS))()
-    n_dst = 0
-    plan_src, plan_pos = [], []
-    for bits in CLASS_BITS:
-        if bits not in views:
-            continue
-        slots, srcs, poss = final[bits]
-        v = views[bits]
+    n_dst, blk0 = 0, 0
+    for bits, n, shp, offs, o_idx in todo:
         d = dst[n_dst]
-        d.bits, d.n_tokens, d.data = bits, slots.size * BLOCK, v[0].data_ptr()
-        d.layout = low_layout if bits == 1 else 0
-        if bits != 16:
-            d.scale, d.zero = v[1].data_ptr(), v[2].data_ptr()
-        d.idx = v[-1].data_ptr()
         n_dst += 1
-        pos = poss if rank_of is None else rank_of[poss]
-        plan_src.append((slots << 24) | srcs)
-        plan_pos.append(pos)
-        idx_t = v[-1]
-        idx_t._hq_blocks = pos.astype(np.int64)
+        idx_t = view(buf64, (n,), o_idx)
+        if bits == 16:
+            data = view(buf16, shp[0], offs[0])
+            sc = zr = None
+        else:
+            data, sc, zr = view(buf32, shp[0], offs[0]), view(buf16, shp[1], offs[1]), view(buf16, shp[2], offs[2])
+            d.scale, d.zero = sc.data_ptr(), zr.data_ptr()
+            if bits == 1:
+                d.layout = low_layout
+        d.bits, d.n_tokens, d.data, d.idx = bits, n, data.data_ptr(), idx_t.data_ptr()
+        idx_t._hq_blocks = pos[blk0:blk0 + n // BLOCK]
         idx_t._hq_host_version = idx_t._version
-        out[bits] = _Cls(v[0], idx_t, v[1] if bits != 16 else None, v[2] if bits != 16 else None)
-    plan_h = np.concatenate(plan_src + plan_pos + [np.zeros(1, dtype=np.int64)]).astype(np.int32)
-    plan = _to_dev(plan_h[:plan_h.size // 2 * 2].view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
+        blk0 += n // BLOCK
+        out[bits] = _Cls(data, idx_t, sc, zr)
+    nb = slots.size
+    plan_h = np.empty(2 * nb + (2 * nb) % 2 + 2, dtype=np.int32)
+    plan_h[:nb] = (slots << 24) | srcs
+    plan_h[nb:2 * nb] = pos
+    plan = _to_dev(plan_h[:(2 * nb + 1) // 2 * 2].view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
     with torch.cuda.device(dev):
         rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src, _SRC_NEW + 1, dst, n_dst, plan.data_ptr(), B * H, D,
                                              _lib.stream_ptr(dev))
     _lib.check(rc, "cache_migrate")
-    # the kernel wrote the position arrays after the version stamps above were taken from fresh views: nothing in
-    # torch's bookkeeping changed, the host copies describe exactly what the kernel wrote
+    # the kernel writes the position arrays behind torch's back: the version stamps taken above still hold, and the
+    # host copies describe exactly what the kernel wrote
     return out
 
 
@@ -583,14 +594,16 @@ def _compress_gather(pkv: tuple, new_K, new_V, res_K, res_V, history: int, compr
     dev = new_V.device
     sides = {}
     for name, is_k, side, new, label in (("k", True, k_side, new_K, k_label), ("v", False, v_side, new_V, v_label)):
-        evicting = n_targets > 5 and bool((label == 5).any())
-        final, alive = _plan_side(old[name], hist_blocks, n_new_blocks, label, evicting)
-        rank_of = None
-        if alive is not None:
-            rank_of = np.full(total_blocks, -1, dtype=np.int64)
+        counts, slots, srcs, old_pos = _plan_side(old[name], hist_blocks, n_new_blocks, label)
+        pos = old_pos
+        evicted = old_pos.size < total_blocks
+        if evicted:   # survivors keep their order; a block's new number is its rank among them
+            alive = np.sort(old_pos)
+            rank_of = np.empty(total_blocks, dtype=np.int64)
             rank_of[alive] = np.arange(alive.size)
-        sides[name] = _gather_side(is_k, side, new, final, rank_of, strategy)
-        if name == "v" and alive is not None:
+            pos = rank_of[old_pos]
+        sides[name] = _gather_side(is_k, side, new, counts, slots, srcs, pos, strategy)
+        if name == "v" and evicted:
             keep_tok = (alive[:, None] * BLOCK + np.arange(BLOCK, dtype=np.int64)).reshape(-1)
             keep_t = _to_dev(keep_tok, dev)
             V_norm = V_norm[keep_t]

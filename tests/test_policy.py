@@ -107,3 +107,34 @@ def test_oracle_policy_invariants_every_step():
                 assert pkv[s].shape == (PC.B, PC.H, PC.D, n * b // 32) and pkv[s + 2].shape == (PC.B, PC.H, PC.D, n // 32)
             if pkv[s + 4] is not None:
                 assert pkv[s + 4].shape == (PC.B, PC.H, pkv[s + 5].numel(), PC.D * b // 32)
+
+
+def test_block_planner_against_the_move_sequence_by_brute_force():
+    """The product's block-level planner (one three-key sort) against the reference's sequence of moves written out
+    with plain loops (quant/hqe_2.py:552-659): for every target from 1 bit up -- its members that stay, the new
+    tokens ranked into it, then what comes down from the fp16, 8, 4 and 2-bit classes in source order; a block
+    ranked into a higher precision stays; evicted blocks appear nowhere."""
+    import numpy as np
+    from hqekv_amd import cache_policy as cp
+    rng = np.random.default_rng(0)
+    for trial in range(300):
+        hist, n_new = int(rng.integers(0, 40)), int(rng.integers(1, 8))
+        parts = np.split(rng.permutation(hist), np.sort(rng.integers(0, hist + 1, 4)))
+        old = {b: parts[i].astype(np.int64) for i, b in enumerate(cp.CLASS_BITS) if parts[i].size}
+        label = rng.integers(0, 6, hist + n_new).astype(np.int8)
+        counts, slots, srcs, pos = cp._plan_side(old, hist, n_new, label)
+        want = []
+        for ti, bits in enumerate(cp.CLASS_BITS):
+            for j, p in enumerate(old.get(bits, [])):
+                if label[p] <= ti:
+                    want.append((ti, ti, j, p))
+            for j in range(n_new):
+                if label[hist + j] == ti:
+                    want.append((ti, 5, j, hist + j))
+            for si in range(ti):
+                for j, p in enumerate(old.get(cp.CLASS_BITS[si], [])):
+                    if label[p] == ti:
+                        want.append((ti, si, j, p))
+        assert [w[1] for w in want] == slots.tolist() and [w[2] for w in want] == srcs.tolist(), trial
+        assert [w[3] for w in want] == pos.tolist(), trial
+        assert counts.tolist() == [sum(1 for w in want if w[0] == t) for t in range(5)]
