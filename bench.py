@@ -428,7 +428,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--layers", type=int, default=None, help="distinct layer caches cycled through")
-    ap.add_argument("--qk-tiling", default="auto", choices=["auto", "8waves", "4waves", "wave512", "wave128"],
+    ap.add_argument("--qk-tiling", default="auto", choices=["auto", "8waves", "4waves", "wave512", "wave256"],
                     help="force one q.K^T tiling instead of the choice by launch size")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

@@ -17,10 +17,12 @@ _LIB_PATH = Path(os.environ.get("HQEKV_LIB", _PKG / "libhqekv.so"))
 
 MAX_SEGS = 8
 FUSE_SOFTMAX = 1
+SEPARATE_COMBINE = 2
+FOLD_COMBINE = 4
 ONLY_QK = 0x100
 ONLY_PV = 0x200
 ONLY_COMBINE = 0x400
-QK_TILINGS = {"8waves": 1, "4waves": 2, "wave512": 3, "wave128": 4}   # HQEKV_QK_TILING_*: tilings a call may force
+QK_TILINGS = {"8waves": 1, "4waves": 2, "wave512": 3, "wave256": 4}   # HQEKV_QK_TILING_*: tilings a call may force
 
 
 def qk_tiling(n: int) -> int:
@@ -137,7 +139,28 @@ def check(rc: int, what: str) -> None:
 
 
 def stream_ptr(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on ``device`` (the cheap lookup: this runs once per launch)."""
+    idx = device.index
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if idx is None else idx)
+
+
+class on_device:
+    """``with on_device(dev):`` -- make ``dev`` the current HIP device for a launch.  Does nothing when it already
+    is (one integer comparison instead of torch's two device switches), which is every call of a one-GPU process."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, device: torch.device):
+        idx = device.index
+        self.ctx = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
 
 
 def require_gpu(t: torch.Tensor, name: str) -> None:

@@ -218,9 +218,12 @@ def decode_workspace(k_segs, n_k: int, v_segs, n_v: int, B: int, Hq: int, Hkv: i
     return torch.empty(max(need, 256) // 4, dtype=torch.float32, device=dev)
 
 
+_environ = os.environ   # (attribute lookups on the module are the slow part of this per-step call)
+
+
 def default_flags() -> int:
     """Fuse the softmax into the two GEMV launches unless HQEKV_UNFUSED=1 asks for the general path."""
-    return 0 if os.environ.get("HQEKV_UNFUSED", "0") == "1" else _lib.FUSE_SOFTMAX
+    return 0 if _environ.get("HQEKV_UNFUSED") == "1" else _lib.FUSE_SOFTMAX
 
 
 class SegmentMemo:
@@ -341,7 +344,7 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev)
     mptr, mstride = _mask_arg(mask, B, Hq, Tall, dev, keep)
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         if memo is not None:
             need = lib.hqekv_decode_workspace_bytes(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D)
             if need < 0:
@@ -381,7 +384,7 @@ class DecodePlan:
         self.weights = torch.zeros(B, Hq, 1, self.Tall, dtype=torch.float16, device=self.dev)
         self.out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=self.dev)
         self.mask_ptr, self.mask_stride = _mask_arg(mask, B, Hq, self.Tall, self.dev, self._keep)
-        with torch.cuda.device(self.dev):
+        with _lib.on_device(self.dev):
             self.ws = decode_workspace(self.k_segs, self.n_k, self.v_segs, self.n_v, B, Hq, self.Hkv, D, self.dev)
         self.flags = default_flags() if flags is None else flags
         if (self.flags & _lib.FUSE_SOFTMAX) and mask is None and not classes_partition_positions(pkv):

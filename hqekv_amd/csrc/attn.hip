@@ -72,13 +72,20 @@ __device__ __forceinline__ int begin_of_seg(const SegTable &tb, int s) {
 // classes as well as the V classes each cover every position exactly once):
 //   q.K^T stores the scaled fp16 logit instead of the raw score and one (max, sum exp) pair per tile and
 //   head; p.V turns a logit into its probability while staging it and writes it back for the caller.
-// The split-K partials are summed by a separate small launch: a "last workgroup sums" scheme needs
-// device-scope release/acquire fences, which write back and invalidate the whole L2 on this chip and cost
-// far more than the launch they would save.
+// The split-K partials are summed by the LAST p.V workgroup of each (b, kv head) to finish, when there are few
+// enough of them; otherwise by a small launch of their own.  Nobody waits for anybody: a workgroup stores its
+// partial rows write-through (agent-scope relaxed stores go past the per-XCD L2), waits for the stores to be
+// acknowledged, and bumps one relaxed agent-scope counter; whoever reads the final count adds the rows up with
+// loads that bypass the L2 as well, in the fixed order of the separate launch.  No release / acquire fences are
+// involved: those write back and invalidate the whole L2 on this chip (the step went from 39 to 146 us with them).
 struct FuseArgs {
   float2 *stats;       // (B*Hq, n_stat) pairs (m, l); nullptr = unfused
   int32_t n_stat;      // tiles per row of stats = number of q.K^T tiles per (b, kv head)
   float inv_sqrt_d;
+  // Folded combine (independent of the softmax fusion): one arrival counter per (b, kv head), zeroed by the q.K^T
+  // launch of the same call; nullptr = the split-K partials are summed by a launch of their own.
+  uint32_t *arrive;
+  half_t *out;         // (B*Hq, D) attention output, written by the last workgroup of each (b, kv head)
 };
 
 // A workgroup learns its segment and its tile/chunk from its block id with two scalar loads at the top of
@@ -164,10 +171,10 @@ __device__ __forceinline__ half2_t dequant_pair_normal1(half2_t c, half2_t a2, h
 
 // Consume one byte pair: 8/BITS dequantised pairs, each dotted with NREP operand pairs.
 // NORMAL (1 bit only): s2 is the spread a2 = rnd16(k * std), z2 the mean.
-template <int BITS, int NREP, int PF, bool NORMAL = false>
+template <int BITS, int NREP, int PF, bool NORMAL = false, int NFIELD = 8 / BITS>
 __device__ __forceinline__ void consume_byte(uint32_t u, half2_t s2, half2_t z2, const half2_t (&a2)[NREP],
                                              float (&acc)[NREP][PF], int tok0) {
-  constexpr int FPB = 8 / BITS;
+  constexpr int FPB = NFIELD;   // fields taken, from the low end of the byte
 #define HQ_FIELD(I_)                                                                     \
   if constexpr (I_ < FPB) {                                                                      \
     const half2_t c2_ = field_pair<BITS, (I_ < FPB ? I_ : 0)>(u);                        \
@@ -508,6 +515,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int bh = blockIdx.x;
   const int b = bh / Hkv, hkv = bh % Hkv;
+  if (fz.arrive && blockIdx.y == 0 && threadIdx.x == 0) fz.arrive[bh] = 0;  // for the p.V launch that follows
   // grid.y counts workgroups; a workgroup takes `tpw` consecutive tiles of one class (1 unless the
   // environment asks for more: longer-lived workgroups stage the query once, but measured no faster)
   const int si = seg_of_unit(tb, blockIdx.y);
@@ -667,52 +675,21 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
 // pairs) and the tile's scale/zero rows in LDS: the rows are fetched with wide loads (a tile's groups of one
 // row are contiguous) and stored pair-interleaved -- {(s_d, s_d+1), (z_d, z_d+1)} per (row pair, group) -- so
 // the inner loop reads both with one 8-byte LDS access and pairs nothing itself.
-// DS = 1: 64 token lanes, tile = 512 tokens, a lane walks all 64 row pairs (least fixed work per code).
-// DS = 4: 16 token lanes x 4 quarters of head_dim, tile = 128 tokens; the quarters sit 16 lanes apart and are
-//         summed with two lane-row swaps: four times the waves for launches that would not fill the chip.
+// TPL = 8 tokens per lane: tile = 512 tokens, least fixed work per code; 128 registers and 9 KB of LDS per wave
+//         allow four waves per SIMD.
+// TPL = 4 tokens per lane: tile = 256 tokens, half the accumulators and half the staged scale/zero rows: eight
+//         waves per SIMD hide the memory latency that four leave exposed, at the price of the per-tile work
+//         (query staging, statistics, stores) being spread over half as many codes.
 // head_dim is 128 here; the host sends other sizes to the tilings above.
-template <int DS>
+template <int TPL>
 struct QwGeom {
-  static constexpr int TL = 64 / DS;       // token lanes
-  static constexpr int TILE = TL * QK_TPL; // tokens per tile
+  static constexpr int TILE = 64 * TPL;    // tokens per tile
   static constexpr int NG = TILE / 32;     // scale/zero groups per tile and row
-  static constexpr int RP = 64 / DS;       // row pairs a lane walks
-  static constexpr int GPI = NG >= 8 ? 8 : NG;  // groups one staging item covers (16 or 8 bytes per row)
+  static constexpr int LPG = 32 / TPL;     // lanes that share a group
+  static constexpr int RP = 64;            // row pairs a lane walks
+  static constexpr int GPI = 8;            // groups one staging item covers (16 bytes per row)
 };
-__host__ __device__ constexpr int qw_tile(int ds) { return (64 / ds) * QK_TPL; }
-
-// sum over the four rows of 16 lanes, valid in lanes 0-15 afterwards (two lane-row swaps per value; the swaps
-// need idle issue slots around them that the compiler does not insert for inline asm)
-__device__ __forceinline__ void rows_sum8(float (&v)[8]) {
-  float o[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = v[i];
-#define HQ_SWAP8(OP_)                                                                                         \
-  asm volatile("s_nop 7\n\t" OP_ " %0, %8\n\t" OP_ " %1, %9\n\t" OP_ " %2, %10\n\t" OP_ " %3, %11\n\t"         \
-               OP_ " %4, %12\n\t" OP_ " %5, %13\n\t" OP_ " %6, %14\n\t" OP_ " %7, %15\n\ts_nop 7"               \
-               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), \
-                 "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]), "+v"(o[7]))
-  HQ_SWAP8("v_permlane16_swap_b32");  // rows 0 and 2: o = the old rows 1 and 3
-#pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = o[i] = v[i] + o[i];
-  HQ_SWAP8("v_permlane32_swap_b32");  // row 0: o = the old row 2
-#undef HQ_SWAP8
-#pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] += o[i];
-}
-// reductions inside a row of 16 lanes (every lane of the row gets the result)
-__device__ __forceinline__ float row_max16(float v) {
-  v = fmaxf(v, dpp_f<0xB1>(v));
-  v = fmaxf(v, dpp_f<0x4E>(v));
-  v = fmaxf(v, dpp_f<0x141>(v));
-  return fmaxf(v, dpp_f<0x140>(v));
-}
-__device__ __forceinline__ float row_sum16(float v) {
-  v += dpp_f<0xB1>(v);
-  v += dpp_f<0x4E>(v);
-  v += dpp_f<0x141>(v);
-  return v + dpp_f<0x140>(v);
-}
+__host__ __device__ constexpr int qw_tile(int tpl) { return 64 * tpl; }
 
 __device__ __forceinline__ uint4 buf_u128(rsrc_t r, uint32_t lane_off, uint32_t row_off) {
   typedef uint32_t v4u __attribute__((ext_vector_type(4)));
@@ -728,21 +705,23 @@ __device__ __forceinline__ uint32_t buf_u8(rsrc_t r, uint32_t lane_off, uint32_t
   return (uint32_t)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(r, (int)lane_off, (int)row_off, 0);
 }
 
-// the 8 codes of one row a lane owns: a byte at 1 bit, 16 bits at 2 bits, a word at 4 bits, two words at 8 bits
-template <int BITS>
+// the TPL codes of one row a lane owns: TPL * BITS bits, fetched with the narrowest load that holds them (at
+// 1 bit and 4 tokens per lane two lanes share a byte and each takes its nibble)
+template <int BITS, int TPL>
 struct QwRow {
-  uint32_t w[BITS == 8 ? 2 : 1];
+  uint32_t w[TPL * BITS > 32 ? 2 : 1];
 };
-template <int BITS>
-__device__ __forceinline__ QwRow<BITS> qw_load_row(rsrc_t rc, uint32_t lane_off, uint32_t row_off) {
-  QwRow<BITS> r;
-  if constexpr (BITS == 8) {
+template <int BITS, int TPL>
+__device__ __forceinline__ QwRow<BITS, TPL> qw_load_row(rsrc_t rc, uint32_t lane_off, uint32_t row_off) {
+  constexpr int NB = TPL * BITS;  // bits per lane and row
+  QwRow<BITS, TPL> r;
+  if constexpr (NB == 64) {
     const uint2 v = buf_u64(rc, lane_off, row_off);
     r.w[0] = v.x;
     r.w[1] = v.y;
-  } else if constexpr (BITS == 4) {
+  } else if constexpr (NB == 32) {
     r.w[0] = buf_u32(rc, lane_off, row_off);
-  } else if constexpr (BITS == 2) {
+  } else if constexpr (NB == 16) {
     r.w[0] = buf_u16(rc, lane_off, row_off);
   } else {
     r.w[0] = buf_u8(rc, lane_off, row_off);
@@ -753,9 +732,9 @@ __device__ __forceinline__ QwRow<BITS> qw_load_row(rsrc_t rc, uint32_t lane_off,
 // Stage the scale/zero rows of one tile: sz[dp * NG + g] = {(s[2dp][g], s[2dp+1][g]), (z[2dp][g], z[2dp+1][g])}.
 // Groups past the end of the class read whatever follows (the next row, or zero past the slab): only lanes
 // whose tokens do not exist look at them.
-template <int DS, bool NORMAL>
+template <int TPL, bool NORMAL>
 __device__ __forceinline__ void qw_stage_sz(const SegDev &sg, int tile, int bh, int lane, uint2 *sz) {
-  using G = QwGeom<DS>;
+  using G = QwGeom<TPL>;
   constexpr int NG = G::NG, GPI = G::GPI;
   constexpr int ITEMS = 64 * NG / GPI;   // (row pair, part of the tile's groups)
   const uint32_t gpr = (uint32_t)(sg.n_tokens >> 5);
@@ -809,28 +788,31 @@ __device__ __forceinline__ void qw_stage_sz(const SegDev &sg, int tile, int bh, 
   }
 }
 
-template <int BITS, int NREP, int DS, bool NORMAL, typename Stage>
+template <int BITS, int NREP, int TPL, bool NORMAL, typename Stage>
 __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int lane, Stage &&stage,
-                                                    const half2_t *q2s, const uint2 *sz, float (&acc)[NREP][QK_TPL]) {
-  using G = QwGeom<DS>;
-  constexpr int U = BITS == 8 ? 2 : 4;  // row pairs per register block; two blocks of loads are in flight
+                                                    const half2_t *q2s, const uint2 *sz, float (&acc)[NREP][TPL]) {
+  using G = QwGeom<TPL>;
+  using Row = QwRow<BITS, TPL>;
+  constexpr int NB = TPL * BITS;                    // bits per lane and row
+  // row pairs per register block (two blocks of loads are in flight): short blocks where registers are scarce --
+  // the wide rows of the 8-bit class, and the 256-token tile, whose extra waves hide latency instead
+  constexpr int U = (NB == 64 || TPL == 4) ? 2 : 4;
   static_assert(G::RP % (2 * U) == 0, "the block loop covers the row pairs exactly");
   const uint32_t n = (uint32_t)sg.n_tokens;
-  const uint32_t rowb = n / 8u * BITS;                       // bytes per channel row
-  const int tl = lane % G::TL, part = lane / G::TL;
-  const uint32_t lane_off = ts / 8u * BITS + (uint32_t)(part * G::RP * 2) * rowb;
+  const uint32_t rowb = n / 8u * BITS;              // bytes per channel row
+  const uint32_t lane_off = ts * BITS / 8u;         // (two lanes share a byte when a lane owns 4 bits)
+  const int nib = (NB == 4) ? (int)(ts & 4u) : 0;   // ... and the odd one takes the upper nibble
   const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * 128 * rowb, 128u * rowb);
-  const half2_t *qp = q2s + part * G::RP * NREP;
-  const uint2 *sp = sz + part * G::RP * G::NG + (tl >> 2);
+  const uint2 *sp = sz + lane / G::LPG;
   struct Block {
-    QwRow<BITS> r0[U], r1[U];
+    Row r0[U], r1[U];
   };
   auto load = [&](int i0, Block &b) {
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t row = (uint32_t)(2 * (i0 + k)) * rowb;  // uniform
-      b.r0[k] = qw_load_row<BITS>(rc, lane_off, row);
-      b.r1[k] = qw_load_row<BITS>(rc, lane_off, row + rowb);
+      b.r0[k] = qw_load_row<BITS, TPL>(rc, lane_off, row);
+      b.r1[k] = qw_load_row<BITS, TPL>(rc, lane_off, row + rowb);
     }
   };
   auto compute = [&](int i0, const Block &b) {
@@ -839,27 +821,24 @@ __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t t
       const int i = i0 + k;
       half2_t q2[NREP];
 #pragma unroll
-      for (int h = 0; h < NREP; ++h) q2[h] = qp[i * NREP + h];
+      for (int h = 0; h < NREP; ++h) q2[h] = q2s[i * NREP + h];
       const uint2 szv = sp[i * G::NG];
       const half2_t s2 = as_h2(szv.x), z2 = as_h2(szv.y);
-      if constexpr (BITS == 1) {
-        consume_byte<1, NREP, QK_TPL, NORMAL>(byte_pair<0>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 0);
-      } else if constexpr (BITS == 2) {
-        consume_byte<2, NREP, QK_TPL>(byte_pair<0>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 0);
-        consume_byte<2, NREP, QK_TPL>(byte_pair<1>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 4);
-      } else if constexpr (BITS == 4) {
-        consume_byte<4, NREP, QK_TPL>(byte_pair<0>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 0);
-        consume_byte<4, NREP, QK_TPL>(byte_pair<1>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 2);
-        consume_byte<4, NREP, QK_TPL>(byte_pair<2>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 4);
-        consume_byte<4, NREP, QK_TPL>(byte_pair<3>(b.r0[k].w[0], b.r1[k].w[0]), s2, z2, q2, acc, 6);
-      } else {
+      constexpr int FPB = 8 / BITS;                 // codes per byte
+      constexpr int NBYTE = (NB + 7) / 8;           // bytes per lane and row
+      constexpr int NF = NB < 8 ? NB / BITS : FPB;  // codes taken from a byte
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          consume_byte<8, NREP, QK_TPL>(byte_pair<0>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 0);
-          consume_byte<8, NREP, QK_TPL>(byte_pair<1>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 1);
-          consume_byte<8, NREP, QK_TPL>(byte_pair<2>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 2);
-          consume_byte<8, NREP, QK_TPL>(byte_pair<3>(b.r0[k].w[j], b.r1[k].w[j]), s2, z2, q2, acc, 4 * j + 3);
+      for (int j = 0; j < NBYTE; ++j) {
+        uint32_t a0 = b.r0[k].w[j / 4], a1 = b.r1[k].w[j / 4];
+        if (NB == 4) {
+          a0 >>= nib;
+          a1 >>= nib;
         }
+        const uint32_t u = (j % 4 == 0)   ? byte_pair<0>(a0, a1)
+                           : (j % 4 == 1) ? byte_pair<1>(a0, a1)
+                           : (j % 4 == 2) ? byte_pair<2>(a0, a1)
+                                          : byte_pair<3>(a0, a1);
+        consume_byte<BITS, NREP, TPL, NORMAL, NF>(u, s2, z2, q2, acc, j * FPB);
       }
     }
   };
@@ -877,41 +856,46 @@ __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t t
   }
 }
 
-// fp16 class stored channel-major (B,Hkv,128,T), T a multiple of 8: a lane reads its 8 tokens of a row as 16 bytes
-template <int NREP, int DS, typename Stage>
+// fp16 class stored channel-major (B,Hkv,128,T), T a multiple of 8: a lane reads its TPL tokens of a row as 16 or 8 bytes
+template <int NREP, int TPL, typename Stage>
 __device__ __forceinline__ void qw_f16_accumulate(const SegDev &sg, uint32_t ts, int bh, int lane, Stage &&stage,
-                                                  const half2_t *q2s, float (&acc)[NREP][QK_TPL]) {
-  using G = QwGeom<DS>;
-  constexpr int U = 2;
+                                                  const half2_t *q2s, float (&acc)[NREP][TPL]) {
+  using G = QwGeom<TPL>;
+  constexpr int U = 2, NW = TPL / 2;   // words per lane and row
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t rowb = n * 2u;
-  const int part = lane / G::TL;
-  const uint32_t lane_off = ts * 2u + (uint32_t)(part * G::RP * 2) * rowb;
+  const uint32_t lane_off = ts * 2u;
   const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * 128 * rowb, 128u * rowb);
-  const half2_t *qp = q2s + part * G::RP * NREP;
   struct Block {
-    uint4 r0[U], r1[U];
+    uint32_t r0[U][NW], r1[U][NW];
+  };
+  auto load_row = [&](uint32_t row, uint32_t (&w)[NW]) {
+    if constexpr (NW == 4) {
+      const uint4 v = buf_u128(rc, lane_off, row);
+      w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    } else {
+      const uint2 v = buf_u64(rc, lane_off, row);
+      w[0] = v.x; w[1] = v.y;
+    }
   };
   auto load = [&](int i0, Block &b) {
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t row = (uint32_t)(2 * (i0 + k)) * rowb;
-      b.r0[k] = buf_u128(rc, lane_off, row);
-      b.r1[k] = buf_u128(rc, lane_off, row + rowb);
+      load_row(row, b.r0[k]);
+      load_row(row + rowb, b.r1[k]);
     }
   };
   auto compute = [&](int i0, const Block &b) {
 #pragma unroll
     for (int k = 0; k < U; ++k) {
-      const uint32_t a[4] = {b.r0[k].x, b.r0[k].y, b.r0[k].z, b.r0[k].w};
-      const uint32_t c[4] = {b.r1[k].x, b.r1[k].y, b.r1[k].z, b.r1[k].w};
       half2_t q2[NREP];
 #pragma unroll
-      for (int h = 0; h < NREP; ++h) q2[h] = qp[(i0 + k) * NREP + h];
+      for (int h = 0; h < NREP; ++h) q2[h] = q2s[(i0 + k) * NREP + h];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const half2_t ka = half_pair<0>(a[i], c[i]);  // token 2i:   (k[d], k[d+1])
-        const half2_t kb = half_pair<1>(a[i], c[i]);  // token 2i+1
+      for (int i = 0; i < NW; ++i) {
+        const half2_t ka = half_pair<0>(b.r0[k][i], b.r1[k][i]);  // token 2i:   (k[d], k[d+1])
+        const half2_t kb = half_pair<1>(b.r0[k][i], b.r1[k][i]);  // token 2i+1
 #pragma unroll
         for (int h = 0; h < NREP; ++h) {
           acc[h][2 * i] = __builtin_amdgcn_fdot2(ka, q2[h], acc[h][2 * i], false);
@@ -935,17 +919,18 @@ __device__ __forceinline__ void qw_f16_accumulate(const SegDev &sg, uint32_t ts,
   }
 }
 
-template <int NREP, int DS>
-__global__ __launch_bounds__(64, NREP <= 4 ? 4 : 2) void qk_wave_kernel(SegTable tb, const half_t *__restrict__ q,
-                                                                       half_t *__restrict__ scores, int Hq, int Hkv,
-                                                                       int64_t Tall, FuseArgs fz) {
-  using G = QwGeom<DS>;
+template <int NREP, int TPL>
+__global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wave_kernel(SegTable tb, const half_t *__restrict__ q,
+                                                                              half_t *__restrict__ scores, int Hq, int Hkv,
+                                                                              int64_t Tall, FuseArgs fz) {
+  using G = QwGeom<TPL>;
   __shared__ half2_t q2s[64 * NREP];                  // [row pair][head]: (q[d], q[d+1])
   __shared__ __align__(16) uint2 sz[64 * G::NG];      // [row pair][group]: {(s_d, s_d+1), (z_d, z_d+1)}
   __shared__ float red[2 * NREP];
   const int lane = threadIdx.x;
   const int bh = blockIdx.x;
   const int b = bh / Hkv, hkv = bh % Hkv;
+  if (fz.arrive && blockIdx.y == 0 && lane == 0) fz.arrive[bh] = 0;  // for the p.V launch that follows
   const int si = seg_of_unit(tb, blockIdx.y);
   const SegDev sg = tb.seg[si];
   const int tile = (int)blockIdx.y - begin_of_seg(tb, si);
@@ -961,19 +946,18 @@ __global__ __launch_bounds__(64, NREP <= 4 ? 4 : 2) void qk_wave_kernel(SegTable
     return;
   }
   const uint32_t n = (uint32_t)sg.n_tokens;
-  const int tl = lane % G::TL;
-  const uint32_t t0 = (uint32_t)tile * G::TILE + (uint32_t)tl * QK_TPL;
-  const bool valid = t0 < n;          // class lengths are multiples of 8: a lane's tokens exist or do not
+  const uint32_t t0 = (uint32_t)tile * G::TILE + (uint32_t)lane * TPL;
+  const bool valid = t0 < n;           // class lengths are multiples of 8: a lane's tokens exist or do not
   const uint32_t ts = valid ? t0 : 0;  // lanes past the end recompute the first tokens and store nothing
-  float acc[NREP][QK_TPL];
+  float acc[NREP][TPL];
 #pragma unroll
   for (int h = 0; h < NREP; ++h)
 #pragma unroll
-    for (int i = 0; i < QK_TPL; ++i) acc[h][i] = 0.f;
+    for (int i = 0; i < TPL; ++i) acc[h][i] = 0.f;
 
   auto stage_quant = [&](auto normal) {
     stage_q();
-    qw_stage_sz<DS, decltype(normal)::value>(sg, tile, bh, lane, sz);
+    qw_stage_sz<TPL, decltype(normal)::value>(sg, tile, bh, lane, sz);
     __syncthreads();
   };
   auto stage_plain = [&]() {
@@ -985,45 +969,40 @@ __global__ __launch_bounds__(64, NREP <= 4 ? 4 : 2) void qk_wave_kernel(SegTable
   switch (sg.bits) {
     case 1:
       if (sg.layout == HQEKV_LAYOUT_NORMAL1)
-        qw_quant_accumulate<1, NREP, DS, true>(sg, ts, bh, lane, [&]() { stage_quant(T{}); }, q2s, sz, acc);
+        qw_quant_accumulate<1, NREP, TPL, true>(sg, ts, bh, lane, [&]() { stage_quant(T{}); }, q2s, sz, acc);
       else
-        qw_quant_accumulate<1, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc);
+        qw_quant_accumulate<1, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc);
       break;
-    case 2: qw_quant_accumulate<2, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
-    case 4: qw_quant_accumulate<4, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
-    case 8: qw_quant_accumulate<8, NREP, DS, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
-    default: qw_f16_accumulate<NREP, DS>(sg, ts, bh, lane, stage_plain, q2s, acc);
+    case 2: qw_quant_accumulate<2, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
+    case 4: qw_quant_accumulate<4, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
+    case 8: qw_quant_accumulate<8, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
+    default: qw_f16_accumulate<NREP, TPL>(sg, ts, bh, lane, stage_plain, q2s, acc);
   }
 
   // positions of the lane's tokens (they index a row of Tall < 2^31 scores, so the low word of each int64 entry
   // is enough); requested here, used after the conversions below
-  uint32_t pos[QK_TPL];
+  uint32_t pos[TPL];
   if (sg.idx) {
     const uint4 *ip = reinterpret_cast<const uint4 *>(sg.idx + ts);
 #pragma unroll
-    for (int i = 0; i < QK_TPL / 2; ++i) {
+    for (int i = 0; i < TPL / 2; ++i) {
       const uint4 v = ip[i];
       pos[2 * i] = v.x;
       pos[2 * i + 1] = v.z;
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < QK_TPL; ++i) pos[i] = (uint32_t)sg.pos_base + ts + i;
+    for (int i = 0; i < TPL; ++i) pos[i] = (uint32_t)sg.pos_base + ts + i;
   }
-  if constexpr (DS > 1) {  // the quarters of head_dim sit 16 lanes apart: their sum lands in lanes 0-15
-#pragma unroll
-    for (int h = 0; h < NREP; ++h) rows_sum8(acc[h]);
-  }
-  const bool owner = valid && lane < G::TL;
   bool contig = true;
 #pragma unroll
-  for (int i = 1; i < QK_TPL; ++i) contig = contig && (pos[i] == pos[0] + i);
+  for (int i = 1; i < TPL; ++i) contig = contig && (pos[i] == pos[0] + i);
 #pragma unroll
   for (int h = 0; h < NREP; ++h) {
-    half_t v[QK_TPL];
+    half_t v[TPL];
     float m_lane = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < QK_TPL; ++i) {
+    for (int i = 0; i < TPL; ++i) {
       v[i] = (half_t)acc[h][i];
       if (fz.stats) {  // the fp16 steps of the reference epilogue: round the score, scale, round again
         v[i] = (half_t)((float)v[i] * fz.inv_sqrt_d);
@@ -1031,25 +1010,25 @@ __global__ __launch_bounds__(64, NREP <= 4 ? 4 : 2) void qk_wave_kernel(SegTable
       }
     }
     if (fz.stats) {  // (max, sum exp) of the tile
-      if (!owner) m_lane = -INFINITY;
-      const float m = DS > 1 ? row_max16(m_lane) : wave_max(m_lane);
+      if (!valid) m_lane = -INFINITY;
+      const float m = wave_max(m_lane);
       float l_lane = 0.f;
 #pragma unroll
-      for (int i = 0; i < QK_TPL; ++i) l_lane += __expf((float)v[i] - m);
-      if (!owner) l_lane = 0.f;
-      const float l = DS > 1 ? row_sum16(l_lane) : wave_sum(l_lane);
+      for (int i = 0; i < TPL; ++i) l_lane += __expf((float)v[i] - m);
+      if (!valid) l_lane = 0.f;
+      const float l = wave_sum(l_lane);
       if (lane == 0)
         fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
     }
-    if (owner) {
+    if (valid) {
       half_t *srow = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
-      // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one 16-byte
+      // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one vector
       // store; otherwise 2-byte scatters through idx
-      if (contig && (((uintptr_t)(srow + pos[0])) & 15) == 0) {
-        __builtin_memcpy(__builtin_assume_aligned(srow + pos[0], 16), v, 16);
+      if (contig && (((uintptr_t)(srow + pos[0])) & (2 * TPL - 1)) == 0) {
+        __builtin_memcpy(__builtin_assume_aligned(srow + pos[0], 2 * TPL), v, 2 * TPL);
       } else {
 #pragma unroll
-        for (int i = 0; i < QK_TPL; ++i) srow[pos[i]] = v[i];
+        for (int i = 0; i < TPL; ++i) srow[pos[i]] = v[i];
       }
     }
   }
@@ -1169,6 +1148,10 @@ __global__ __launch_bounds__(SM_THREADS) void scale_softmax_reg_kernel(half_t *_
 }
 
 // =============================================================================== p.V
+constexpr int CB_CH = 32;      // combine: channels per workgroup
+constexpr int CB_SLICES = 32;  // combine: chunk slices, slice s adds chunks s, s + 32, ...
+constexpr int CB_FOLD_MAX = 64;  // most chunks per (b, kv head) the last p.V workgroup adds up itself
+constexpr int64_t CB_FOLD_MIN_TOKEN_ROWS = 2 << 20;  // ... and the least V token rows (tokens x B x Hkv) for which it pays
 constexpr int PV_THREADS = 256;
 constexpr int PV_WAVES = 4;
 constexpr int PV_CPL = 8;                        // channels per lane
@@ -1467,19 +1450,78 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
     }
   }
   __syncthreads();
+  const bool fold = fz.arrive != nullptr;
   for (int k = threadIdx.x; k < NREP * D; k += PV_THREADS) {
     const float v = red[k] + red[NREP * D + k] + red[2 * NREP * D + k] + red[3 * NREP * D + k];
     const int h = k / D, d = k % D;
-    partial[((int64_t)chunk_id * n_bhq + (int64_t)b * Hq + hkv * NREP + h) * D + d] = v;
+    float *dst = partial + ((int64_t)chunk_id * n_bhq + (int64_t)b * Hq + hkv * NREP + h) * D + d;
+    if (fold) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // write-through
+    else *dst = v;
   }
+  if (!fold) return;
+  // ---- the last workgroup of this (b, kv head) to get here adds up all partial rows
+  __shared__ uint32_t s_last;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial stores are acknowledged
+  __syncthreads();
+  const int n_chunks = tb.total_units;
+  if (threadIdx.x == 0) {
+    const uint32_t seen = __hip_atomic_fetch_add(&fz.arrive[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (seen + 1u == (uint32_t)n_chunks) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  // Same association as pv_combine_kernel: 32 slices (chunks s, s + 32, ...) each summed ascending from zero,
+  // slices 2w and 2w + 1 added, the 16 pair sums added in order.  A thread owns two adjacent channels of one
+  // query head (8-byte loads, which go past the L2 like the stores did).
+  static_assert(D % 2 == 0, "channel pairs");
+  for (int o = threadIdx.x; o < NREP * (D / 2); o += PV_THREADS) {
+    const int h = o / (D / 2), d = 2 * (o % (D / 2));
+    const int64_t row = (int64_t)b * Hq + hkv * NREP + h;
+    const uint64_t *src = reinterpret_cast<const uint64_t *>(partial + row * D + d);
+    const int64_t cstride = n_bhq * D / 2;  // in 8-byte units
+    float t0 = 0.f, t1 = 0.f;
+    static_assert(CB_FOLD_MAX == 2 * CB_SLICES, "a slice holds at most two chunks here");
+#pragma unroll
+    for (int w0 = 0; w0 < CB_SLICES / 2; w0 += 4) {
+      // sixteen loads requested together (a missing chunk re-reads chunk 0 and counts as zero), then the sums
+      uint64_t raw[4][2][2];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+#pragma unroll
+          for (int r = 0; r < 2; ++r) {
+            const int c = 2 * (w0 + k) + e + r * CB_SLICES;
+            raw[k][e][r] = __hip_atomic_load(src + (int64_t)(c < n_chunks ? c : 0) * cstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float v[2][2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          v[e][0] = v[e][1] = 0.f;
+#pragma unroll
+          for (int r = 0; r < 2; ++r) {
+            const int c = 2 * (w0 + k) + e + r * CB_SLICES;
+            const bool in = c < n_chunks;
+            v[e][0] += in ? __builtin_bit_cast(float, (uint32_t)raw[k][e][r]) : 0.f;
+            v[e][1] += in ? __builtin_bit_cast(float, (uint32_t)(raw[k][e][r] >> 32)) : 0.f;
+          }
+        }
+        const float p0 = v[0][0] + v[1][0], p1 = v[0][1] + v[1][1];
+        t0 = (w0 + k == 0) ? p0 : t0 + p0;
+        t1 = (w0 + k == 0) ? p1 : t1 + p1;
+      }
+    }
+    *reinterpret_cast<half2_t *>(fz.out + row * D + d) = pack_h2((half_t)t0, (half_t)t1);
+  }
+  if (threadIdx.x == 0) __hip_atomic_store(&fz.arrive[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // fixed-order sum over chunks: deterministic replacement for the reference's half atomics
 // (quant/csrc/gemv_cuda_wv_uniform.cu:110).  One workgroup per (b, hq) row and 128 channels; CB_SLICES
 // slices of the chunk list are summed in parallel (strided, ascending within a slice, eight requests in
 // flight per thread), then the slices in order.
-constexpr int CB_CH = 32;      // channels per workgroup
-constexpr int CB_SLICES = 32;  // chunk slices per workgroup: slice s adds chunks s, s + 32, ...
 __global__ __launch_bounds__(CB_CH * CB_SLICES) void pv_combine_kernel(const float *__restrict__ partial,
                                                                       half_t *__restrict__ out, int n_chunks,
                                                                       int64_t n_bhq, int D) {
@@ -1587,9 +1629,9 @@ static int check_heads(const char *who, int64_t B, int64_t Hq, int64_t Hkv, int6
 }
 
 // q.K^T tilings (HQEKV_QK_TILING_*): 1 = 8 waves per 512-token tile, 2 = 4 waves per tile (both split head_dim
-// over the waves of a workgroup), 3 = one wave per 512-token tile, 4 = one wave per 128-token tile.
+// over the waves of a workgroup), 3 = one wave per 512-token tile, 4 = one wave per 256-token tile.
 static int qk_tiling_of(int flags) { return (flags >> 4) & 0xf; }
-static int64_t qk_tile_of(int tiling) { return tiling == 4 ? qw_tile(4) : QK_TILE; }
+static int64_t qk_tile_of(int tiling) { return tiling == 4 ? qw_tile(4) : QK_TILE; }   // qw_tile(8) == QK_TILE
 
 // The one-wave tilings read head_dim 128 with 16-byte row accesses: every channel-major fp16 class must hold a
 // multiple of 8 tokens.
@@ -1627,11 +1669,11 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
   const int nrep = (int)(Hq / Hkv);
   dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units);
   if (tiling >= 3) {
-#define LAUNCH(N_, DS_)                                                                                        \
-  hipLaunchKernelGGL((qk_wave_kernel<N_, DS_>), grid, dim3(64), 0, st, tb, (const half_t *)q, (half_t *)scores, \
+#define LAUNCH(N_, TPL_)                                                                                        \
+  hipLaunchKernelGGL((qk_wave_kernel<N_, TPL_>), grid, dim3(64), 0, st, tb, (const half_t *)q, (half_t *)scores, \
                      (int)Hq, (int)Hkv, Tall, fz)
 #define LAUNCH_DS(N_) \
-  if (tiling == 3) LAUNCH(N_, 1); else LAUNCH(N_, 4)
+  if (tiling == 3) LAUNCH(N_, 8); else LAUNCH(N_, 4)
     switch (nrep) {
       case 1: LAUNCH_DS(1); break;
       case 2: LAUNCH_DS(2); break;
@@ -1703,7 +1745,7 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
     int rc = check_launch("pv_hybrid_kernel");
     if (rc) return rc;
   }
-  if (!(stages & 2)) return HQEKV_OK;
+  if (!(stages & 2) || fz.arrive) return HQEKV_OK;   // folded: the last p.V workgroups have written the output
   hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq, (unsigned)((D + CB_CH - 1) / CB_CH)), dim3(CB_CH * CB_SLICES), 0, st, partial,
                      (half_t *)out, (int)tb.total_units, n_bhq, (int)D);
   return check_launch("pv_combine_kernel");
@@ -1783,8 +1825,8 @@ extern "C" int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, v
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 struct DecodeLayout {  // carve-up of the caller's workspace
-  int64_t chunk, partial_bytes, stats_off, stats_bytes, total;
-  int64_t n_stat;
+  int64_t chunk, partial_bytes, stats_off, stats_bytes, arrive_off, total;
+  int64_t n_stat, chunks;
 };
 
 static int decode_layout(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v, int64_t B,
@@ -1801,7 +1843,7 @@ static int decode_layout(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_se
   for (int k = 0; k < n_k; ++k)
     if (k_segs[k].n_tokens > 0) {
       // room for the statistics of the smallest tile any tiling uses (the token-major residual: 64 tokens)
-      const int64_t per = (k_segs[k].bits == 16 && k_segs[k].layout == HQEKV_LAYOUT_TOKEN_MAJOR) ? 64 : qw_tile(4);
+      const int64_t per = (k_segs[k].bits == 16 && k_segs[k].layout == HQEKV_LAYOUT_TOKEN_MAJOR) ? 64 : qw_tile(4);   // 256
       tiles += (k_segs[k].n_tokens + per - 1) / per;
     }
   if (tiles == 0) tiles = 1;
@@ -1809,7 +1851,9 @@ static int decode_layout(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_se
   L->partial_bytes = align_up(chunks * B * Hq * D * (int64_t)sizeof(float), 256);
   L->stats_off = L->partial_bytes;
   L->stats_bytes = align_up(B * Hq * tiles * (int64_t)sizeof(float2), 256);
-  L->total = L->stats_off + L->stats_bytes;
+  L->arrive_off = L->stats_off + L->stats_bytes;
+  L->chunks = chunks;
+  L->total = L->arrive_off + align_up(B * Hkv * (int64_t)sizeof(uint32_t), 256);
   return HQEKV_OK;
 }
 
@@ -1853,6 +1897,17 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
     fz.stats = (float2 *)(ws + L.stats_off);
     fz.n_stat = (int32_t)kt.total_units;
     fz.inv_sqrt_d = 1.0f / (float)sqrt((double)D);
+  }
+  // Few chunks per (b, kv head) and a long p.V launch: the last p.V workgroup of each (b, kv head) adds the
+  // partials up and the combine launch is dropped.  The write-through stores, the counter and the final loads
+  // lengthen every workgroup's tail by 5-8 us, which only a launch of some 100 us absorbs (B=8 at 64k context:
+  // step 204 -> 198 us; B=1 at 32k: p.V 14 -> 22 us against a 3 us combine, so short launches keep the combine).
+  const bool fold_pays = seg_total_tokens(v_segs, n_v) * B * Hkv >= CB_FOLD_MIN_TOKEN_ROWS;
+  const bool fold_forced = (flags & HQEKV_FOLD_COMBINE) != 0;
+  if (kt.total_units > 0 && vt.total_units > 0 && vt.total_units <= CB_FOLD_MAX && !(flags & HQEKV_SEPARATE_COMBINE) &&
+      (fold_pays || fold_forced)) {
+    fz.arrive = (uint32_t *)(ws + L.arrive_off);
+    fz.out = (half_t *)attn_out;
   }
   const int only = flags & (HQEKV_ONLY_QK | HQEKV_ONLY_PV | HQEKV_ONLY_COMBINE);
   const bool only_qk = only == HQEKV_ONLY_QK;

@@ -46,7 +46,7 @@ def _gemv_group(entry: str, who: str, group_size: int, fA: torch.Tensor, qB: tor
         raise ValueError("scales/zeros shape does not match qB")
     lib = _lib.load()
     out = torch.empty(B, nh_q, 1, N, dtype=torch.float16, device=fA.device)
-    with torch.cuda.device(fA.device):
+    with _lib.on_device(fA.device):
         need = lib.hqekv_gemv_workspace_bytes(B, nh_q, nh_kv, K, N, bits)
         ws = torch.empty(max(need, 16) // 4, dtype=torch.float32, device=fA.device)
         rc = getattr(lib, entry)(fA.data_ptr(), qB.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
@@ -139,7 +139,7 @@ def cuda_bmm_forward_qk_group_hq(group_size, nh_kv, in_vector, matrix_16, matrix
         raise ValueError("cache shape does not match nh_kv / head_dim")
     out = torch.zeros(B, nh_q, 1, Tall, dtype=torch.float16, device=dev)
     segs = _lib.make_segs(items)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = _lib.load().hqekv_qk_hybrid(segs, len(items), in_vector.data_ptr(), out.data_ptr(), B, nh_q,
                                          nh_kv, D, Tall, _lib.stream_ptr(dev))
     _lib.check(rc, "cuda_bmm_forward_qk_group_hq")
@@ -171,7 +171,7 @@ def cuda_bmm_forward_wv_group_hq(group_size, nh_kv, in_vector, matrix_16, matrix
         raise ValueError("cache shape does not match nh_kv")
     out = torch.empty(B, nh_q, 1, D, dtype=torch.float16, device=dev)
     segs = _lib.make_segs(items)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         ws = _att.workspace_for(segs, len(items), B, nh_q, nh_kv, D, dev)
         rc = _lib.load().hqekv_pv_hybrid(segs, len(items), in_vector.data_ptr(), out.data_ptr(), B, nh_q,
                                          nh_kv, D, Tall, ws.data_ptr(), ws.numel() * 4, _lib.stream_ptr(dev))

@@ -65,7 +65,7 @@ def pack_along_last_dim(data: torch.Tensor, bit: int) -> torch.Tensor:
         raise ValueError("last dim must be a multiple of 32 // bit")
     data = data.contiguous()
     code = torch.empty(B, nh, D, T // pf, dtype=torch.int32, device=data.device)
-    with torch.cuda.device(data.device):
+    with _lib.on_device(data.device):
         _lib.check(_lib.load().hqekv_pack_i32(data.data_ptr(), code.data_ptr(), B * nh * D, T, bit,
                                               _lib.stream_ptr(data.device)), "pack_along_last_dim")
     return code
@@ -81,7 +81,7 @@ def unpack_along_last_dim(code: torch.Tensor, bit: int) -> torch.Tensor:
     code = code.contiguous()
     T = Td * pf
     out = torch.empty(B, nh, D, T, dtype=torch.float16, device=code.device)
-    with torch.cuda.device(code.device):
+    with _lib.on_device(code.device):
         _lib.check(_lib.load().hqekv_dequant_unpack_rows(
             code.data_ptr(), 0, Td, None, None, 0, 0, out.data_ptr(), 0, T, 1, B * nh * D, T, bit,
             _lib.stream_ptr(code.device)), "unpack_along_last_dim")
@@ -119,7 +119,7 @@ def quantize_pack_into(
         raise ValueError("scale and mn must share strides")
     lib = _lib.load()
     st = _lib.stream_ptr(data.device)
-    with torch.cuda.device(data.device):
+    with _lib.on_device(data.device):
         tm = (data.stride(2) == 1 and data.stride(3) == R and data.stride(1) == R * L
               and data.stride(0) == nh * R * L and R % 2 == 0 and R > 1)
         if tm:
@@ -170,7 +170,7 @@ def uniform_group_dequantize_unpack_last_dim(
         raise ValueError("scale/mn shapes do not match the codes")
     code, scale, mn = code.contiguous(), scale.contiguous(), mn.contiguous()
     out = torch.empty(B, nh, D, T, dtype=torch.float16, device=code.device)
-    with torch.cuda.device(code.device):
+    with _lib.on_device(code.device):
         _lib.check(_lib.load().hqekv_dequant_unpack_rows(
             code.data_ptr(), 0, Td, scale.data_ptr(), mn.data_ptr(), 0, T // GROUP,
             out.data_ptr(), 0, T, 1, B * nh * D, T, bit, _lib.stream_ptr(code.device)),
@@ -207,7 +207,7 @@ def normal_group_quantize_pack_last_dim(data: torch.Tensor, group_size: int, bit
         return code, std, mean
     lib = _lib.load()
     st = _lib.stream_ptr(dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         tm = (data.stride(2) == 1 and data.stride(3) == R and data.stride(1) == R * L
               and data.stride(0) == nh * R * L and R % 2 == 0 and R > 1)
         if tm:   # the transposed view of token-major K, read in place
@@ -241,7 +241,7 @@ def normal_group_dequantize_unpack_last_dim(code: torch.Tensor, std: torch.Tenso
         raise ValueError("std/mean shapes do not match the codes")
     code, std, mean = code.contiguous(), std.contiguous(), mean.contiguous()
     out = torch.empty(B, nh, D, T, dtype=torch.float16, device=code.device)
-    with torch.cuda.device(code.device):
+    with _lib.on_device(code.device):
         _lib.check(_lib.load().hqekv_normal1_dequant_unpack_rows(
             code.data_ptr(), 0, Td, std.data_ptr(), mean.data_ptr(), 0, T // GROUP,
             out.data_ptr(), 0, T, 1, B * nh * D, T, _lib.stream_ptr(code.device)),

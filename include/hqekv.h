@@ -228,12 +228,17 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
  * (the summation order over head_dim differs), so tests and measurements can name a tiling per call.
  */
 #define HQEKV_FUSE_SOFTMAX 1
+#define HQEKV_SEPARATE_COMBINE 2 /* always sum the split-K partials with a launch of their own                       */
+#define HQEKV_FOLD_COMBINE 4     /* let the last p.V workgroup of each (b, kv head) sum them whenever there are at
+                                    most 64 chunks; by default that is done only for long launches (>= 2^21 V token
+                                    rows), where it saves more than it costs.  Both ways add in the same order and
+                                    give the same bits                                                            */
 #define HQEKV_QK_TILING(n) (((n) & 0xf) << 4)
 #define HQEKV_QK_TILING_8WAVES 1 /* 512-token tile, head_dim split over 8 waves (launches of <= 1024 tiles) */
 #define HQEKV_QK_TILING_4WAVES 2 /* 512-token tile, head_dim split over 4 waves                              */
 #define HQEKV_QK_TILING_WAVE512 3 /* one wave per 512-token tile, no split of head_dim (launches of > 1024 tiles;
                                      needs head_dim 128 and fp16 classes of a multiple of 8 tokens)          */
-#define HQEKV_QK_TILING_WAVE128 4 /* one wave per 128-token tile, head_dim split over four groups of 16 lanes */
+#define HQEKV_QK_TILING_WAVE256 4 /* one wave per 256-token tile: twice the waves per SIMD (same requirements)  */
 #define HQEKV_ONLY_QK 0x100
 #define HQEKV_ONLY_PV 0x200
 #define HQEKV_ONLY_COMBINE 0x400

@@ -332,6 +332,29 @@ def test_segment_memo_gives_the_same_bits(dev):
             assert memo.lookup(tuple(c), torch.device(dev), True)
 
 
+@pytest.mark.parametrize("case", [CASES[1], CASES[2], CASES[5], CASES[6]], ids=lambda c: f"B{c['B']}Hq{c['Hq']}T{c['T']}")
+@pytest.mark.parametrize("fused", [1, 0], ids=["fused", "general"])
+def test_folded_combine_equals_the_combine_launch(dev, case, fused):
+    """The split-K partials are added up by the last p.V workgroup of each (b, kv head) (HQEKV_FOLD_COMBINE; the
+    default for long launches) or by a launch of their own (HQEKV_SEPARATE_COMBINE): same order of additions, so
+    the outputs are bit-identical -- on repeated calls over one workspace as well (the arrival counters are
+    re-armed by every call)."""
+    from hqekv_amd import _lib
+    from hqekv_amd.attention import DecodePlan
+    q, cache = _case(**case)
+    c = synth.cache_to(cache, dev)
+    folded = DecodePlan(q.to(dev), c, flags=fused | _lib.FOLD_COMBINE)
+    apart = DecodePlan(q.to(dev), c, flags=fused | _lib.SEPARATE_COMBINE)
+    g = torch.Generator().manual_seed(5)
+    for rep in range(4):
+        qn = torch.randn(q.shape, generator=g).half().to(dev)
+        w0, o0 = [x.clone() for x in folded.run(qn)]
+        w1, o1 = [x.clone() for x in apart.run(qn)]
+        assert torch.equal(w0, w1) and torch.equal(o0, o1), rep
+    w_ref, o_ref = O.qkv_matmul(qn.cpu(), cache, None, case["D"], use_mask=False, round_per_class=False)
+    _close(o0, o_ref, "attn_output")
+
+
 @pytest.mark.parametrize("flags", [1, 0], ids=["fused", "general"])
 def test_plan_replayed_from_a_hip_graph(dev, flags):
     """A captured decode step (no allocation, no memset inside) replayed several times with new queries,

@@ -62,7 +62,7 @@ def _c4_mix_case(permute: bool):
 
 
 @pytest.mark.parametrize("permute", [False, True], ids=["blockidx", "randperm"])
-@pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave128", "auto"])
+@pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave256", "auto"])
 @pytest.mark.parametrize("fused", [True, False], ids=["fused", "general"])
 def test_config4_mix_batch8_every_row(dev, tiling, permute, fused):
     """Configuration 4's class mix at B=8, 32 query heads over 8 KV heads, 16384 tokens: a launch of more than
@@ -80,7 +80,7 @@ def test_config4_mix_batch8_every_row(dev, tiling, permute, fused):
     torch.testing.assert_close(w.float().sum(-1).cpu(), torch.ones(B, Hq, 1), rtol=0, atol=5e-3)
 
 
-@pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave128"])
+@pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave256"])
 @pytest.mark.parametrize("n_rep", [1, 2, 4, 8])
 @pytest.mark.parametrize("low_normal", [False, True], ids=["uniform1", "normal1"])
 def test_every_tiling_every_gqa_ratio(dev, tiling, n_rep, low_normal):
