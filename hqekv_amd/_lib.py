@@ -19,6 +19,7 @@ MAX_SEGS = 8
 FUSE_SOFTMAX = 1
 SEPARATE_COMBINE = 2
 FOLD_COMBINE = 4
+TWO_STEP_DEQUANT = 8
 ONLY_QK = 0x100
 ONLY_PV = 0x200
 ONLY_COMBINE = 0x400

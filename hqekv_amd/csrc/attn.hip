@@ -86,6 +86,7 @@ struct FuseArgs {
   // launch of the same call; nullptr = the split-K partials are summed by a launch of their own.
   uint32_t *arrive;
   half_t *out;         // (B*Hq, D) attention output, written by the last workgroup of each (b, kv head)
+  int32_t two_step;    // never fold the bias removal of a code into its multiply (HQEKV_TWO_STEP_DEQUANT)
 };
 
 // A workgroup learns its segment and its tile/chunk from its block id with two scalar loads at the top of
@@ -151,6 +152,29 @@ __device__ __forceinline__ half2_t field_pair(uint32_t u) {
   return biased - bias;                                 // c, exact
 }
 
+// The same field still carrying its bias: 2^(10-POS) + c.
+template <int BITS, int I>
+__device__ __forceinline__ half2_t field_pair_biased(uint32_t u) {
+  constexpr int POS = I * BITS;
+  constexpr uint32_t FMASK = ((1u << BITS) - 1u) << POS;
+  constexpr uint32_t MASK = FMASK | (FMASK << 16);
+  constexpr uint32_t EXPO = (uint32_t)(10 - POS + 15) << 10;
+  constexpr uint32_t MAGIC = EXPO | (EXPO << 16);
+  uint32_t r;
+  const uint32_t magic_v = MAGIC;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(u), "s"(MASK), "v"(magic_v));
+  return as_h2(r);
+}
+// -2^(10-POS) * s for field I: with it rnd16(c * s) is ONE fused multiply-add on the biased field,
+// (2^(10-POS) + c) * s - 2^(10-POS) * s = c * s before the single rounding -- exactly the product the reference
+// rounds -- provided 2^(10-POS) * s is itself an fp16 number, i.e. |s| < 64 at POS = 0 (scaling by a power of two
+// is exact short of overflow).  Callers take this route only after checking the scales of the whole tile.
+template <int BITS, int I>
+__device__ __forceinline__ half2_t bias_times_scale(half2_t s2) {
+  constexpr _Float16 NB = (_Float16)(-(float)(1 << (10 - I * BITS)));
+  return s2 * (half2_t){NB, NB};
+}
+
 // the reference dequantiser's two roundings (quant/pack_unpack.py:331-332) on a pair of codes
 __device__ __forceinline__ half2_t dequant_pair(half2_t c, half2_t s2, half2_t z2) {
   const half2_t m = c * s2;
@@ -181,6 +205,29 @@ __device__ __forceinline__ void consume_byte(uint32_t u, half2_t s2, half2_t z2,
     const half2_t x2 = NORMAL ? dequant_pair_normal1(c2_, s2, z2) : dequant_pair(c2_, s2, z2);  \
     _Pragma("unroll") for (int h = 0; h < NREP; ++h)                                     \
         acc[h][tok0 + I_] = __builtin_amdgcn_fdot2(x2, a2[h], acc[h][tok0 + I_], false); \
+  }
+  HQ_FIELD(0)
+  HQ_FIELD(1)
+  HQ_FIELD(2)
+  HQ_FIELD(3)
+  HQ_FIELD(4)
+  HQ_FIELD(5)
+  HQ_FIELD(6)
+  HQ_FIELD(7)
+#undef HQ_FIELD
+}
+
+// The same with the bias removal folded into the multiply (see bias_times_scale): nb[I] = -2^(10-POS_I) * s2.
+template <int BITS, int NREP, int PF, int NFIELD>
+__device__ __forceinline__ void consume_byte_fused_bias(uint32_t u, half2_t s2, half2_t z2, const half2_t (&nb)[8 / BITS],
+                                                        const half2_t (&a2)[NREP], float (&acc)[NREP][PF], int tok0) {
+#define HQ_FIELD(I_)                                                                      \
+  if constexpr (I_ < NFIELD) {                                                            \
+    const half2_t b2_ = field_pair_biased<BITS, (I_ < NFIELD ? I_ : 0)>(u);               \
+    const half2_t m2_ = __builtin_elementwise_fma(b2_, s2, nb[I_ < NFIELD ? I_ : 0]);     \
+    const half2_t x2 = m2_ + z2;                                                          \
+    _Pragma("unroll") for (int h = 0; h < NREP; ++h)                                      \
+        acc[h][tok0 + I_] = __builtin_amdgcn_fdot2(x2, a2[h], acc[h][tok0 + I_], false);  \
   }
   HQ_FIELD(0)
   HQ_FIELD(1)
@@ -732,8 +779,9 @@ __device__ __forceinline__ QwRow<BITS, TPL> qw_load_row(rsrc_t rc, uint32_t lane
 // Stage the scale/zero rows of one tile: sz[dp * NG + g] = {(s[2dp][g], s[2dp+1][g]), (z[2dp][g], z[2dp+1][g])}.
 // Groups past the end of the class read whatever follows (the next row, or zero past the slab): only lanes
 // whose tokens do not exist look at them.
+// Returns true when every scale this lane staged is finite and below 32 in magnitude.
 template <int TPL, bool NORMAL>
-__device__ __forceinline__ void qw_stage_sz(const SegDev &sg, int tile, int bh, int lane, uint2 *sz) {
+__device__ __forceinline__ bool qw_stage_sz(const SegDev &sg, int tile, int bh, int lane, uint2 *sz) {
   using G = QwGeom<TPL>;
   constexpr int NG = G::NG, GPI = G::GPI;
   constexpr int ITEMS = 64 * NG / GPI;   // (row pair, part of the tile's groups)
@@ -741,6 +789,7 @@ __device__ __forceinline__ void qw_stage_sz(const SegDev &sg, int tile, int bh, 
   const rsrc_t rs = make_rsrc(sg.scale + (int64_t)bh * 128 * gpr, 128u * gpr * 2u);
   const rsrc_t rz = make_rsrc(sg.zero + (int64_t)bh * 128 * gpr, 128u * gpr * 2u);
   const uint32_t g0 = (uint32_t)tile * NG;
+  uint32_t big = 0;  // bit 15 / 31 set once an |scale| >= 32 (fp16 0x5000), an infinity or a NaN has been seen
 #pragma unroll 1   // one item's sixteen registers at a time: the accumulators are live across this
   for (int k = 0; k < ITEMS / 64; ++k) {
     const int it = lane + 64 * k;
@@ -778,6 +827,7 @@ __device__ __forceinline__ void qw_stage_sz(const SegDev &sg, int tile, int bh, 
     uint4 *dst = reinterpret_cast<uint4 *>(sz + dp * NG + part * GPI);
 #pragma unroll
     for (int j = 0; j < GPI / 2; ++j) {
+      big |= ((sa[j] & 0x7fff7fffu) + 0x30003000u) | ((sb[j] & 0x7fff7fffu) + 0x30003000u);
       half2_t s_lo = half_pair<0>(sa[j], sb[j]), s_hi = half_pair<1>(sa[j], sb[j]);
       if (NORMAL) {  // the spread a = rnd16(k * std) once per group instead of once per use
         s_lo = normal1_spread(s_lo);
@@ -786,6 +836,7 @@ __device__ __forceinline__ void qw_stage_sz(const SegDev &sg, int tile, int bh, 
       dst[j] = make_uint4(as_u32(s_lo), as_u32(half_pair<0>(za[j], zb[j])), as_u32(s_hi), as_u32(half_pair<1>(za[j], zb[j])));
     }
   }
+  return (big & 0x80008000u) == 0;
 }
 
 template <int BITS, int NREP, int TPL, bool NORMAL, typename Stage>
@@ -815,7 +866,8 @@ __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t t
       b.r1[k] = qw_load_row<BITS, TPL>(rc, lane_off, row + rowb);
     }
   };
-  auto compute = [&](int i0, const Block &b) {
+  auto compute = [&](int i0, const Block &b, auto fused_bias) {
+    constexpr bool FB = decltype(fused_bias)::value;
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const int i = i0 + k;
@@ -827,6 +879,13 @@ __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t t
       constexpr int FPB = 8 / BITS;                 // codes per byte
       constexpr int NBYTE = (NB + 7) / 8;           // bytes per lane and row
       constexpr int NF = NB < 8 ? NB / BITS : FPB;  // codes taken from a byte
+      half2_t nb[FPB];
+      if constexpr (FB) {   // -2^(10-pos) * s for every field position, once per row pair
+#define HQ_NB(I_) \
+  if constexpr (I_ < NF) nb[I_ < FPB ? I_ : 0] = bias_times_scale<BITS, (I_ < FPB ? I_ : 0)>(s2);
+        HQ_NB(0) HQ_NB(1) HQ_NB(2) HQ_NB(3) HQ_NB(4) HQ_NB(5) HQ_NB(6) HQ_NB(7)
+#undef HQ_NB
+      }
 #pragma unroll
       for (int j = 0; j < NBYTE; ++j) {
         uint32_t a0 = b.r0[k].w[j / 4], a1 = b.r1[k].w[j / 4];
@@ -838,22 +897,35 @@ __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t t
                            : (j % 4 == 1) ? byte_pair<1>(a0, a1)
                            : (j % 4 == 2) ? byte_pair<2>(a0, a1)
                                           : byte_pair<3>(a0, a1);
-        consume_byte<BITS, NREP, TPL, NORMAL, NF>(u, s2, z2, q2, acc, j * FPB);
+        if constexpr (FB) consume_byte_fused_bias<BITS, NREP, TPL, NF>(u, s2, z2, nb, q2, acc, j * FPB);
+        else consume_byte<BITS, NREP, TPL, NORMAL, NF>(u, s2, z2, q2, acc, j * FPB);
       }
     }
   };
   Block ba, bb;
-  load(0, ba);
-  stage();  // query and scale/zero into LDS while the first block is on its way; ends with the barrier
+  load(0, ba);   // in flight across the staging
+  // Query and scale/zero into LDS; the staging also says whether every scale of the tile is small enough for the
+  // multiply that removes the bias on the way (one packed op fewer per pair of codes).  Worth it where a lane has
+  // more codes per row pair than field positions: 8, 4 and 2 bits.
+  const bool small_scales = stage();
+  auto run = [&](auto fused_bias) {
 #pragma unroll 1
-  for (int i0 = 0; i0 < G::RP; i0 += 2 * U) {
-    load(i0 + U, bb);
-    HQ_LOADS_ABOVE();
-    compute(i0, ba);
-    if (i0 + 2 * U < G::RP) load(i0 + 2 * U, ba);
-    HQ_LOADS_ABOVE();
-    compute(i0 + U, bb);
+    for (int i0 = 0; i0 < G::RP; i0 += 2 * U) {
+      load(i0 + U, bb);
+      HQ_LOADS_ABOVE();
+      compute(i0, ba, fused_bias);
+      if (i0 + 2 * U < G::RP) load(i0 + 2 * U, ba);
+      HQ_LOADS_ABOVE();
+      compute(i0 + U, bb, fused_bias);
+    }
+  };
+  if constexpr (!NORMAL && BITS != 1) {
+    if (__builtin_amdgcn_ballot_w64(!small_scales) == 0) {
+      run(std::true_type{});
+      return;
+    }
   }
+  run(std::false_type{});
 }
 
 // fp16 class stored channel-major (B,Hkv,128,T), T a multiple of 8: a lane reads its TPL tokens of a row as 16 or 8 bytes
@@ -957,8 +1029,9 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
 
   auto stage_quant = [&](auto normal) {
     stage_q();
-    qw_stage_sz<TPL, decltype(normal)::value>(sg, tile, bh, lane, sz);
+    const bool small_scales = qw_stage_sz<TPL, decltype(normal)::value>(sg, tile, bh, lane, sz);
     __syncthreads();
+    return small_scales && !fz.two_step;
   };
   auto stage_plain = [&]() {
     stage_q();
@@ -969,13 +1042,13 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
   switch (sg.bits) {
     case 1:
       if (sg.layout == HQEKV_LAYOUT_NORMAL1)
-        qw_quant_accumulate<1, NREP, TPL, true>(sg, ts, bh, lane, [&]() { stage_quant(T{}); }, q2s, sz, acc);
+        qw_quant_accumulate<1, NREP, TPL, true>(sg, ts, bh, lane, [&]() { return stage_quant(T{}); }, q2s, sz, acc);
       else
-        qw_quant_accumulate<1, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc);
+        qw_quant_accumulate<1, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc);
       break;
-    case 2: qw_quant_accumulate<2, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
-    case 4: qw_quant_accumulate<4, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
-    case 8: qw_quant_accumulate<8, NREP, TPL, false>(sg, ts, bh, lane, [&]() { stage_quant(F{}); }, q2s, sz, acc); break;
+    case 2: qw_quant_accumulate<2, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
+    case 4: qw_quant_accumulate<4, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
+    case 8: qw_quant_accumulate<8, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
     default: qw_f16_accumulate<NREP, TPL>(sg, ts, bh, lane, stage_plain, q2s, acc);
   }
 
@@ -1902,6 +1975,7 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
   // partials up and the combine launch is dropped.  The write-through stores, the counter and the final loads
   // lengthen every workgroup's tail by 5-8 us, which only a launch of some 100 us absorbs (B=8 at 64k context:
   // step 204 -> 198 us; B=1 at 32k: p.V 14 -> 22 us against a 3 us combine, so short launches keep the combine).
+  fz.two_step = (flags & HQEKV_TWO_STEP_DEQUANT) ? 1 : 0;
   const bool fold_pays = seg_total_tokens(v_segs, n_v) * B * Hkv >= CB_FOLD_MIN_TOKEN_ROWS;
   const bool fold_forced = (flags & HQEKV_FOLD_COMBINE) != 0;
   if (kt.total_units > 0 && vt.total_units > 0 && vt.total_units <= CB_FOLD_MAX && !(flags & HQEKV_SEPARATE_COMBINE) &&

@@ -233,6 +233,12 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
                                     most 64 chunks; by default that is done only for long launches (>= 2^21 V token
                                     rows), where it saves more than it costs.  Both ways add in the same order and
                                     give the same bits                                                            */
+#define HQEKV_TWO_STEP_DEQUANT 8  /* The kernels read a code c out of a packed word as the fp16 number bias + c.  The
+                                    one-wave q.K^T tilings turn a tile whose scales are all below 32 in magnitude into
+                                    c * s with one fused multiply-add, (bias + c) * s - bias * s (bias * s is exact
+                                    there, so the product is rounded once, like the reference's), and any other tile
+                                    with a subtraction and a multiplication.  This flag takes the second route for
+                                    every tile; the bits are the same, and tests compare the two                  */
 #define HQEKV_QK_TILING(n) (((n) & 0xf) << 4)
 #define HQEKV_QK_TILING_8WAVES 1 /* 512-token tile, head_dim split over 8 waves (launches of <= 1024 tiles) */
 #define HQEKV_QK_TILING_4WAVES 2 /* 512-token tile, head_dim split over 4 waves                              */

@@ -105,6 +105,43 @@ def test_every_tiling_every_gqa_ratio(dev, tiling, n_rep, low_normal):
         _close(o, o_ref, f"attn_output fused={fused}")
 
 
+@pytest.mark.parametrize("tiling", ["wave512", "wave256"])
+@pytest.mark.parametrize("outliers", [False, True], ids=["small_scales", "large_scales"])
+def test_fused_bias_removal_gives_the_same_bits(dev, tiling, outliers):
+    """The one-wave tilings dequantise a tile whose scales are all below 32 with one fused multiply-add per pair of
+    codes, and any other tile with the subtraction and the multiplication apart; the flag that forces the second
+    route everywhere must not change a bit of the probabilities.  With outliers, some 32-token blocks of K are
+    scaled up until their 2-, 4- and 8-bit scales pass 32 (both routes inside one launch), and the oracle still
+    agrees; the query is zero in the outlier channels' share so that the logits stay in range."""
+    from hqekv_amd import _lib
+    from hqekv_amd.attention import decode_attention
+    B, Hq, Hkv, D, residual = 2, 8, 2, 128, 11
+    T = 96 * 32 + residual
+    q, K, V = synth.make_qkv(B, Hq, Hkv, T, D, 77)
+    if outliers:
+        g = torch.Generator().manual_seed(78)
+        blocks = torch.randperm((T - residual) // 32, generator=g)[:24]
+        for j in blocks.tolist():
+            K[:, :, j * 32:(j + 1) * 32, 8:16] *= 3000.0   # 8-bit scale ~ 6 * 3000 / 255 = 70
+        assert bool(torch.isfinite(K).all())
+        q[..., 8:16] = 0
+    classes = synth.split_blocks(T - residual, (0.1, 0.2, 0.3, 0.3, 0.1, 0.0), 77)
+    cache = synth.build_cache(K, V, classes, residual, O.uniform_group_quantize_pack_last_dim)
+    if outliers:
+        assert max(float(cache[s].abs().max()) for s in (6, 14, 22) if cache[s] is not None) >= 32.0  # K scales
+    Tall = cache[41]
+    w_ref, o_ref = O.qkv_matmul(q, cache, None, D, use_mask=False, round_per_class=False)
+    n = dict(_tilings())[tiling]
+    dcache = synth.cache_to(cache, dev)
+    for fused in (True, False):
+        w1, o1 = decode_attention(q.to(dev), dcache, None, Tall, zero_init=True, flags=_flags(fused, n))
+        w2, o2 = decode_attention(q.to(dev), dcache, None, Tall, zero_init=True,
+                                  flags=_flags(fused, n) | _lib.TWO_STEP_DEQUANT)
+        assert torch.equal(w1, w2) and torch.equal(o1, o2)
+        _close(w1, w_ref, "attn_weights")
+        _close(o1, o_ref, "attn_output")
+
+
 def test_unknown_tiling_is_an_error(dev):
     from hqekv_amd import _lib
     from hqekv_amd.attention import decode_attention
