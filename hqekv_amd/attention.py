@@ -258,41 +258,50 @@ class SegmentMemo:
         self.keep = []
         k_items, hk, dk = key_segments(pkv, dev, 0, self.keep, low_uniform, residual=False)
         v_items, hv, dv = value_segments(pkv, dev, 0, self.keep, low_uniform, residual=False)
-        if len(k_items) + 1 > _lib.MAX_SEGS or len(v_items) + 1 > _lib.MAX_SEGS:
+        if len(k_items) + 2 > _lib.MAX_SEGS or len(v_items) + 2 > _lib.MAX_SEGS:
             raise ValueError("too many segments")
         self.n_k, self.n_v = len(k_items), len(v_items)
-        self.k_arr = (_lib.Seg * (self.n_k + 1))()   # one spare entry each for the residual
-        self.v_arr = (_lib.Seg * (self.n_v + 1))()
+        self.k_arr = (_lib.Seg * (self.n_k + 2))()   # two spare entries each: the residual and the step's new token
+        self.v_arr = (_lib.Seg * (self.n_v + 2))()
         for dst, src in ((self.k_arr, _lib.make_segs(k_items)), (self.v_arr, _lib.make_segs(v_items))):
-            for i in range(len(dst) - 1):
+            for i in range(len(dst) - 2):
                 C.memmove(C.byref(dst[i]), C.byref(src[i]), C.sizeof(_lib.Seg))
+        self.need = {}                                # workspace bytes per (residual, tail, B, Hq) of this cache
         self.Hkv = hk if hk is not None else hv
         self.dims = (dk, dv)
         self.held = tuple(pkv[:NEW_K])
         self.key = (dev, low_uniform)
         self.partition = classes_partition_positions(pkv)
 
-    def tables(self, pkv: tuple, Tall: int, keep: list):
-        """-> (k_segs, n_k, v_segs, n_v, Hkv, (dk, dv)) with this step's residual filled in."""
+    @staticmethod
+    def _fill(s, t: torch.Tensor, end: int, layout: int, keep: list):
+        """Table entry of an fp16 token-major block (B,Hkv,n,D) whose last token sits at position end - 1."""
+        tc = t.contiguous()
+        keep.append(tc)
+        n = tc.shape[2]
+        s.bits, s.layout, s.n_tokens, s.pos_base, s.data = 16, layout, n, end - n, tc.data_ptr()
+        return tc.shape[1], tc.shape[3]
+
+    def tables(self, pkv: tuple, Tall: int, keep: list, tail=None):
+        """-> (k_segs, n_k, v_segs, n_v, Hkv, (dk, dv), (residual tokens, tail tokens)) with this step's residual
+        -- and the tokens of ``tail`` = (k, v), which follow it -- filled in."""
         n_k, n_v, Hkv, (dk, dv) = self.n_k, self.n_v, self.Hkv, self.dims
+        n_tail = tail[0].shape[2] if tail is not None else 0
+        n_res = 0
         new_K, new_V = pkv[NEW_K], pkv[NEW_V]
         if new_K is not None and new_K.shape[2] > 0:
-            nk = new_K.contiguous()
-            keep.append(nk)
-            s = self.k_arr[n_k]
-            s.bits, s.layout, s.n_tokens, s.pos_base = 16, _lib.LAYOUT_TOKEN_MAJOR, nk.shape[2], Tall - nk.shape[2]
-            s.data = nk.data_ptr()
+            n_res = new_K.shape[2]
+            Hkv, dk = self._fill(self.k_arr[n_k], new_K, Tall - n_tail, _lib.LAYOUT_TOKEN_MAJOR, keep)
             n_k += 1
-            Hkv, dk = nk.shape[1], nk.shape[3]
         if new_V is not None and new_V.shape[2] > 0:
-            nv = new_V.contiguous()
-            keep.append(nv)
-            s = self.v_arr[n_v]
-            s.bits, s.layout, s.n_tokens, s.pos_base = 16, 0, nv.shape[2], Tall - nv.shape[2]
-            s.data = nv.data_ptr()
+            Hkv, dv = self._fill(self.v_arr[n_v], new_V, Tall - n_tail, 0, keep)
             n_v += 1
-            Hkv, dv = nv.shape[1], nv.shape[3]
-        return self.k_arr, n_k, self.v_arr, n_v, Hkv, (dk, dv)
+        if n_tail:
+            Hkv, dk = self._fill(self.k_arr[n_k], tail[0], Tall, _lib.LAYOUT_TOKEN_MAJOR, keep)
+            Hkv, dv = self._fill(self.v_arr[n_v], tail[1], Tall, 0, keep)
+            n_k += 1
+            n_v += 1
+        return self.k_arr, n_k, self.v_arr, n_v, Hkv, (dk, dv), (n_res, n_tail)
 
     def workspace(self, need: int, dev) -> torch.Tensor:
         if self.ws is None or self.ws.numel() * 4 < need or self.ws.device != dev:
@@ -301,7 +310,7 @@ class SegmentMemo:
 
 
 def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool, flags: Optional[int] = None,
-                     low_uniform: bool = True, memo: Optional[SegmentMemo] = None):
+                     low_uniform: bool = True, memo: Optional[SegmentMemo] = None, tail=None):
     """q (B,Hq,1,D) fp16 -> (attn_weights (B,Hq,1,Tall) fp16 probabilities, attn_output (B,Hq,1,D) fp16).
 
     One q.K^T launch over all K classes and one p.V launch over all V classes with the softmax fused
@@ -309,6 +318,9 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     (q.K^T, scale+mask+clamp+softmax, p.V, fixed-order combine).  Runs on torch's current stream.
     ``memo``: a ``SegmentMemo`` the caller keeps per layer, so that steps between two compressions rebuild
     only the residual's table entry.
+    ``tail`` = (k, v), each (B,Hkv,L,D) fp16: tokens that follow the tuple's residual without being part of it yet
+    (``Tall`` counts them).  The kernels read them as one more fp16 segment per side, so a caller can start the
+    attention of a decode step before it appends the step's key and value to the residual.
     """
     _lib.require_gpu(q, "q")
     if q.dtype != torch.float16:
@@ -322,7 +334,7 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     if memo is not None:
         if not memo.lookup(pkv, dev, low_uniform):
             memo.build(pkv, dev, low_uniform)
-        k_segs, n_k, v_segs, n_v, Hkv, (dk, dv) = memo.tables(pkv, Tall, keep)
+        k_segs, n_k, v_segs, n_v, Hkv, (dk, dv), res_tail = memo.tables(pkv, Tall, keep, tail)
         covered = memo.partition
     else:
         covered = not (use_flags & _lib.FUSE_SOFTMAX) or mask is not None or classes_partition_positions(pkv)
@@ -330,8 +342,15 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
         use_flags &= ~_lib.FUSE_SOFTMAX
         zero_init = True
     if memo is None:
-        k_items, hk, dk = key_segments(pkv, dev, Tall, keep, low_uniform)
-        v_items, hv, dv = value_segments(pkv, dev, Tall, keep, low_uniform)
+        n_tail = tail[0].shape[2] if tail is not None else 0
+        k_items, hk, dk = key_segments(pkv, dev, Tall - n_tail, keep, low_uniform)
+        v_items, hv, dv = value_segments(pkv, dev, Tall - n_tail, keep, low_uniform)
+        if n_tail:
+            tk, tv = tail[0].contiguous(), tail[1].contiguous()
+            keep += [tk, tv]
+            k_items.append(dict(bits=16, n_tokens=n_tail, data=tk, idx=None, pos_base=Tall - n_tail, token_major=1))
+            v_items.append(dict(bits=16, n_tokens=n_tail, data=tv, idx=None, pos_base=Tall - n_tail))
+            hk, dk, hv, dv = tk.shape[1], tk.shape[3], tv.shape[1], tv.shape[3]
         Hkv = hk if hk is not None else hv
         k_segs, v_segs, n_k, n_v = _lib.make_segs(k_items), _lib.make_segs(v_items), len(k_items), len(v_items)
     if Hkv is None:
@@ -346,7 +365,10 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     lib = _lib.load()
     with _lib.on_device(dev):
         if memo is not None:
-            need = lib.hqekv_decode_workspace_bytes(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D)
+            need_key = (res_tail, B, Hq)
+            need = memo.need.get(need_key)
+            if need is None:
+                need = memo.need[need_key] = lib.hqekv_decode_workspace_bytes(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D)
             if need < 0:
                 raise ValueError("invalid segment table")
             ws = memo.workspace(need, dev)

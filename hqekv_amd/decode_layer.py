@@ -122,16 +122,21 @@ class HqeAttentionLayer:
         self.current_length += L
         kv_seq_len = L + (past_key_value[-1] if past_key_value is not None else 0)
         if past_key_value is not None:
+            # The attention reads this step's key and value where they are, as a segment behind the residual, and
+            # is queued first; the copies that append them to the residual [131-133] follow it on the stream, off
+            # the step's critical path.
+            attn_weights, attn_output = qkv_matmul_hqe_2(query_states, past_key_value, attention_mask,
+                                                         self.head_dim, self.quant_strategy, memo=self._memo,
+                                                         tail=(key_states, value_states))
+            self.last_weights.update(attn_weights)
             new_K = torch.cat((past_key_value[-3], key_states), dim=2) if past_key_value[-3] is not None else key_states
             new_V = torch.cat((past_key_value[-2], value_states), dim=2) if past_key_value[-2] is not None else value_states
             past_key_value = past_key_value[:-3] + (new_K, new_V, kv_seq_len)
-            attn_weights, attn_output = qkv_matmul_hqe_2(query_states, past_key_value, attention_mask,
-                                                         self.head_dim, self.quant_strategy, memo=self._memo)
         else:
             attn_weights, attn_output = self._prefill(query_states, key_states, value_states, attention_mask)
             past_key_value = (None,) * 39 + (key_states, value_states, kv_seq_len)
+            self.last_weights.update(attn_weights)
 
-        self.last_weights.update(attn_weights)
         if self.current_length < BLOCK:
             self.token_num += 1
             return attn_output, attn_weights, past_key_value, None

@@ -332,6 +332,41 @@ def test_segment_memo_gives_the_same_bits(dev):
             assert memo.lookup(tuple(c), torch.device(dev), True)
 
 
+@pytest.mark.parametrize("ci", [0, 1, 6])
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "general"])
+def test_step_tokens_as_a_tail_segment(dev, ci, fused, monkeypatch):
+    """A decode step may hand its new key / value rows over beside the tuple (``tail``) instead of appending them to
+    the residual first.  Same probabilities bit for bit on the general path (every logit is computed alike and the
+    softmax runs over the whole row), the oracle's result to tolerance on both paths, with and without a memo, for
+    a cache with and without a residual."""
+    from hqekv_amd.attention import SegmentMemo
+    from hqekv_amd.hqe_matmul import qkv_matmul_hqe_2
+    if not fused:
+        monkeypatch.setenv("HQEKV_UNFUSED", "1")
+    case = CASES[ci]
+    q, cache = _case(**case)
+    g = torch.Generator().manual_seed(31 + ci)
+    nk = torch.randn(case["B"], case["Hkv"], 1, case["D"], generator=g).half()
+    nv = torch.randn(case["B"], case["Hkv"], 1, case["D"], generator=g).half()
+    appended = list(cache)
+    appended[39] = nk if cache[39] is None else torch.cat((cache[39], nk), 2)
+    appended[40] = nv if cache[40] is None else torch.cat((cache[40], nv), 2)
+    appended[41] = int(cache[41]) + 1
+    w_ref, o_ref = O.qkv_matmul(q, tuple(appended), None, case["D"], use_mask=False, round_per_class=False)
+    c, ca = synth.cache_to(cache, dev), synth.cache_to(tuple(appended), dev)
+    w0, o0 = qkv_matmul_hqe_2(q.to(dev), ca, None, case["D"], "uniform_group")
+    memo = SegmentMemo()
+    for m in (None, memo, memo):
+        w, o = qkv_matmul_hqe_2(q.to(dev), c, None, case["D"], "uniform_group", memo=m,
+                                tail=(nk.to(dev), nv.to(dev)))
+        assert w.shape == w0.shape
+        if not fused:
+            assert torch.equal(w, w0)
+        _close(w, w_ref, "attn_weights")
+        _close(o, o_ref, "attn_output")
+        _close(o, o0.cpu(), "tail vs appended")
+
+
 @pytest.mark.parametrize("case", [CASES[1], CASES[2], CASES[5], CASES[6]], ids=lambda c: f"B{c['B']}Hq{c['Hq']}T{c['T']}")
 @pytest.mark.parametrize("fused", [1, 0], ids=["fused", "general"])
 def test_folded_combine_equals_the_combine_launch(dev, case, fused):
