@@ -79,9 +79,9 @@ def recorded_traffic(workload: str, kernel: str):
 def side_bytes(pkv, k_side: bool) -> int:
     """Algorithmic bytes of the K side (q.K^T launch) or V side (p.V launch) of one layer-step."""
     if k_side:
-        slots = (0, 1, 4, 5, 6, 7, 12, 13, 14, 15, 20, 21, 22, 23, 39)
+        slots = (0, 1, 4, 5, 6, 7, 12, 13, 14, 15, 20, 21, 22, 23, 28, 29, 30, 31, 39)
     else:
-        slots = (2, 3, 8, 9, 10, 11, 16, 17, 18, 19, 24, 25, 26, 27, 40)
+        slots = (2, 3, 8, 9, 10, 11, 16, 17, 18, 19, 24, 25, 26, 27, 32, 33, 34, 35, 40)
     return sum(pkv[i].numel() * pkv[i].element_size() for i in slots if torch.is_tensor(pkv[i]))
 
 
