@@ -186,48 +186,102 @@ __device__ __forceinline__ void quant_group_normal1(const GroupRef &r, const uin
   *r.z = st.mean_h;
 }
 
+// One quantisation group: lane = channel (K) or (token, channel group) (V) of source block sb -> destination block db.
 template <bool IS_K>
-__global__ __launch_bounds__(128) void cache_migrate_kernel(MigArgs a, int D) {
-  const int u = blockIdx.x;
-  const int64_t bh = blockIdx.y;
+__device__ __forceinline__ void migrate_group(const MigClass &sc, const MigClass &dc, int64_t bh, int64_t sb, int64_t db,
+                                              int lane, int D) {
+  const GroupRef sr = group_ref<IS_K>(sc, bh, sb, lane, D);
+  const GroupRef dr = group_ref<IS_K>(dc, bh, db, lane, D);
+  if (sc.bits != 16 && sc.bits == dc.bits) {  // a survivor of a quantised class keeps its bytes
+    for (int i = 0; i < sc.bits; ++i) dr.words[i] = sr.words[i];
+    *dr.s = *sr.s;
+    *dr.z = *sr.z;
+    return;
+  }
+  uint32_t xp[16];
+  const bool sn = sc.layout == HQEKV_LAYOUT_NORMAL1;
+  switch (sc.bits) {
+    case 16: load_f16(sr, xp); break;
+    case 8: dequant_group<8, false>(sr, xp); break;
+    case 4: dequant_group<4, false>(sr, xp); break;
+    case 2: dequant_group<2, false>(sr, xp); break;
+    default:
+      if (sn) dequant_group<1, true>(sr, xp);
+      else dequant_group<1, false>(sr, xp);
+  }
+  switch (dc.bits) {
+    case 16: store_f16(dr, xp); break;
+    case 8: quant_group<8>(dr, xp); break;
+    case 4: quant_group<4>(dr, xp); break;
+    case 2: quant_group<2>(dr, xp); break;
+    default:
+      if (dc.layout == HQEKV_LAYOUT_NORMAL1) quant_group_normal1(dr, xp);
+      else quant_group<1>(dr, xp);
+  }
+}
+
+__device__ __forceinline__ int dst_class_of(const MigArgs &a, int u) {
   int ci = 0;
 #pragma unroll
   for (int k = 1; k < HQEKV_MAX_SEGS; ++k) ci += (k < a.n_dst && u >= a.dst_begin[k]) ? 1 : 0;
-  const MigClass dc = a.dst[ci];
-  const int64_t db = u - a.dst_begin[ci];  // block inside the destination class
-  const int32_t code = a.plan_src[u];
-  const MigClass sc = a.src[code >> 24];
-  const int64_t sb = code & 0xffffff;
-  if (bh == 0 && threadIdx.x < 32 && dc.idx) dc.idx[db * 32 + threadIdx.x] = (int64_t)a.plan_pos[u] * 32 + threadIdx.x;
-  const int lanes = IS_K ? D : D;  // K: one lane per channel; V: 32 tokens x D/32 groups
-  for (int lane = threadIdx.x; lane < lanes; lane += blockDim.x) {
-    const GroupRef sr = group_ref<IS_K>(sc, bh, sb, lane, D);
-    const GroupRef dr = group_ref<IS_K>(dc, bh, db, lane, D);
-    if (sc.bits != 16 && sc.bits == dc.bits) {  // a survivor of a quantised class keeps its bytes
-      for (int i = 0; i < sc.bits; ++i) dr.words[i] = sr.words[i];
-      *dr.s = *sr.s;
-      *dr.z = *sr.z;
-      continue;
+  return ci;
+}
+
+constexpr int MIG_THREADS = 128;
+constexpr int MIG_KB = 16;  // K side: destination blocks per workgroup
+
+// V side: a workgroup per destination block; its 32 tokens x D/32 groups are one contiguous stretch of every plane.
+// K side: a group is 32 tokens of ONE channel row -- b words of the row -- and a block's groups lie a whole row
+// apart, so a workgroup takes 16 consecutive destination blocks and lets neighbouring lanes take neighbouring
+// blocks of a row: 16 b-word pieces side by side (64 bytes at 1 bit ... 512 at 8), and as long as the blocks come
+// from consecutive places of one source class (survivors of a class stay in order) the reads line up the same
+// way.  (A lane per channel, as on the V side, touched a separate cache line per lane: the K launch took four to
+// six times as long as the V launch for the same bytes.)  Blocks of new tokens arrive token-major, where the
+// channels of a token are what is contiguous: a workgroup that holds any of those walks its blocks one by one
+// with a lane per channel.
+template <bool IS_K>
+__global__ __launch_bounds__(MIG_THREADS) void cache_migrate_kernel(MigArgs a, int D) {
+  const int64_t bh = blockIdx.y;
+  const int total = a.dst_begin[HQEKV_MAX_SEGS];
+  if constexpr (!IS_K) {
+    const int u = blockIdx.x;
+    const MigClass dc = a.dst[dst_class_of(a, u)];
+    const int64_t db = u - a.dst_begin[dst_class_of(a, u)];
+    const int32_t code = a.plan_src[u];
+    if (bh == 0 && threadIdx.x < 32 && dc.idx) dc.idx[db * 32 + threadIdx.x] = (int64_t)a.plan_pos[u] * 32 + threadIdx.x;
+    for (int lane = threadIdx.x; lane < D; lane += MIG_THREADS)
+      migrate_group<false>(a.src[code >> 24], dc, bh, code & 0xffffff, db, lane, D);
+  } else {
+    const int u0 = blockIdx.x * MIG_KB;
+    const int u = u0 + (int)(threadIdx.x % MIG_KB);
+    const bool live = u < total;
+    const int uc = live ? u : u0;   // (u0 < total by the grid size)
+    const int ci = dst_class_of(a, uc);
+    const int64_t db = uc - a.dst_begin[ci];
+    const int32_t code = a.plan_src[uc];
+    const int si = code >> 24;
+    const bool token_major = a.src[si].bits == 16 && a.src[si].layout == HQEKV_LAYOUT_TOKEN_MAJOR;
+    if (bh == 0) {  // positions of the blocks' tokens
+      for (int e = threadIdx.x; e < MIG_KB * 32; e += MIG_THREADS) {
+        const int ue = u0 + e / 32;
+        if (ue < total) {
+          const int ce = dst_class_of(a, ue);
+          int64_t *idx = a.dst[ce].idx;
+          if (idx) idx[(int64_t)(ue - a.dst_begin[ce]) * 32 + e % 32] = (int64_t)a.plan_pos[ue] * 32 + e % 32;
+        }
+      }
     }
-    uint32_t xp[16];
-    const bool sn = sc.layout == HQEKV_LAYOUT_NORMAL1;
-    switch (sc.bits) {
-      case 16: load_f16(sr, xp); break;
-      case 8: dequant_group<8, false>(sr, xp); break;
-      case 4: dequant_group<4, false>(sr, xp); break;
-      case 2: dequant_group<2, false>(sr, xp); break;
-      default:
-        if (sn) dequant_group<1, true>(sr, xp);
-        else dequant_group<1, false>(sr, xp);
-    }
-    switch (dc.bits) {
-      case 16: store_f16(dr, xp); break;
-      case 8: quant_group<8>(dr, xp); break;
-      case 4: quant_group<4>(dr, xp); break;
-      case 2: quant_group<2>(dr, xp); break;
-      default:
-        if (dc.layout == HQEKV_LAYOUT_NORMAL1) quant_group_normal1(dr, xp);
-        else quant_group<1>(dr, xp);
+    if (__syncthreads_or(live && token_major)) {
+      for (int j = 0; j < MIG_KB && u0 + j < total; ++j) {
+        const int cj = dst_class_of(a, u0 + j);
+        const int32_t code_j = a.plan_src[u0 + j];
+        for (int lane = threadIdx.x; lane < D; lane += MIG_THREADS)
+          migrate_group<true>(a.src[code_j >> 24], a.dst[cj], bh, code_j & 0xffffff, u0 + j - a.dst_begin[cj], lane, D);
+      }
+    } else if (live) {
+      const MigClass sc = a.src[si], dc = a.dst[ci];
+      for (int d = threadIdx.x / MIG_KB; d < D; d += MIG_THREADS / MIG_KB)
+        migrate_group<true>(sc, dc, bh, code & 0xffffff, db, d, D);
     }
   }
 }
@@ -285,8 +339,12 @@ extern "C" int hqekv_cache_migrate(int is_k, const hqekv_cache_class *src, int n
   a.n_dst = n_dst;
   a.plan_src = plan;
   a.plan_pos = plan + total;
-  const dim3 grid((unsigned)total, (unsigned)BH), block(128);
-  if (is_k) hipLaunchKernelGGL(cache_migrate_kernel<true>, grid, block, 0, (hipStream_t)stream, a, (int)D);
-  else hipLaunchKernelGGL(cache_migrate_kernel<false>, grid, block, 0, (hipStream_t)stream, a, (int)D);
+  const dim3 block(MIG_THREADS);
+  if (is_k)
+    hipLaunchKernelGGL(cache_migrate_kernel<true>, dim3((unsigned)((total + MIG_KB - 1) / MIG_KB), (unsigned)BH), block, 0,
+                       (hipStream_t)stream, a, (int)D);
+  else
+    hipLaunchKernelGGL(cache_migrate_kernel<false>, dim3((unsigned)total, (unsigned)BH), block, 0, (hipStream_t)stream, a,
+                       (int)D);
   return check_launch("cache_migrate_kernel");
 }
