@@ -139,3 +139,122 @@ def test_gather_engine_declines_selections_that_split_blocks(dev):
     want, _ = O.compress_cache(O.empty_cache(K, V, 128), 128, 0, ragged, counts, counts.clone(), imp)
     for slot in range(42):
         _same(got[slot], want[slot], f"slot {slot}")
+
+
+@pytest.mark.parametrize("is_k", [True, False], ids=["K", "V"])
+@pytest.mark.parametrize("low_normal", [False, True], ids=["uniform1", "normal1"])
+def test_cache_migrate_random_plans(dev, is_k, low_normal):
+    """hqekv_cache_migrate through the C ABI on plans drawn at random: every (source class, destination class)
+    pair with destination bits <= source bits, sources in any order, more blocks than one workgroup's 16 (K side),
+    a last workgroup that is not full, new tokens read from the head of a longer token-major tensor.  Expected
+    bytes from the oracle: a block that keeps its width is copied, any other is dequantised (two roundings) and
+    quantised again; the position arrays are the plan's block numbers expanded to tokens."""
+    from hqekv_amd import _lib
+    B, H, D = 2, 2, 128
+    bits_of = (16, 8, 4, 2, 1)
+    g = torch.Generator().manual_seed(5 + (2 if is_k else 0) + (1 if low_normal else 0))
+    rnd = lambda *s: torch.randn(*s, generator=g).half()
+    n_src = [int(x) for x in torch.randint(6, 20, (5,), generator=g)] + [9]     # blocks per source; last: new tokens
+    tail = 7                                                                      # residual tokens behind the new ones
+    quant = lambda x, b: (O.normal_group_quantize_pack_last_dim(x, 32, 1) if (b == 1 and low_normal)
+                          else O.uniform_group_quantize_pack_last_dim(x, 32, b))
+    dequant = lambda c, s, z, b: (O.normal_group_dequantize_unpack_last_dim(c, s, z, 32, 1) if (b == 1 and low_normal)
+                                  else O.uniform_group_dequantize_unpack_last_dim(c, s, z, 32, b))
+    grp = (lambda x: x.transpose(2, 3).contiguous()) if is_k else (lambda x: x)   # groups along the last dim
+    ungrp = grp if is_k else (lambda x: x)
+    # sources as token-major fp16 values (B,H,n,D) and as stored
+    src_vals, src_store = [], []
+    for si, b in enumerate(bits_of):
+        x = rnd(B, H, n_src[si] * 32, D)
+        if b == 16:
+            src_vals.append(x)
+            src_store.append((grp(x), None, None))
+        else:
+            c, s, z = quant(grp(x), b)
+            src_vals.append(ungrp(dequant(c, s, z, b)))
+            src_store.append((c, s, z))
+    new_full = rnd(B, H, n_src[5] * 32 + tail, D)
+    src_vals.append(new_full[:, :, :n_src[5] * 32])
+    # plan: every source block goes somewhere it may go (or nowhere: evicted), in random order
+    cand = [(si, j) for si in range(6) for j in range(n_src[si])]
+    perm = torch.randperm(len(cand), generator=g).tolist()
+    dest_blocks = {di: [] for di in range(5)}
+    for p in perm:
+        si, j = cand[p]
+        lo = 0 if si == 5 else si                       # new tokens may go anywhere, a class only down or stay
+        di = int(torch.randint(lo, 6, (1,), generator=g))
+        if di < 5:
+            dest_blocks[di].append((si, j))
+    total = sum(len(v) for v in dest_blocks.values())
+    assert total > 16   # more than one workgroup on the K side
+    pos = torch.randperm(total, generator=g).tolist()   # new block numbers, any bijection
+    # expected stores
+    want, plan_src, plan_pos, u = {}, [], [], 0
+    for di, b in enumerate(bits_of):
+        blocks = dest_blocks[di]
+        if not blocks:
+            continue
+        vals = torch.cat([src_vals[si][:, :, 32 * j:32 * j + 32] for si, j in blocks], dim=2)
+        if b == 16:
+            c, s, z = grp(vals), None, None
+        else:
+            c, s, z = quant(grp(vals), b)
+            c, s, z = c.clone(), s.clone(), z.clone()
+            pf = 32 // b
+            for k, (si, j) in enumerate(blocks):        # same width: the stored bytes move
+                if si < 5 and bits_of[si] == b:
+                    sc, ss, sz = src_store[si]
+                    if is_k:
+                        c[..., k * 32 // pf:(k + 1) * 32 // pf] = sc[..., j * 32 // pf:(j + 1) * 32 // pf]
+                        s[..., k], z[..., k] = ss[..., j], sz[..., j]
+                    else:
+                        c[:, :, 32 * k:32 * k + 32] = sc[:, :, 32 * j:32 * j + 32]
+                        s[:, :, 32 * k:32 * k + 32], z[:, :, 32 * k:32 * k + 32] = ss[:, :, 32 * j:32 * j + 32], sz[:, :, 32 * j:32 * j + 32]
+        idx = torch.cat([torch.arange(32) + 32 * pos[u + k] for k in range(len(blocks))]).to(torch.int64)
+        want[b] = (c, s, z, idx)
+        plan_src += [(si << 24) | j for si, j in blocks]
+        plan_pos += pos[u:u + len(blocks)]
+        u += len(blocks)
+    # device side
+    keep = []
+    def up(t):
+        t = t.to(dev).contiguous()
+        keep.append(t)
+        return t
+    src = (_lib.CacheClass * 6)()
+    for si, b in enumerate(bits_of):
+        c, s, z = src_store[si]
+        e = src[si]
+        e.bits, e.n_tokens, e.data = b, n_src[si] * 32, up(c).data_ptr()
+        if b != 16:
+            e.scale, e.zero = up(s).data_ptr(), up(z).data_ptr()
+            e.layout = _lib.LAYOUT_NORMAL1 if (b == 1 and low_normal) else 0
+    newd = up(new_full)
+    e = src[5]
+    e.bits, e.n_tokens, e.slab_tokens, e.data = 16, n_src[5] * 32, new_full.shape[2], newd.data_ptr()
+    e.layout = _lib.LAYOUT_TOKEN_MAJOR if is_k else 0
+    dst = (_lib.CacheClass * 5)()
+    got, n_dst = {}, 0
+    for di, b in enumerate(bits_of):
+        if b not in want:
+            continue
+        c, s, z, idx = want[b]
+        oc = torch.empty_like(c, device=dev)
+        oi = torch.empty_like(idx, device=dev)
+        d = dst[n_dst]
+        n_dst += 1
+        d.bits, d.n_tokens, d.data, d.idx = b, idx.numel(), oc.data_ptr(), oi.data_ptr()
+        os_ = oz = None
+        if b != 16:
+            os_, oz = torch.empty_like(s, device=dev), torch.empty_like(z, device=dev)
+            d.scale, d.zero = os_.data_ptr(), oz.data_ptr()
+            d.layout = _lib.LAYOUT_NORMAL1 if (b == 1 and low_normal) else 0
+        got[b] = (oc, os_, oz, oi)
+    plan = torch.tensor(plan_src + plan_pos, dtype=torch.int32).to(dev)
+    rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src, 6, dst, n_dst, plan.data_ptr(), B * H, D,
+                                         _lib.stream_ptr(torch.device(dev)))
+    _lib.check(rc, "cache_migrate")
+    torch.cuda.synchronize()
+    for b in want:
+        for name, a, w in zip(("code", "scale", "zero", "idx"), got[b], want[b]):
+            _same(a, w, f"{b}-bit class {name}")
