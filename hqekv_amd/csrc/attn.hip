@@ -636,19 +636,29 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
         if (h0 > 0) __syncthreads();
 #pragma unroll
         for (int j = 0; j < RH; ++j) {
-          float4 *dst = reinterpret_cast<float4 *>(red + (wave * RH + j) * QK_TILE + lane * QK_TPL);
-          dst[0] = make_float4(acc[h0 + j][0], acc[h0 + j][1], acc[h0 + j][2], acc[h0 + j][3]);
-          dst[1] = make_float4(acc[h0 + j][4], acc[h0 + j][5], acc[h0 + j][6], acc[h0 + j][7]);
+          // a partial row is parked as two planes -- tokens 0-3 and tokens 4-7 of every lane -- so that the lanes of
+          // a wave write adjacent 16-byte pieces (one plane of [lane][8] would put them 32 bytes apart: two-way
+          // bank conflicts on every 128-bit access)
+          float *row = red + (wave * RH + j) * QK_TILE;
+          *reinterpret_cast<float4 *>(row + lane * 4) = make_float4(acc[h0 + j][0], acc[h0 + j][1], acc[h0 + j][2], acc[h0 + j][3]);
+          *reinterpret_cast<float4 *>(row + QK_TILE / 2 + lane * 4) = make_float4(acc[h0 + j][4], acc[h0 + j][5], acc[h0 + j][6], acc[h0 + j][7]);
         }
         __syncthreads();
         const int h = h0 + hl;
         float a[VPT];
 #pragma unroll
         for (int i = 0; i < VPT; ++i) a[i] = 0.f;
+        constexpr int PIECE = VPT < 4 ? VPT : 4;                 // adjacent tokens that lie together in a plane
+        const int tk = (int)(threadIdx.x * VPT) % QK_TILE;       // first of this thread's tokens inside the tile
 #pragma unroll
         for (int w = 0; w < QK_WAVES; ++w) {
+          const float *row = red + (w * RH + hl) * QK_TILE;
           float part[VPT];
-          __builtin_memcpy(part, red + (w * RH + hl) * QK_TILE + (threadIdx.x * VPT) % QK_TILE, VPT * 4);
+#pragma unroll
+          for (int i0 = 0; i0 < VPT; i0 += PIECE) {
+            const int t = tk + i0;  // token t = 8 * lane + i sits at plane i / 4, [lane][i % 4]
+            __builtin_memcpy(part + i0, row + ((t & 4) ? QK_TILE / 2 : 0) + (t >> 3) * 4 + (t & 3), PIECE * 4);
+          }
 #pragma unroll
           for (int i = 0; i < VPT; ++i) a[i] += part[i];
         }
