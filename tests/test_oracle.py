@@ -418,3 +418,18 @@ def test_gpu_tree_statistics_restatement():
     assert bool(((std.double() - s64).abs() <= step(s64)).all()) and bool(((mean.double() - m64).abs() <= step(m64)).all())
     t_std, t_mean = torch.std_mean(g, dim=-1, keepdim=True)
     assert float((t_std != std).float().mean()) < 0.005 and float((t_mean != mean).float().mean()) < 0.005
+
+
+def test_gpu_tree_statistics_known_answer_next_to_a_rounding_boundary():
+    """A group whose std lies 5e-9 below the midpoint of two fp16 numbers (fp32 std 0.88549799, midpoint
+    0.88549805): ``torch.std_mean`` on the GPU and the HIP quantiser both give 0.88525390625 / 0.09979248046875
+    (recorded from a run on an MI355X).  A square root that is one fp32 unit off -- torch.sqrt on one AVX-512 host
+    was -- lands on the other side; the restatement takes it through float64."""
+    vals = [0.2332763671875, -0.167236328125, -0.96826171875, -0.53662109375, 1.751953125, 1.48046875, -0.126953125,
+            0.1861572265625, -1.0458984375, -1.5888671875, 1.720703125, 0.2330322265625, -1.201171875, 1.0595703125,
+            -0.75244140625, -0.381591796875, 0.8837890625, -0.1619873046875, 0.9853515625, -0.08868408203125,
+            -0.2069091796875, 0.73486328125, 1.580078125, 0.5078125, -0.798828125, 0.023773193359375, -0.2061767578125,
+            -0.11798095703125, 0.1656494140625, -0.93408203125, -0.221435546875, 1.15234375]
+    g = torch.tensor(vals, dtype=torch.float16).reshape(1, 1, 32)
+    std, mean = O.std_mean_gpu_tree(g)
+    assert std.dtype == torch.float16 and float(std) == 0.88525390625 and float(mean) == 0.09979248046875
