@@ -143,16 +143,17 @@ def test_gather_engine_declines_selections_that_split_blocks(dev):
 
 @pytest.mark.parametrize("is_k", [True, False], ids=["K", "V"])
 @pytest.mark.parametrize("low_normal", [False, True], ids=["uniform1", "normal1"])
-def test_cache_migrate_random_plans(dev, is_k, low_normal):
+@pytest.mark.parametrize("D", [128, 64, 256])
+def test_cache_migrate_random_plans(dev, is_k, low_normal, D):
     """hqekv_cache_migrate through the C ABI on plans drawn at random: every (source class, destination class)
     pair with destination bits <= source bits, sources in any order, more blocks than one workgroup's 16 (K side),
     a last workgroup that is not full, new tokens read from the head of a longer token-major tensor.  Expected
     bytes from the oracle: a block that keeps its width is copied, any other is dequantised (two roundings) and
     quantised again; the position arrays are the plan's block numbers expanded to tokens."""
     from hqekv_amd import _lib
-    B, H, D = 2, 2, 128
+    B, H = 2, 2
     bits_of = (16, 8, 4, 2, 1)
-    g = torch.Generator().manual_seed(5 + (2 if is_k else 0) + (1 if low_normal else 0))
+    g = torch.Generator().manual_seed(5 + (2 if is_k else 0) + (1 if low_normal else 0) + D)
     rnd = lambda *s: torch.randn(*s, generator=g).half()
     n_src = [int(x) for x in torch.randint(6, 20, (5,), generator=g)] + [9]     # blocks per source; last: new tokens
     tail = 7                                                                      # residual tokens behind the new ones
