@@ -144,8 +144,24 @@ __device__ __forceinline__ void quant_group(const GroupRef &r, const uint32_t (&
     lo2 = __builtin_elementwise_min(lo2, bits_h2(xp[j]));
     hi2 = __builtin_elementwise_max(hi2, bits_h2(xp[j]));
   }
-  const half_t mn_h = (half_t)__builtin_fminf((float)lo2[0], (float)lo2[1]);
-  const float mn = (float)mn_h, mx = __builtin_fmaxf((float)hi2[0], (float)hi2[1]);
+  half_t mn_h = (half_t)__builtin_fminf((float)lo2[0], (float)lo2[1]);
+  float mn = (float)mn_h, mx = __builtin_fmaxf((float)hi2[0], (float)hi2[1]);
+  // a zero extreme takes the sign of the group's first zero (torch's tie rule); rare, so the wave branches around it
+  if (__builtin_amdgcn_ballot_w64(mn == 0.0f || mx == 0.0f) != 0 && (mn == 0.0f || mx == 0.0f)) {
+    half_t v[32];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const half2_t h = bits_h2(xp[j]);
+      v[2 * j] = h[0];
+      v[2 * j + 1] = h[1];
+    }
+    const half_t z = __builtin_bit_cast(half_t, (unsigned short)first_zero_bits(v));
+    if (mn == 0.0f) {
+      mn_h = z;
+      mn = (float)z;
+    }
+    if (mx == 0.0f) mx = (float)z;
+  }
   const half_t d = (half_t)(mx - mn);
   const half_t sc = (half_t)((float)d * INV_QMAX);
   const float rcp = group_recip((float)sc);

@@ -66,6 +66,21 @@ __device__ __forceinline__ uint32_t horner_pack(const uint32_t *z) {
   return w;
 }
 
+// torch.min / torch.max over a group return the element with the LOWEST INDEX among equal ones (ATen's
+// MinOps / MaxOps break ties by index), which decides the sign of a minimum or maximum that is zero when the group
+// holds both +0 and -0.  The hardware minimum prefers -0 and the maximum +0, so groups whose minimum or maximum is
+// a zero look the sign up: the bit pattern of the first zero among N values in index order, or 1 if there is none.
+template <int N>
+__device__ __forceinline__ uint32_t first_zero_bits(const half_t (&x)[N]) {
+  uint32_t r = 1u;
+#pragma unroll
+  for (int i = N - 1; i >= 0; --i) {
+    const uint32_t b = (uint32_t)__builtin_bit_cast(unsigned short, x[i]);
+    if ((b & 0x7fffu) == 0u) r = b;
+  }
+  return r;
+}
+
 struct Normal1Stats {
   half_t mean_h, std_h;
   float thr;  // std * 2^-25

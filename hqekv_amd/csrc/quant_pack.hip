@@ -51,8 +51,31 @@ __global__ __launch_bounds__(256) void quant_rows_kernel(
   half2_t mm = {(half_t)__builtin_fminf((float)lo2[0], (float)lo2[1]), (half_t)(-__builtin_fmaxf((float)hi2[0], (float)hi2[1]))};
   mm = __builtin_elementwise_min(mm, bits_h2(quad_xor_u<1>(h2_bits(mm))));
   mm = __builtin_elementwise_min(mm, bits_h2(quad_xor_u<2>(h2_bits(mm))));
-  const half_t mn_h = mm[0];
-  const float mn = (float)mn_h, mx = -(float)mm[1];
+  half_t mn_h = mm[0];
+  float mn = (float)mn_h, mx = -(float)mm[1];
+  // A zero extreme takes the sign of the group's first zero (torch's tie rule, see first_zero_bits).  The wave
+  // branches around this as a whole (a scalar branch on the ballot): groups with a zero extreme are rare, and a
+  // predicated copy of the block in every lane's path cost the kernel 5-10 %.
+  const bool zero_extreme = __builtin_fminf(__builtin_fabsf(mn), __builtin_fabsf(mx)) == 0.0f;   // mn == 0 or mx == 0
+  if (__builtin_amdgcn_ballot_w64(zero_extreme) != 0 && zero_extreme) {
+    // (the condition is the same for the four lanes of a group: they hold its minimum and maximum)
+    const half_t mine[8] = {p[0][0], p[0][1], p[1][0], p[1][1], p[2][0], p[2][1], p[3][0], p[3][1]};
+    const uint32_t own = first_zero_bits(mine);
+    const uint32_t x1 = quad_xor_u<1>(own), x2 = quad_xor_u<2>(own), x3 = quad_xor_u<1>(x2);  // lanes sub^1, sub^2, sub^3
+    uint32_t by_lane[4];
+#pragma unroll
+    for (int l = 0; l < 4; ++l) by_lane[l] = (sub == (uint32_t)l) ? own : (sub == (uint32_t)(l ^ 1)) ? x1 : (sub == (uint32_t)(l ^ 2)) ? x2 : x3;
+    uint32_t first = 1u;
+#pragma unroll
+    for (int l = 3; l >= 0; --l)
+      if (by_lane[l] != 1u) first = by_lane[l];
+    const half_t z = __builtin_bit_cast(half_t, (unsigned short)first);   // (a zero extreme implies a zero element)
+    if (mn == 0.0f) {
+      mn_h = z;
+      mn = (float)z;
+    }
+    if (mx == 0.0f) mx = (float)z;
+  }
 
   const half_t d = (half_t)(mx - mn);
   const half_t sc = (half_t)((float)d * INV_QMAX);
@@ -141,6 +164,19 @@ __global__ __launch_bounds__(512) void quant_k_tokenmajor_kernel(
     for (int k = 1; k < 32; ++k) {
       lo2 = __builtin_elementwise_min(lo2, t[k]);
       hi2 = __builtin_elementwise_max(hi2, t[k]);
+    }
+    const bool zero_extreme = (float)lo2[0] == 0.0f || (float)hi2[0] == 0.0f || (float)lo2[1] == 0.0f || (float)hi2[1] == 0.0f;
+    if (__builtin_amdgcn_ballot_w64(zero_extreme) != 0)   // rare: the wave branches around it as a whole
+#pragma unroll
+    for (int ch = 0; ch < 2; ++ch) {
+      if ((float)lo2[ch] == 0.0f || (float)hi2[ch] == 0.0f) {  // a zero extreme takes the sign of the group's first zero
+        half_t col[32];
+#pragma unroll
+        for (int k = 0; k < 32; ++k) col[k] = t[k][ch];
+        const half_t z = __builtin_bit_cast(half_t, (unsigned short)first_zero_bits(col));
+        if ((float)lo2[ch] == 0.0f) lo2[ch] = z;
+        if ((float)hi2[ch] == 0.0f) hi2[ch] = z;
+      }
     }
     half_t sc[2];
     float rcp[2];

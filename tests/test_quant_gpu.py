@@ -297,3 +297,38 @@ def test_wave_reductions_on_integer_data(dev):
     o = out.cpu()
     assert torch.equal(o[:, 0], x.sum(1)) and torch.equal(o[:, 1], x.max(1)[0])
     assert torch.equal(o[:, 2], o[:, 0]) and torch.equal(o[:, 3], o[:, 1])
+
+
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
+@pytest.mark.parametrize("layout", ["rows", "token_major"])
+def test_signed_zero_extremes_follow_torch_tie_rule(dev, bit, layout):
+    """torch.min / torch.max return the lowest-indexed element among equal ones, so a group whose minimum (or
+    maximum) is zero stores the sign of its FIRST zero when it holds both +0 and -0.  Zero point, scale and codes
+    are compared bit for bit, sign bits included, with torch's op chain on the device and with the oracle."""
+    from hqekv_amd import pack_unpack as P
+    g = torch.Generator().manual_seed(40 + bit)
+    x = torch.randn(1, 2, 16, 64, generator=g).abs().half()           # groups of positive values ...
+    nz = torch.tensor(-0.0, dtype=torch.float16)
+    x[0, 0, 0, 3], x[0, 0, 0, 9] = 0.0, nz                            # ... minimum zero: +0 first
+    x[0, 0, 1, 3], x[0, 0, 1, 9] = nz, 0.0                            # -0 first
+    x[0, 0, 2, 31], x[0, 0, 2, 0] = nz, 0.0                           # first and last element of a group
+    x[0, 0, 3, 8], x[0, 0, 3, 7] = 0.0, nz                            # across the lanes that share a group
+    x[0, 1, 0, :32] = -x[0, 1, 0, :32]                                # maximum zero
+    x[0, 1, 0, 5], x[0, 1, 0, 20] = nz, 0.0
+    x[0, 1, 1, 32:] = 0.0                                             # a group of zeros only, mixed signs
+    x[0, 1, 1, 40], x[0, 1, 1, 63] = nz, nz
+    x[0, 1, 2, :32] = nz                                              # all -0
+    x[0, 1, 3, :32] = 0.0
+    x[0, 1, 3, 0] = nz                                                # -0 first, +0 after
+    data = x if layout == "rows" else x.transpose(2, 3).contiguous().transpose(2, 3)
+    code, scale, mn = P.uniform_group_quantize_pack_last_dim(data.to(dev), 32, bit)
+    t = x.to(dev).reshape(2 * 16, 2, 32).clone()
+    t_mn = torch.min(t, dim=-1, keepdim=True)[0]
+    t_mx = torch.max(t, dim=-1, keepdim=True)[0]
+    t_scale = (t_mx - t_mn) / (2 ** bit - 1)
+    bits = lambda a: a.reshape(-1).view(torch.int16)
+    assert torch.equal(bits(mn), bits(t_mn)), "zero point (sign of a zero minimum)"
+    assert torch.equal(bits(scale), bits(t_scale)), "scale (sign of a zero range)"
+    oc, os_, om = O.uniform_group_quantize_pack_last_dim(x, 32, bit)
+    assert torch.equal(code.cpu(), oc)
+    assert torch.equal(bits(scale.cpu()), bits(os_)) and torch.equal(bits(mn.cpu()), bits(om))
