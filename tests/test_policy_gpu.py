@@ -154,7 +154,15 @@ def test_cache_migrate_random_plans(dev, is_k, low_normal, D):
     B, H = 2, 2
     bits_of = (16, 8, 4, 2, 1)
     g = torch.Generator().manual_seed(5 + (2 if is_k else 0) + (1 if low_normal else 0) + D)
-    rnd = lambda *s: torch.randn(*s, generator=g).half()
+    def rnd(*s):   # (B, H, tokens, D) values with a few groups whose minimum is a zero of either sign
+        x = torch.randn(*s, generator=g).half()
+        x[..., :8] = x[..., :8].abs()                       # K groups (32 tokens of a channel) of channels 0-7 ...
+        x[:, :, 3::32, :8] = 0.0                            # ... hold +0 first,
+        x[:, :, 9::32, :8] = -0.0                           # then -0
+        x[:, :, 5::32, :32] = x[:, :, 5::32, :32].abs()     # V groups (32 channels of a token): -0 first
+        x[:, :, 5::32, 2] = -0.0
+        x[:, :, 5::32, 6] = 0.0
+        return x
     n_src = [int(x) for x in torch.randint(6, 20, (5,), generator=g)] + [9]     # blocks per source; last: new tokens
     tail = 7                                                                      # residual tokens behind the new ones
     quant = lambda x, b: (O.normal_group_quantize_pack_last_dim(x, 32, 1) if (b == 1 and low_normal)
