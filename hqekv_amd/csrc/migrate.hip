@@ -118,16 +118,18 @@ __device__ __forceinline__ void dequant_group(const GroupRef &r, uint32_t (&xp)[
   uint32_t w[BITS];
 #pragma unroll
   for (int i = 0; i < BITS; ++i) w[i] = r.words[i];
-  const float s = (float)*r.s, z = (float)*r.z;
+  const half_t s = *r.s, z = *r.z;
+  // fp16 multiply and add, each one rounding of the exact result (through fp32 the compiler's mixed-precision fma
+  // with a +0 addend would lose the sign of a -0 product)
 #pragma unroll
   for (int j = 0; j < 16; ++j) {
     half2_t v;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
       const int k = 2 * j + e;
-      const float c = (float)code_at<BITS>(w[k / PF], k % PF);
-      const half_t m = NORMAL ? (half_t)((c != 0.f ? 0.67431640625f : -0.67431640625f) * s) : (half_t)(c * s);
-      v[e] = (half_t)((float)m + z);
+      const uint32_t ci = code_at<BITS>(w[k / PF], k % PF);
+      const half_t m = NORMAL ? (ci != 0u ? (half_t)0.67431640625f : (half_t)-0.67431640625f) * s : (half_t)(float)ci * s;
+      v[e] = m + z;
     }
     xp[j] = h2_bits(v);
   }

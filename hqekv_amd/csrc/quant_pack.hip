@@ -381,24 +381,27 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(
   const int64_t r = rr % n_rows;
   const int64_t o = rr / n_rows;
   const uint32_t w = code[o * co + r * cr + j];
-  float s = 1.0f, z = 0.0f;
+  half_t s = (half_t)1.0f, z = (half_t)0.0f;
   if (DEQUANT) {
     const int64_t g = (j * PF) / 32;
-    s = (float)scale[o * so + r * sr + g];
-    z = (float)zero[o * so + r * sr + g];
+    s = scale[o * so + r * sr + g];
+    z = zero[o * so + r * sr + g];
   }
+  // Both steps as fp16 operations (each a single rounding of the exact result).  Written through fp32 the
+  // compiler turns the product into a mixed-precision fma with a +0 addend, which loses the sign of a -0
+  // product (code 0 times a negative or -0 scale; the -0.6745 centre times a std of +0).
   half_t vals[PF];
 #pragma unroll
   for (int i = 0; i < PF; ++i) {
-    const float c = (float)code_at<BITS>(w, i);
+    const uint32_t ci = code_at<BITS>(w, i);
     if (NORMAL) {
-      const half_t m = (half_t)((c != 0.f ? 0.67431640625f : -0.67431640625f) * s);
-      vals[i] = (half_t)((float)m + z);
+      const half_t m = (ci != 0u ? (half_t)0.67431640625f : (half_t)-0.67431640625f) * s;
+      vals[i] = m + z;
     } else if (DEQUANT) {
-      const half_t m = (half_t)(c * s);  // exact product, one rounding
-      vals[i] = (half_t)((float)m + z);  // second rounding
+      const half_t m = (half_t)(float)ci * s;  // first rounding (the code itself is exact in fp16)
+      vals[i] = m + z;                         // second rounding
     } else {
-      vals[i] = (half_t)c;
+      vals[i] = (half_t)(float)ci;
     }
   }
   half_t *po = out + o * oo + r * orow + j * PF;

@@ -332,3 +332,34 @@ def test_signed_zero_extremes_follow_torch_tie_rule(dev, bit, layout):
     oc, os_, om = O.uniform_group_quantize_pack_last_dim(x, 32, bit)
     assert torch.equal(code.cpu(), oc)
     assert torch.equal(bits(scale.cpu()), bits(os_)) and torch.equal(bits(mn.cpu()), bits(om))
+
+
+def test_dequant_keeps_the_sign_of_zero_products(dev):
+    """rnd16(c * s) is -0 for code 0 and a negative (or -0) scale, and for the -0.6745 centre times a std of +0;
+    with a zero point of -0 the value then stays -0, as torch's ``mul_`` / ``add_`` chain on the device gives it
+    (a mixed-precision fma with a +0 addend would answer +0).  Arbitrary fp16 bit patterns for scale and zero
+    (infinities, NaNs, denormals) ride along."""
+    from hqekv_amd import pack_unpack as P
+    nz = -0.0
+    scale = torch.tensor([-1.5, nz, 0.0, 2.0, -6e-8, float("inf"), 65504.0, 3e-7], dtype=torch.float16).reshape(1, 1, 1, 8)
+    zero = torch.tensor([nz, nz, nz, nz, nz, 1.0, nz, nz], dtype=torch.float16).reshape(1, 1, 1, 8)
+    g = torch.Generator().manual_seed(3)
+    for bit in (1, 2, 4, 8):
+        code = torch.randint(-2 ** 31, 2 ** 31 - 1, (1, 1, 1, 8 * bit), generator=g, dtype=torch.int64).to(torch.int32)
+        code[..., ::2] = 0                                   # every other word: zero codes
+        out = P.uniform_group_dequantize_unpack_last_dim(code.to(dev), scale.to(dev), zero.to(dev), 32, bit)
+        c = O.unpack_codes(code, bit).to(dev).to(torch.float16).reshape(1, 1, 1, 8, 32)
+        ref = (c * scale.to(dev).unsqueeze(-1) + zero.to(dev).unsqueeze(-1)).reshape(1, 1, 1, 256)
+        nan = torch.isnan(ref)
+        assert torch.equal(torch.isnan(out), nan)
+        assert torch.equal(out[~nan].view(torch.int16), ref[~nan].view(torch.int16)), bit
+        assert bool((out[..., :32 // bit].view(torch.int16) == -32768).all())   # code 0, scale -1.5, zero -0  ->  -0
+    code = torch.tensor([[[[0x0000FFFF] * 8]]], dtype=torch.int32)
+    out = P.normal_group_dequantize_unpack_last_dim(code.to(dev), scale.abs().to(dev), zero.to(dev), 32, 1)
+    c = O.unpack_codes(code, 1).to(dev).reshape(1, 1, 1, 8, 32)
+    k = torch.tensor(O.NORMAL1_CENTER, dtype=torch.float16, device=dev)
+    ref = (torch.where(c > 0, k, -k) * scale.abs().to(dev).unsqueeze(-1) + zero.to(dev).unsqueeze(-1)).reshape(1, 1, 1, 256)
+    nan = torch.isnan(ref)
+    assert torch.equal(torch.isnan(out), nan)
+    assert torch.equal(out[~nan].view(torch.int16), ref[~nan].view(torch.int16))
+    assert bool((out[0, 0, 0, 32 + 16:64].view(torch.int16) == -32768).all())   # std +0, mean -0, code 0  ->  -0
