@@ -19,7 +19,8 @@ from typing import Optional
 
 import torch
 
-from .attention import K_BASE, NEW_K, NEW_V, V_BASE, SegmentMemo, decode_attention
+from . import _lib
+from .attention import K_BASE, NEW_K, NEW_V, V_BASE, SegmentMemo, decode_attention, default_flags
 from .pack_unpack import uniform_group_quantize_pack_last_dim
 
 
@@ -46,6 +47,9 @@ class KiviAttentionLayer:
         self.group_size, self.residual_length = group_size, residual_length
         self.scaling = head_dim ** -0.5
         self._memo = SegmentMemo()
+        self._k_segs = (_lib.Seg * 2)()   # (quantised class, fp16 tail) of each side, rewritten every step
+        self._v_segs = (_lib.Seg * 2)()
+        self._ws: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------ prompt
     def _prefill(self, q, k, v, attention_mask):
@@ -69,6 +73,55 @@ class KiviAttentionLayer:
                                                               self.v_bits)
         return out, (kq, k_full, ks, kz, vq, v_full, vs, vz)
 
+    # ------------------------------------------------------------------ decode attention
+    def _attend(self, q, kq, ks, kz, k_full, vq, vs, vz, v_full, T: int):
+        """The step's attention straight from the tuple's fields: per side the quantised class at positions
+        [0, n) and the fp16 tail behind it -- two table entries whose pointers and lengths are rewritten in place
+        (the class tensors are new objects after every step here, so a memo keyed on them would be rebuilt every
+        time).  Both sides cover every position once by construction, so the softmax rides in the two launches."""
+        B, Hq, _, D = q.shape
+        dev = q.device
+        keep = []
+
+        def fill(segs, code, scale, zero, bits, n_class, tail, layout_tail):
+            n = 0
+            if code is not None:
+                code, scale, zero = code.contiguous(), scale.contiguous(), zero.contiguous()
+                keep.extend((code, scale, zero))
+                e = segs[0]
+                e.bits, e.layout, e.n_tokens, e.pos_base = bits, 0, n_class, 0
+                e.data, e.scale, e.zero, e.idx = code.data_ptr(), scale.data_ptr(), zero.data_ptr(), None
+                n = 1
+            if tail is not None and tail.shape[2] > 0:
+                tail = tail.contiguous()
+                keep.append(tail)
+                e = segs[n]
+                e.bits, e.layout, e.n_tokens, e.pos_base = 16, layout_tail, tail.shape[2], n_class
+                e.data, e.scale, e.zero, e.idx = tail.data_ptr(), None, None, None
+                n += 1
+            return n
+
+        Hkv = (k_full if k_full is not None else kq).shape[1]
+        n_kq = 0 if kq is None else kq.shape[3] * (32 // self.k_bits)
+        n_vq = 0 if vq is None else vq.shape[2]
+        n_k = fill(self._k_segs, kq, ks, kz, self.k_bits, n_kq, k_full, _lib.LAYOUT_TOKEN_MAJOR)
+        n_v = fill(self._v_segs, vq, vs, vz, self.v_bits, n_vq, v_full, 0)
+        qc = q.contiguous()
+        weights = torch.empty(B, Hq, 1, T, dtype=torch.float16, device=dev)
+        out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev)
+        lib = _lib.load()
+        with _lib.on_device(dev):
+            need = lib.hqekv_decode_workspace_bytes(self._k_segs, n_k, self._v_segs, n_v, B, Hq, Hkv, D)
+            if need < 0:
+                raise ValueError("invalid segment table")
+            if self._ws is None or self._ws.numel() * 4 < need or self._ws.device != dev:
+                self._ws = torch.empty(max(need + need // 4, 256) // 4, dtype=torch.float32, device=dev)
+            rc = lib.hqekv_decode_attn(self._k_segs, n_k, self._v_segs, n_v, qc.data_ptr(), None, 0,
+                                       weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, T, self._ws.data_ptr(),
+                                       self._ws.numel() * 4, default_flags(), _lib.stream_ptr(dev))
+        _lib.check(rc, "KiviAttentionLayer")
+        return weights, out
+
     # ------------------------------------------------------------------ one call
     def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
                 attention_mask: Optional[torch.Tensor] = None, past_key_value: Optional[tuple] = None):
@@ -87,18 +140,21 @@ class KiviAttentionLayer:
         k_full = key_states if k_full is None else torch.cat((k_full, key_states), dim=2)
         v_full = value_states if v_full is None else torch.cat((v_full, value_states), dim=2)
 
-        # the quantised class and the fp16 tail of each side as fields of the hybrid tuple: positions
-        # [0, Tq) are the class (no index list: it sits at the head of the row), the tail follows
-        t = [None] * 42
-        if kq is not None:
-            kb = K_BASE[self.k_bits]
-            t[kb], t[kb + 2], t[kb + 3] = kq, ks, kz
-        if vq is not None:
-            vb = V_BASE[self.v_bits]
-            t[vb], t[vb + 2], t[vb + 3] = vq, vs, vz
-        t[NEW_K], t[NEW_V], t[41] = k_full, v_full, kv_seq_len
-        attn_weights, attn_output = decode_attention(query_states, tuple(t), attention_mask, kv_seq_len,
-                                                     zero_init=False, memo=self._memo)
+        if attention_mask is None and query_states.is_cuda and self.head_dim == query_states.shape[-1]:
+            attn_weights, attn_output = self._attend(query_states, kq, ks, kz, k_full, vq, vs, vz, v_full, kv_seq_len)
+        else:
+            # with a mask: the quantised class and the fp16 tail of each side as fields of the hybrid tuple
+            # (positions [0, Tq) are the class -- no index list: it sits at the head of the row --, the tail follows)
+            t = [None] * 42
+            if kq is not None:
+                kb = K_BASE[self.k_bits]
+                t[kb], t[kb + 2], t[kb + 3] = kq, ks, kz
+            if vq is not None:
+                vb = V_BASE[self.v_bits]
+                t[vb], t[vb + 2], t[vb + 3] = vq, vs, vz
+            t[NEW_K], t[NEW_V], t[41] = k_full, v_full, kv_seq_len
+            attn_weights, attn_output = decode_attention(query_states, tuple(t), attention_mask, kv_seq_len,
+                                                         zero_init=False, memo=self._memo)
 
         if k_full.shape[-2] == R:   # a full block of fp16 keys: quantise it per channel, straight from its rows
             c, s, z = uniform_group_quantize_pack_last_dim(k_full.transpose(2, 3), self.group_size, self.k_bits)
