@@ -430,6 +430,8 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="distinct layer caches cycled through")
     ap.add_argument("--qk-tiling", default="auto", choices=["auto", "8waves", "4waves", "wave512", "wave256"],
                     help="force one q.K^T tiling instead of the choice by launch size")
+    ap.add_argument("--dot", default="auto", choices=["auto", "mfma", "valu"],
+                    help="form of the inner products: matrix cores, vector ALU, or the library's default")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--end-to-end", action="store_true",
@@ -473,6 +475,7 @@ def main():
     from hqekv_amd import _lib as _L
     from hqekv_amd.attention import default_flags
     plan_flags = default_flags() | _L.qk_tiling(_L.QK_TILINGS.get(args.qk_tiling, 0))
+    plan_flags |= {"auto": 0, "mfma": _L.DOT_MFMA, "valu": _L.DOT_VALU}[args.dot]
     plans = [DecodePlan(q, cache, flags=plan_flags) for q, cache in layers]
     qs = [q.contiguous() for q, _ in layers]
     cfg = synth.CONFIGS[args.workload]
@@ -560,7 +563,7 @@ def main():
         "config": {"workload": f"{args.workload}: {WORKLOADS[args.workload]}", "B": cfg["B"], "Hq": cfg["Hq"],
                    "Hkv": cfg["Hkv"], "head_dim": cfg["D"], "context": cfg["T"], "kept_tokens": pkv0[41],
                    "layers_cycled": n_layers, "launch": "eager" if graph is None else "hip-graph replay",
-                   "qk_tiling": args.qk_tiling,
+                   "qk_tiling": args.qk_tiling, "dot": args.dot,
                    "softmax": "fused into the two GEMV launches" if fused else "separate launch",
                    "algorithmic_bytes_per_step": alg_bytes},
         "achieved_GBps": round(alg_bytes / (us_per_step * 1e-6) / 1e9, 1),

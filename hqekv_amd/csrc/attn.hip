@@ -10,7 +10,9 @@
 // Codes become fp16 integers without a shift or an int->float convert: a byte permute lines up the
 // same byte of two rows in the two 16-bit halves of a register, one AND-OR drops a code field into
 // the mantissa of 2^(10-pos) (giving 2^(10-pos) + c exactly) and one packed subtract removes the bias.
-// No MFMA and no packed-fp32 instructions are used.
+// With four query heads per KV head the products of those values with the query (or the probabilities) run as
+// 4x4x4 fp16 matrix instructions (same dequantised bits, exact products, fp32 accumulation; HQEKV_DOT_VALU keeps them
+// on the vector ALU).  No packed-fp32 instructions are used.
 //
 // Layouts are consumed exactly as the cache stores them:
 //   K class: code (B,Hkv,D,T/pf) -- a lane owns one packed word (pf tokens) and walks the D rows two
@@ -23,10 +25,15 @@
 #include <stdlib.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "common.h"
 
 #pragma clang fp contract(off)  // the two fp16 roundings of the dequantiser must stay separate
+
+#ifndef HQ_DEFAULT_DOT_MFMA
+#define HQ_DEFAULT_DOT_MFMA true   // the form of the dot products for calls that name neither (see dot_on_matrix_cores)
+#endif
 
 namespace hq {
 
@@ -250,6 +257,75 @@ __device__ __forceinline__ void consume_words(uint32_t w0, uint32_t w1, half2_t 
   consume_byte<BITS, NREP, PF>(byte_pair<3>(w0, w1), s2, z2, a2, acc, 3 * FPB);
 }
 
+// ------------------------------------------------------------------------------- matrix-core form of the dot products
+// With four query heads per KV head the inner product is a 4 x 4 x 4 matrix product per lane group: heads x
+// (four elements of the reduction axis) x (the four lanes' tokens or channels).  v_mfma_f32_4x4x4_16b_f16 runs sixteen
+// such blocks per wave, a block per four consecutive lanes: lane l supplies row l % 4 of its block's A (four fp16) and
+// column l % 4 of its block's B, and receives column l % 4 of D (four fp32).  A holds the query (or the probabilities)
+// of head l % 4, B the lane's own dequantised values -- bit for bit the ones the vector-ALU form feeds to its
+// dot products -- so D is (4 heads) x (this lane's token or channel): one instruction on the matrix pipe in place of
+// eight two-element dot products on the vector ALU.  Products are exact in fp32, accumulation is fp32; only the order
+// of the additions differs from the vector-ALU form.
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f4_t mfma_4x4x4(half2_t a01, half2_t a23, half2_t b01, half2_t b23, f4_t c) {
+  const half4_t a = __builtin_shufflevector(a01, a23, 0, 1, 2, 3);
+  const half4_t b = __builtin_shufflevector(b01, b23, 0, 1, 2, 3);
+  return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 0, 0, 0);
+}
+
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// field I of a byte pair, dequantised with the reference's two roundings
+template <int BITS, int I, bool NORMAL>
+__device__ __forceinline__ half2_t dequant_field(uint32_t u, half2_t s2, half2_t z2) {
+  const half2_t c2 = field_pair<BITS, I>(u);
+  return NORMAL ? dequant_pair_normal1(c2, s2, z2) : dequant_pair(c2, s2, z2);
+}
+// the same with the bias removal folded into the multiply: nb = bias_times_scale<BITS, I>(s2)
+template <int BITS, int I>
+__device__ __forceinline__ half2_t dequant_field_fused_bias(uint32_t u, half2_t s2, half2_t z2, half2_t nb) {
+  const half2_t m2 = __builtin_elementwise_fma(field_pair_biased<BITS, I>(u), s2, nb);
+  return m2 + z2;
+}
+
+// Matrix-core form of consume_byte: byte pair `ua` belongs to elements 0, 1 of the reduction axis (a row pair of K, a
+// token pair of V), `ub` to elements 2, 3; (a01, a23) is the A operand for those four elements.
+template <int BITS, bool NORMAL, int NFIELD, int N>
+__device__ __forceinline__ void consume_bytes_mfma(uint32_t ua, uint32_t ub, half2_t sa, half2_t za, half2_t sb, half2_t zb,
+                                                   half2_t a01, half2_t a23, f4_t (&acc)[N], int tok0) {
+  static_for<NFIELD>([&](auto I_) {
+    constexpr int I = decltype(I_)::value;
+    const half2_t xa = dequant_field<BITS, I, NORMAL>(ua, sa, za);
+    const half2_t xb = dequant_field<BITS, I, NORMAL>(ub, sb, zb);
+    acc[tok0 + I] = mfma_4x4x4(a01, a23, xa, xb, acc[tok0 + I]);
+  });
+}
+template <int BITS, int NFIELD, int N>
+__device__ __forceinline__ void consume_bytes_mfma_fused_bias(uint32_t ua, uint32_t ub, half2_t sa, half2_t za, half2_t sb,
+                                                              half2_t zb, const half2_t (&nba)[8 / BITS],
+                                                              const half2_t (&nbb)[8 / BITS], half2_t a01, half2_t a23,
+                                                              f4_t (&acc)[N], int tok0) {
+  static_for<NFIELD>([&](auto I_) {
+    constexpr int I = decltype(I_)::value;
+    const half2_t xa = dequant_field_fused_bias<BITS, I>(ua, sa, za, nba[I]);
+    const half2_t xb = dequant_field_fused_bias<BITS, I>(ub, sb, zb, nbb[I]);
+    acc[tok0 + I] = mfma_4x4x4(a01, a23, xa, xb, acc[tok0 + I]);
+  });
+}
+__device__ __forceinline__ uint32_t byte_pair_at(uint32_t lo, uint32_t hi, int k) {  // byte_pair<k>, k known after unrolling
+  return k == 0 ? byte_pair<0>(lo, hi) : k == 1 ? byte_pair<1>(lo, hi) : k == 2 ? byte_pair<2>(lo, hi) : byte_pair<3>(lo, hi);
+}
+
 // =============================================================================== q.K^T
 // A tile is worked on by W = 8 waves (small launches: shortest critical path per tile) or W = 4 waves
 // (large launches: more independent workgroups per CU, so one tile's load and reduce phases overlap
@@ -276,10 +352,11 @@ struct QkBlock {
 // with the workgroup barrier), and each later block is requested while the previous one is consumed, so a
 // wave always has one block of loads in flight; the rolled loop keeps the code small enough to stay in the
 // instruction cache from one launch to the next.
-template <int BITS, int NREP, int QK_WAVES, bool NORMAL, typename StageQ>
+template <int BITS, int NREP, int QK_WAVES, bool NORMAL, bool MF, typename StageQ>
 __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int D, int wave,
                                                     StageQ &&stage_q, const half2_t *q2s,
                                                     float (&acc)[NREP][QK_TPL]) {
+  static_assert(!MF || NREP == 4, "the matrix-core form is a 4-head product");
   constexpr int PF = 32 / BITS;
   constexpr int QK_UNR = qk_unr(QK_WAVES);
   using Block = QkBlock<BITS, QK_UNR>;
@@ -314,7 +391,35 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
       r.z1[k] = buf_u16(rz, gofs, grow + gpr * 2u);
     }
   };
-  auto compute = [&](int dp0, const Block &r) {
+  f4_t av[QK_TPL];  // matrix-core form: (4 heads) per token of this lane
+#pragma unroll
+  for (int i = 0; i < QK_TPL; ++i) av[i] = (f4_t){0.f, 0.f, 0.f, 0.f};
+  const int hl = threadIdx.x & 3;  // the head whose query this lane supplies to the matrix product
+  // two row pairs = four channels per matrix product (head_dim is a multiple of 32, so a block's row pairs all exist)
+  auto compute_mf = [&](int dp0, const Block &r) {
+#pragma unroll
+    for (int k = 0; k < QK_UNR; k += 2) {
+      const int dpa = dp0 + QK_WAVES * k, dpb = dpa + QK_WAVES;
+      const half2_t qa = q2s[dpa * NREP + hl], qb = q2s[dpb * NREP + hl];
+      half2_t sa = half_pair<0>(r.s0[k], r.s1[k]), sb = half_pair<0>(r.s0[k + 1], r.s1[k + 1]);
+      const half2_t za = half_pair<0>(r.z0[k], r.z1[k]), zb = half_pair<0>(r.z0[k + 1], r.z1[k + 1]);
+      if (NORMAL) {
+        sa = normal1_spread(sa);
+        sb = normal1_spread(sb);
+      }
+      constexpr int FPB = 8 / BITS;
+      constexpr int NBYTE = BITS;            // bytes that hold a lane's 8 codes of one row
+      constexpr int NF = BITS == 1 ? 8 : FPB;
+#pragma unroll
+      for (int j = 0; j < NBYTE; ++j) {
+        const int sh = BITS <= 2 ? sh2 : 0;
+        const uint32_t ua = byte_pair_at(r.w0[k][j / 4] >> sh, r.w1[k][j / 4] >> sh, j % 4);
+        const uint32_t ub = byte_pair_at(r.w0[k + 1][j / 4] >> sh, r.w1[k + 1][j / 4] >> sh, j % 4);
+        consume_bytes_mfma<BITS, NORMAL, NF, QK_TPL>(ua, ub, sa, za, sb, zb, qa, qb, av, j * FPB);
+      }
+    }
+  };
+  auto compute_valu = [&](int dp0, const Block &r) {
 #pragma unroll
     for (int k = 0; k < QK_UNR; ++k) {
       const int dp = dp0 + QK_WAVES * k;
@@ -349,6 +454,10 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
     }
   };
 
+  auto compute = [&](int dp0, const Block &r) {
+    if constexpr (MF) compute_mf(dp0, r);
+    else compute_valu(dp0, r);
+  };
   // two register blocks in turn: while one is consumed the other one's loads are in flight
   constexpr int STEP = QK_WAVES * QK_UNR;
   Block ba, bb;
@@ -363,13 +472,20 @@ __device__ __forceinline__ void qk_quant_accumulate(const SegDev &sg, uint32_t t
     HQ_LOADS_ABOVE();
     if (dp0 + STEP < DP) compute(dp0 + STEP, bb);
   }
+  if constexpr (MF) {
+#pragma unroll
+    for (int h = 0; h < NREP; ++h)
+#pragma unroll
+      for (int i = 0; i < QK_TPL; ++i) acc[h][i] = av[i][h];
+  }
 }
 
 // fp16 class stored channel-major (B,Hkv,D,T): a lane owns 8 adjacent tokens of each row
-template <int NREP, int QK_WAVES, typename StageQ>
+template <int NREP, int QK_WAVES, bool MF, typename StageQ>
 __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t t0, int bh, int D, int wave,
                                                      StageQ &&stage_q, const half2_t *q2s,
                                                      float (&acc)[NREP][QK_TPL]) {
+  static_assert(!MF || NREP == 4, "the matrix-core form is a 4-head product");
   const uint32_t n = (uint32_t)sg.n_tokens;
   const half_t *kp = (const half_t *)sg.data + (int64_t)bh * D * n;
   const bool vec = (n & 7) == 0 && (((uintptr_t)kp) & 15) == 0 && t0 < n;  // rows stay 16-byte aligned
@@ -399,20 +515,35 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
       load8(kp + (size_t)(d + 1) * n, r.r1[k]);
     }
   };
-  auto compute = [&](int dp0, const Rows &r) {
+  f4_t av[QK_TPL];
 #pragma unroll
-    for (int k = 0; k < UNR; ++k) {
-      const int dp = dp0 + QK_WAVES * k;
-      if (dp >= DP) break;  // uniform
+  for (int i = 0; i < QK_TPL; ++i) av[i] = (f4_t){0.f, 0.f, 0.f, 0.f};
+  const int hl = threadIdx.x & 3;
+  auto compute = [&](int dp0, const Rows &r) {
+    if constexpr (MF) {   // the block's two row pairs = four channels per matrix product
+      static_assert(UNR == 2, "one matrix product per token and block");
+      const int dpa = dp0, dpb = dp0 + QK_WAVES;
+      const half2_t qa = q2s[dpa * NREP + hl], qb = q2s[dpb * NREP + hl];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const half2_t ka = half_pair<0>(r.r0[k][i], r.r1[k][i]);  // token 2i:   (k[d], k[d+1])
-        const half2_t kb = half_pair<1>(r.r0[k][i], r.r1[k][i]);  // token 2i+1
+        av[2 * i] = mfma_4x4x4(qa, qb, half_pair<0>(r.r0[0][i], r.r1[0][i]), half_pair<0>(r.r0[1][i], r.r1[1][i]), av[2 * i]);
+        av[2 * i + 1] = mfma_4x4x4(qa, qb, half_pair<1>(r.r0[0][i], r.r1[0][i]), half_pair<1>(r.r0[1][i], r.r1[1][i]), av[2 * i + 1]);
+      }
+    } else {
 #pragma unroll
-        for (int h = 0; h < NREP; ++h) {
-          const half2_t q2 = q2s[dp * NREP + h];
-          acc[h][2 * i] = __builtin_amdgcn_fdot2(ka, q2, acc[h][2 * i], false);
-          acc[h][2 * i + 1] = __builtin_amdgcn_fdot2(kb, q2, acc[h][2 * i + 1], false);
+      for (int k = 0; k < UNR; ++k) {
+        const int dp = dp0 + QK_WAVES * k;
+        if (dp >= DP) break;  // uniform
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const half2_t ka = half_pair<0>(r.r0[k][i], r.r1[k][i]);  // token 2i:   (k[d], k[d+1])
+          const half2_t kb = half_pair<1>(r.r0[k][i], r.r1[k][i]);  // token 2i+1
+#pragma unroll
+          for (int h = 0; h < NREP; ++h) {
+            const half2_t q2 = q2s[dp * NREP + h];
+            acc[h][2 * i] = __builtin_amdgcn_fdot2(ka, q2, acc[h][2 * i], false);
+            acc[h][2 * i + 1] = __builtin_amdgcn_fdot2(kb, q2, acc[h][2 * i + 1], false);
+          }
         }
       }
     }
@@ -429,6 +560,12 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
     if (dp0 + 2 * STEP < DP) load(dp0 + 2 * STEP, ba);
     HQ_LOADS_ABOVE();
     if (dp0 + STEP < DP) compute(dp0 + STEP, bb);
+  }
+  if constexpr (MF) {
+#pragma unroll
+    for (int h = 0; h < NREP; ++h)
+#pragma unroll
+      for (int i = 0; i < QK_TPL; ++i) acc[h][i] = av[i][h];
   }
 }
 
@@ -549,7 +686,7 @@ struct QkReduce {
 // One workgroup = one tile of one class for one (b, kv head).  The class-specific code is only the
 // accumulation; the cross-wave reduction and the (scattered) store are shared by every class.
 //
-template <int NREP, int QK_WAVES>
+template <int NREP, int QK_WAVES, bool MF = false>
 __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
                                                                half_t *__restrict__ scores, int Hq,
                                                                int Hkv, int D, int64_t Tall, FuseArgs fz, int tpw) {
@@ -713,14 +850,14 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   switch (sg.bits) {
     case 1:
       if (sg.layout == HQEKV_LAYOUT_NORMAL1)
-        run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<1, NREP, QK_WAVES, true>(sg, ts, bh, D, wave, stage_q, q2s, acc); });
+        run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<1, NREP, QK_WAVES, true, MF>(sg, ts, bh, D, wave, stage_q, q2s, acc); });
       else
-        run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<1, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); });
+        run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<1, NREP, QK_WAVES, false, MF>(sg, ts, bh, D, wave, stage_q, q2s, acc); });
       break;
-    case 2: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<2, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
-    case 4: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<4, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
-    case 8: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<8, NREP, QK_WAVES, false>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
-    default: run_tiles([&](uint32_t, uint32_t t0, Acc acc) { qk_f16_cm_accumulate<NREP, QK_WAVES>(sg, t0, bh, D, wave, stage_q, q2s, acc); });
+    case 2: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<2, NREP, QK_WAVES, false, MF>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
+    case 4: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<4, NREP, QK_WAVES, false, MF>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
+    case 8: run_tiles([&](uint32_t ts, uint32_t, Acc acc) { qk_quant_accumulate<8, NREP, QK_WAVES, false, MF>(sg, ts, bh, D, wave, stage_q, q2s, acc); }); break;
+    default: run_tiles([&](uint32_t, uint32_t t0, Acc acc) { qk_f16_cm_accumulate<NREP, QK_WAVES, MF>(sg, t0, bh, D, wave, stage_q, q2s, acc); });
   }
 }
 
@@ -849,16 +986,29 @@ __device__ __forceinline__ bool qw_stage_sz(const SegDev &sg, int tile, int bh, 
   return (big & 0x80008000u) == 0;
 }
 
-template <int BITS, int NREP, int TPL, bool NORMAL, typename Stage>
+// Register blocks per wave (one is consumed, the others are in flight).  Deeper rings and larger blocks were measured
+// on the matrix-core form (rings of 4, blocks of 1-4 KB, 2-4 waves per SIMD): no gain, the launch is not bound by the
+// depth of a wave's load queue.
+__host__ __device__ constexpr int qw_ring_blocks(bool) { return 2; }
+__host__ __device__ constexpr int qw_rows_per_block(int nb, int tpl, bool) {
+  return (nb == 64 || tpl == 4) ? 2 : 4;
+}
+
+// matrix-core form: the query is staged head-major, q2s[h * QW_QH_STRIDE + row pair], so that a lane reads the four (or
+// two) row pairs of a register block for its head, lane % 4, with one LDS access; the stride keeps the four heads' reads
+// in distinct banks and 16-byte aligned
+constexpr int QW_QH_STRIDE = 68;
+
+template <int BITS, int NREP, int TPL, bool NORMAL, bool MF, typename Stage>
 __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t ts, int bh, int lane, Stage &&stage,
                                                     const half2_t *q2s, const uint2 *sz, float (&acc)[NREP][TPL]) {
+  static_assert(!MF || NREP == 4, "the matrix-core form is a 4-head product");
   using G = QwGeom<TPL>;
   using Row = QwRow<BITS, TPL>;
   constexpr int NB = TPL * BITS;                    // bits per lane and row
   // row pairs per register block (two blocks of loads are in flight): short blocks where registers are scarce --
-  // the wide rows of the 8-bit class, and the 256-token tile, whose extra waves hide latency instead
-  constexpr int U = (NB == 64 || TPL == 4) ? 2 : 4;
-  static_assert(G::RP % (2 * U) == 0, "the block loop covers the row pairs exactly");
+  // the wide rows of the 8-bit class, and the 256-token tile, whose extra waves hide latency instead.
+  constexpr int U = qw_rows_per_block(NB, TPL, MF);
   const uint32_t n = (uint32_t)sg.n_tokens;
   const uint32_t rowb = n / 8u * BITS;              // bytes per channel row
   const uint32_t lane_off = ts * BITS / 8u;         // (two lanes share a byte when a lane owns 4 bits)
@@ -876,7 +1026,51 @@ __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t t
       b.r1[k] = qw_load_row<BITS, TPL>(rc, lane_off, row + rowb);
     }
   };
-  auto compute = [&](int i0, const Block &b, auto fused_bias) {
+  f4_t av[TPL];  // matrix-core form: (4 heads) per token of this lane
+#pragma unroll
+  for (int i = 0; i < TPL; ++i) av[i] = (f4_t){0.f, 0.f, 0.f, 0.f};
+  const half2_t *qh = q2s + (lane & 3) * QW_QH_STRIDE;  // the head whose query this lane supplies
+  auto compute_mf = [&](int i0, const Block &b, auto fused_bias) {
+    constexpr bool FB = decltype(fused_bias)::value;
+    constexpr int FPB = 8 / BITS;                 // codes per byte
+    constexpr int NBYTE = (NB + 7) / 8;           // bytes per lane and row
+    constexpr int NF = NB < 8 ? NB / BITS : FPB;  // codes taken from a byte
+    half2_t qa[U];
+#pragma unroll
+    for (int k = 0; k < U; k += 4) {
+      if constexpr (U % 4 == 0) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(qh + i0 + k);
+        qa[k] = as_h2(v.x); qa[k + 1] = as_h2(v.y); qa[k + 2] = as_h2(v.z); qa[k + 3] = as_h2(v.w);
+      } else {
+        const uint2 v = *reinterpret_cast<const uint2 *>(qh + i0 + k);
+        qa[k] = as_h2(v.x); qa[k + 1] = as_h2(v.y);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < U; k += 2) {   // two row pairs = four channels per matrix product
+      const uint2 sza = sp[(i0 + k) * G::NG], szb = sp[(i0 + k + 1) * G::NG];
+      const half2_t sa = as_h2(sza.x), za = as_h2(sza.y), sb = as_h2(szb.x), zb = as_h2(szb.y);
+      half2_t nba[FPB], nbb[FPB];
+      if constexpr (FB) {
+        static_for<NF>([&](auto I_) {
+          constexpr int I = decltype(I_)::value;
+          nba[I] = bias_times_scale<BITS, I>(sa);
+          nbb[I] = bias_times_scale<BITS, I>(sb);
+        });
+      }
+#pragma unroll
+      for (int j = 0; j < NBYTE; ++j) {
+        uint32_t a0 = b.r0[k].w[j / 4], a1 = b.r1[k].w[j / 4], c0 = b.r0[k + 1].w[j / 4], c1 = b.r1[k + 1].w[j / 4];
+        if (NB == 4) {
+          a0 >>= nib; a1 >>= nib; c0 >>= nib; c1 >>= nib;
+        }
+        const uint32_t ua = byte_pair_at(a0, a1, j % 4), ub = byte_pair_at(c0, c1, j % 4);
+        if constexpr (FB) consume_bytes_mfma_fused_bias<BITS, NF, TPL>(ua, ub, sa, za, sb, zb, nba, nbb, qa[k], qa[k + 1], av, j * FPB);
+        else consume_bytes_mfma<BITS, NORMAL, NF, TPL>(ua, ub, sa, za, sb, zb, qa[k], qa[k + 1], av, j * FPB);
+      }
+    }
+  };
+  auto compute_valu = [&](int i0, const Block &b, auto fused_bias) {
     constexpr bool FB = decltype(fused_bias)::value;
 #pragma unroll
     for (int k = 0; k < U; ++k) {
@@ -912,36 +1106,56 @@ __device__ __forceinline__ void qw_quant_accumulate(const SegDev &sg, uint32_t t
       }
     }
   };
-  Block ba, bb;
-  load(0, ba);   // in flight across the staging
+  auto compute = [&](int i0, const Block &b, auto fused_bias) {
+    if constexpr (MF) compute_mf(i0, b, fused_bias);
+    else compute_valu(i0, b, fused_bias);
+  };
+  // A ring of NBLK register blocks: block b is requested NBLK - 1 blocks of arithmetic before it is consumed.
+  constexpr int NBLK = qw_ring_blocks(MF);
+  static_assert(G::RP % (NBLK * U) == 0, "the ring loop covers the row pairs exactly");
+  Block ring[NBLK];
+#pragma unroll
+  for (int j = 0; j < NBLK - 1; ++j) load(j * U, ring[j]);   // in flight across the staging
   // Query and scale/zero into LDS; the staging also says whether every scale of the tile is small enough for the
   // multiply that removes the bias on the way (one packed op fewer per pair of codes).  Worth it where a lane has
   // more codes per row pair than field positions: 8, 4 and 2 bits.
   const bool small_scales = stage();
+  auto finish = [&]() {
+    if constexpr (MF) {
+#pragma unroll
+      for (int h = 0; h < NREP; ++h)
+#pragma unroll
+        for (int i = 0; i < TPL; ++i) acc[h][i] = av[i][h];
+    }
+  };
   auto run = [&](auto fused_bias) {
 #pragma unroll 1
-    for (int i0 = 0; i0 < G::RP; i0 += 2 * U) {
-      load(i0 + U, bb);
-      HQ_LOADS_ABOVE();
-      compute(i0, ba, fused_bias);
-      if (i0 + 2 * U < G::RP) load(i0 + 2 * U, ba);
-      HQ_LOADS_ABOVE();
-      compute(i0 + U, bb, fused_bias);
+    for (int i0 = 0; i0 < G::RP; i0 += NBLK * U) {
+#pragma unroll
+      for (int j = 0; j < NBLK; ++j) {
+        const int nxt = i0 + (j + NBLK - 1) * U;   // the block whose turn it is NBLK - 1 blocks from now
+        if (nxt < G::RP) load(nxt, ring[(j + NBLK - 1) % NBLK]);   // uniform
+        HQ_LOADS_ABOVE();
+        compute(i0 + j * U, ring[j], fused_bias);
+      }
     }
   };
   if constexpr (!NORMAL && BITS != 1) {
     if (__builtin_amdgcn_ballot_w64(!small_scales) == 0) {
       run(std::true_type{});
+      finish();
       return;
     }
   }
   run(std::false_type{});
+  finish();
 }
 
 // fp16 class stored channel-major (B,Hkv,128,T), T a multiple of 8: a lane reads its TPL tokens of a row as 16 or 8 bytes
-template <int NREP, int TPL, typename Stage>
+template <int NREP, int TPL, bool MF, typename Stage>
 __device__ __forceinline__ void qw_f16_accumulate(const SegDev &sg, uint32_t ts, int bh, int lane, Stage &&stage,
                                                   const half2_t *q2s, float (&acc)[NREP][TPL]) {
+  static_assert(!MF || NREP == 4, "the matrix-core form is a 4-head product");
   using G = QwGeom<TPL>;
   constexpr int U = 2, NW = TPL / 2;   // words per lane and row
   const uint32_t n = (uint32_t)sg.n_tokens;
@@ -968,45 +1182,70 @@ __device__ __forceinline__ void qw_f16_accumulate(const SegDev &sg, uint32_t ts,
       load_row(row + rowb, b.r1[k]);
     }
   };
+  f4_t av[TPL];
+#pragma unroll
+  for (int i = 0; i < TPL; ++i) av[i] = (f4_t){0.f, 0.f, 0.f, 0.f};
+  const half2_t *qh = q2s + (lane & 3) * QW_QH_STRIDE;
   auto compute = [&](int i0, const Block &b) {
-#pragma unroll
-    for (int k = 0; k < U; ++k) {
-      half2_t q2[NREP];
-#pragma unroll
-      for (int h = 0; h < NREP; ++h) q2[h] = q2s[(i0 + k) * NREP + h];
+    if constexpr (MF) {   // the block's two row pairs = four channels per matrix product
+      static_assert(U == 2, "one matrix product per token and block");
+      const uint2 qv = *reinterpret_cast<const uint2 *>(qh + i0);
+      const half2_t qa = as_h2(qv.x), qb = as_h2(qv.y);
 #pragma unroll
       for (int i = 0; i < NW; ++i) {
-        const half2_t ka = half_pair<0>(b.r0[k][i], b.r1[k][i]);  // token 2i:   (k[d], k[d+1])
-        const half2_t kb = half_pair<1>(b.r0[k][i], b.r1[k][i]);  // token 2i+1
+        av[2 * i] = mfma_4x4x4(qa, qb, half_pair<0>(b.r0[0][i], b.r1[0][i]), half_pair<0>(b.r0[1][i], b.r1[1][i]), av[2 * i]);
+        av[2 * i + 1] = mfma_4x4x4(qa, qb, half_pair<1>(b.r0[0][i], b.r1[0][i]), half_pair<1>(b.r0[1][i], b.r1[1][i]), av[2 * i + 1]);
+      }
+    } else {
 #pragma unroll
-        for (int h = 0; h < NREP; ++h) {
-          acc[h][2 * i] = __builtin_amdgcn_fdot2(ka, q2[h], acc[h][2 * i], false);
-          acc[h][2 * i + 1] = __builtin_amdgcn_fdot2(kb, q2[h], acc[h][2 * i + 1], false);
+      for (int k = 0; k < U; ++k) {
+        half2_t q2[NREP];
+#pragma unroll
+        for (int h = 0; h < NREP; ++h) q2[h] = q2s[(i0 + k) * NREP + h];
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+          const half2_t ka = half_pair<0>(b.r0[k][i], b.r1[k][i]);  // token 2i:   (k[d], k[d+1])
+          const half2_t kb = half_pair<1>(b.r0[k][i], b.r1[k][i]);  // token 2i+1
+#pragma unroll
+          for (int h = 0; h < NREP; ++h) {
+            acc[h][2 * i] = __builtin_amdgcn_fdot2(ka, q2[h], acc[h][2 * i], false);
+            acc[h][2 * i + 1] = __builtin_amdgcn_fdot2(kb, q2[h], acc[h][2 * i + 1], false);
+          }
         }
       }
     }
   };
-  static_assert(G::RP % (2 * U) == 0, "the block loop covers the row pairs exactly");
-  Block ba, bb;
-  load(0, ba);
+  constexpr int NBLK = qw_ring_blocks(MF);
+  static_assert(G::RP % (NBLK * U) == 0, "the ring loop covers the row pairs exactly");
+  Block ring[NBLK];
+#pragma unroll
+  for (int j = 0; j < NBLK - 1; ++j) load(j * U, ring[j]);
   stage();
 #pragma unroll 1
-  for (int i0 = 0; i0 < G::RP; i0 += 2 * U) {
-    load(i0 + U, bb);
-    HQ_LOADS_ABOVE();
-    compute(i0, ba);
-    if (i0 + 2 * U < G::RP) load(i0 + 2 * U, ba);
-    HQ_LOADS_ABOVE();
-    compute(i0 + U, bb);
+  for (int i0 = 0; i0 < G::RP; i0 += NBLK * U) {
+#pragma unroll
+    for (int j = 0; j < NBLK; ++j) {
+      const int nxt = i0 + (j + NBLK - 1) * U;
+      if (nxt < G::RP) load(nxt, ring[(j + NBLK - 1) % NBLK]);   // uniform
+      HQ_LOADS_ABOVE();
+      compute(i0 + j * U, ring[j]);
+    }
+  }
+  if constexpr (MF) {
+#pragma unroll
+    for (int h = 0; h < NREP; ++h)
+#pragma unroll
+      for (int i = 0; i < TPL; ++i) acc[h][i] = av[i][h];
   }
 }
 
-template <int NREP, int TPL>
+template <int NREP, int TPL, bool MF = false>
 __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wave_kernel(SegTable tb, const half_t *__restrict__ q,
                                                                               half_t *__restrict__ scores, int Hq, int Hkv,
                                                                               int64_t Tall, FuseArgs fz) {
   using G = QwGeom<TPL>;
-  __shared__ half2_t q2s[64 * NREP];                  // [row pair][head]: (q[d], q[d+1])
+  // [row pair][head]: (q[d], q[d+1]); matrix-core form: [head][row pair], QW_QH_STRIDE pairs per head
+  __shared__ __align__(16) half2_t q2s[MF ? NREP * QW_QH_STRIDE : 64 * NREP];
   __shared__ __align__(16) uint2 sz[64 * G::NG];      // [row pair][group]: {(s_d, s_d+1), (z_d, z_d+1)}
   __shared__ float red[2 * NREP];
   const int lane = threadIdx.x;
@@ -1016,13 +1255,22 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
   const int si = seg_of_unit(tb, blockIdx.y);
   const SegDev sg = tb.seg[si];
   const int tile = (int)blockIdx.y - begin_of_seg(tb, si);
+
   const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * 128);
-  auto stage_q = [&]() {
+  auto stage_q_pairs = [&]() {
 #pragma unroll
     for (int h = 0; h < NREP; ++h) q2s[lane * NREP + h] = as_h2(qsrc[h * 64 + lane]);
   };
+  auto stage_q = [&]() {
+    if constexpr (MF) {
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) q2s[h * QW_QH_STRIDE + lane] = as_h2(qsrc[h * 64 + lane]);
+    } else {
+      stage_q_pairs();
+    }
+  };
   if (sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR) {
-    stage_q();
+    stage_q_pairs();
     __syncthreads();
     qk_f16_tm_tile<NREP, 1>(sg, tile, bh, b, hkv, 128, Hq, Tall, 0, lane, q2s, scores, fz, red);
     return;
@@ -1052,14 +1300,14 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
   switch (sg.bits) {
     case 1:
       if (sg.layout == HQEKV_LAYOUT_NORMAL1)
-        qw_quant_accumulate<1, NREP, TPL, true>(sg, ts, bh, lane, [&]() { return stage_quant(T{}); }, q2s, sz, acc);
+        qw_quant_accumulate<1, NREP, TPL, true, MF>(sg, ts, bh, lane, [&]() { return stage_quant(T{}); }, q2s, sz, acc);
       else
-        qw_quant_accumulate<1, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc);
+        qw_quant_accumulate<1, NREP, TPL, false, MF>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc);
       break;
-    case 2: qw_quant_accumulate<2, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
-    case 4: qw_quant_accumulate<4, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
-    case 8: qw_quant_accumulate<8, NREP, TPL, false>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
-    default: qw_f16_accumulate<NREP, TPL>(sg, ts, bh, lane, stage_plain, q2s, acc);
+    case 2: qw_quant_accumulate<2, NREP, TPL, false, MF>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
+    case 4: qw_quant_accumulate<4, NREP, TPL, false, MF>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
+    case 8: qw_quant_accumulate<8, NREP, TPL, false, MF>(sg, ts, bh, lane, [&]() { return stage_quant(F{}); }, q2s, sz, acc); break;
+    default: qw_f16_accumulate<NREP, TPL, MF>(sg, ts, bh, lane, stage_plain, q2s, acc);
   }
 
   // positions of the lane's tokens (they index a row of Tall < 2^31 scores, so the low word of each int64 entry
@@ -1240,6 +1488,9 @@ constexpr int PV_WAVES = 4;
 constexpr int PV_CPL = 8;                        // channels per lane
 constexpr int PV_BLOCK = 512;                    // tokens staged in LDS at a time (256 token pairs)
 constexpr int PV_UNR = 4;                        // word pairs per lane in flight together (steps = 4 / words per token)
+#ifndef HQ_PV_MF_UNR
+#define HQ_PV_MF_UNR 4                           // the same for the matrix-core form
+#endif
 
 // LDS block, pair-interleaved: per token pair {s2, z2} for each of the D/32 groups and p2 for each
 // query head, so one 8-byte and one 4*NREP-byte LDS read feed a whole step of a lane.
@@ -1291,11 +1542,23 @@ __device__ __forceinline__ void pv_fetch(const SegDev &sg, int64_t t0, int nt, i
   }
 }
 
-template <int NREP, int NG, bool QUANT>
+template <int NREP, int NG, bool QUANT, bool ZERO_FILL = false>
 __device__ __forceinline__ void pv_commit(const PvPair<NREP, NG> &pr, half_t *const (&prow)[NREP],
                                           PvStage<NREP, NG> &st, bool fused, const float *sm_ml) {
-  if (!pr.valid) return;
   const int tp = threadIdx.x;
+  if (!pr.valid) {
+    // The matrix-core form runs whole step blocks without looking at the pair count: a pair that does not exist
+    // carries p = 0 and scale = zero = 0, so whatever code words its lanes hold turn into exact zeros.
+    if (ZERO_FILL) {
+#pragma unroll
+      for (int h = 0; h < NREP; ++h) st.p2[tp][h] = pack_h2((half_t)0, (half_t)0);
+      if (QUANT) {
+#pragma unroll
+        for (int g = 0; g < NG; ++g) st.sz[tp][g] = make_uint2(0u, 0u);
+      }
+    }
+    return;
+  }
   half_t va[NREP], vb[NREP];
 #pragma unroll
   for (int h = 0; h < NREP; ++h) {
@@ -1334,16 +1597,20 @@ __device__ __forceinline__ void pv_commit(const PvPair<NREP, NG> &pr, half_t *co
 // word at 2 bits, one word at 4 bits, two words at 8 bits, 16 bytes of fp16), 4 token pairs per wave step, so the reduction over
 // tokens needs only two butterfly steps across lanes.  Code words are requested one step-block ahead of
 // their use, and the staging requests of a block are issued before the previous block is consumed.
-template <int BITS, int NREP, int D, bool NORMAL = false>
+template <int BITS, int NREP, int D, bool NORMAL = false, bool MF = false>
 __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh, int wave, int lane,
                                          half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
                                          float (&acc)[NREP][PV_CPL], bool fused, const float *sm_ml) {
   static_assert(D == 128, "16 lanes x 8 channels cover one token row");
+  static_assert(!MF || NREP == 4, "the matrix-core form is a 4-head product");
   constexpr int NG = D / 32;
   constexpr bool QUANT = BITS != 16;
   constexpr int WPL = BITS == 16 ? 4 : (BITS == 8 ? 2 : 1);  // 32-bit words per lane per token
   constexpr int ROWB = D * BITS / 8;                          // bytes per token row
-  constexpr int UNR = PV_UNR / WPL;                           // wave steps per block: 8 words in flight per lane
+  // wave steps per block: 8 words in flight per lane; the matrix-core form takes two token pairs (steps) per product
+  // and, its arithmetic no longer hiding the memory latency, keeps more words in flight
+  // (fp16 rows fill a lane's registers with one token pair per step: there a product takes one pair and two zeros)
+  constexpr int UNR = MF ? ((HQ_PV_MF_UNR / WPL < 1) ? 1 : HQ_PV_MF_UNR / WPL) : PV_UNR / WPL;
   const int cl = lane & 15, tl = lane >> 4;
   const int g = cl >> 2;
   const int sh2 = (BITS == 2) ? (cl & 1) * 16 : (BITS == 1) ? (cl & 3) * 8 : 0;
@@ -1369,6 +1636,9 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
     }
   };
 
+  f4_t av[PV_CPL];  // matrix-core form: (4 heads) per channel of this lane
+#pragma unroll
+  for (int i = 0; i < PV_CPL; ++i) av[i] = (f4_t){0.f, 0.f, 0.f, 0.f};
   PvPair<NREP, NG> pr;
   Words cur;
   {
@@ -1383,7 +1653,7 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
     const bool more = t0 + PV_BLOCK < c1;
     const int nt_next = more ? (int)min((int64_t)PV_BLOCK, c1 - t0 - PV_BLOCK) : 0;
     __syncthreads();  // previous block fully consumed (and sm_ml published)
-    pv_commit<NREP, NG, QUANT>(pr, prow, st, fused, sm_ml);
+    pv_commit<NREP, NG, QUANT, MF>(pr, prow, st, fused, sm_ml);
     if (more) pv_fetch<NREP, NG, QUANT>(sg, t0 + PV_BLOCK, nt_next, bh, prow, pr);
     __syncthreads();
 #pragma unroll 1
@@ -1392,6 +1662,49 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
       if (s0 + UNR < nsteps) load_steps(t0, nt, s0 + UNR, nxt);
       else if (more) load_steps(t0 + PV_BLOCK, nt_next, 0, nxt);
       HQ_LOADS_ABOVE();
+      if constexpr (MF && UNR == 1) {
+        // one token pair per step block (fp16 rows): the product's other two tokens are zeros
+        static_assert(!(MF && UNR == 1) || BITS == 16, "only fp16 rows have single-pair step blocks");
+        const int tpa = 4 * (s0 * PV_WAVES + wave) + tl;
+        const half2_t pa = st.p2[tpa][lane & 3], zero2 = (half2_t){(_Float16)0, (_Float16)0};
+#pragma unroll
+        for (int j = 0; j < (BITS == 16 ? 4 : 0); ++j) {
+          av[2 * j] = mfma_4x4x4(pa, zero2, half_pair<0>(cur.w0[0][j], cur.w1[0][j]), zero2, av[2 * j]);
+          av[2 * j + 1] = mfma_4x4x4(pa, zero2, half_pair<1>(cur.w0[0][j], cur.w1[0][j]), zero2, av[2 * j + 1]);
+        }
+      } else if constexpr (MF) {
+        // two token pairs = four tokens per matrix product; pairs past the end of the block were staged as zeros
+#pragma unroll
+        for (int k = 0; k + 1 < UNR; k += 2) {
+          const int tpa = 4 * ((s0 + k) * PV_WAVES + wave) + tl, tpb = tpa + 4 * PV_WAVES;
+          const half2_t pa = st.p2[tpa][lane & 3], pb = st.p2[tpb][lane & 3];
+          if constexpr (BITS == 16) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              av[2 * j] = mfma_4x4x4(pa, pb, half_pair<0>(cur.w0[k][j], cur.w1[k][j]),
+                                     half_pair<0>(cur.w0[k + 1][j], cur.w1[k + 1][j]), av[2 * j]);
+              av[2 * j + 1] = mfma_4x4x4(pa, pb, half_pair<1>(cur.w0[k][j], cur.w1[k][j]),
+                                         half_pair<1>(cur.w0[k + 1][j], cur.w1[k + 1][j]), av[2 * j + 1]);
+            }
+          } else {
+            const uint2 sza = st.sz[tpa][g], szb = st.sz[tpb][g];
+            half2_t sa = as_h2(sza.x), sb = as_h2(szb.x);
+            const half2_t za = as_h2(sza.y), zb = as_h2(szb.y);
+            if (NORMAL) {
+              sa = normal1_spread(sa);
+              sb = normal1_spread(sb);
+            }
+            constexpr int FPB = 8 / BITS;
+            constexpr int NBYTE = BITS;   // bytes that hold a lane's 8 channels of one token
+#pragma unroll
+            for (int j = 0; j < NBYTE; ++j) {
+              const uint32_t ua = byte_pair_at(cur.w0[k][j / 4] >> sh2, cur.w1[k][j / 4] >> sh2, j % 4);
+              const uint32_t ub = byte_pair_at(cur.w0[k + 1][j / 4] >> sh2, cur.w1[k + 1][j / 4] >> sh2, j % 4);
+              consume_bytes_mfma<BITS, NORMAL, FPB, PV_CPL>(ua, ub, sa, za, sb, zb, pa, pb, av, j * FPB);
+            }
+          }
+        }
+      } else {
 #pragma unroll
       for (int k = 0; k < UNR; ++k) {
         const int tp = 4 * ((s0 + k) * PV_WAVES + wave) + tl;
@@ -1440,13 +1753,23 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
           }
         }
       }
+      }
       cur = nxt;
     }
   }
+  if constexpr (MF) {
+#pragma unroll
+    for (int h = 0; h < NREP; ++h)
+#pragma unroll
+      for (int i = 0; i < PV_CPL; ++i) acc[h][i] = av[i][h];
+  }
 }
 
-template <int NREP, int D>
-__global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half_t *__restrict__ p,
+#ifndef HQ_PV_MF_WAVES
+#define HQ_PV_MF_WAVES 4   // waves per SIMD the matrix-core form is held to (its accumulators live in the AGPR half of the file)
+#endif
+template <int NREP, int D, bool MF = false>
+__global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid_kernel(SegTable tb, half_t *__restrict__ p,
                                                                float *__restrict__ partial, int Hq, int Hkv,
                                                                int64_t Tall, int64_t chunk_tokens,
                                                                int64_t n_bhq, FuseArgs fz) {
@@ -1491,13 +1814,13 @@ __global__ __launch_bounds__(PV_THREADS) void pv_hybrid_kernel(SegTable tb, half
     for (int i = 0; i < PV_CPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {  // (the first barrier inside pv_chunk also publishes sm_ml)
     case 1:
-      if (sg.layout == HQEKV_LAYOUT_NORMAL1) pv_chunk<1, NREP, D, true>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
-      else pv_chunk<1, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
+      if (sg.layout == HQEKV_LAYOUT_NORMAL1) pv_chunk<1, NREP, D, true, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
+      else pv_chunk<1, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
       break;
-    case 2: pv_chunk<2, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
-    case 4: pv_chunk<4, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
-    case 8: pv_chunk<8, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
-    default: pv_chunk<16, NREP, D>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
+    case 2: pv_chunk<2, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
+    case 4: pv_chunk<4, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
+    case 8: pv_chunk<8, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
+    default: pv_chunk<16, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
   }
   // Lanes 16, 32 and 48 apart hold the same channels of other tokens.  Their sum is needed in lanes 0-15
   // only: two lane-row swaps on the vector ALU per value (a swap exchanges rows of 16 lanes between two
@@ -1746,21 +2069,32 @@ static int resolve_qk_tiling(int forced, const hqekv_seg *segs, int nseg, int64_
   return HQEKV_OK;
 }
 
+// Which form of the dot products a call uses: the matrix-core one exists for four query heads per KV head.
+static bool dot_on_matrix_cores(int flags, int64_t nrep) {
+  if (nrep != 4 || (flags & HQEKV_DOT_VALU)) return false;
+  if (flags & HQEKV_DOT_MFMA) return true;
+  return HQ_DEFAULT_DOT_MFMA;
+}
+
 static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
-                     int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling) {
+                     int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf) {
   if (tb.total_units == 0) return HQEKV_OK;
   const int nrep = (int)(Hq / Hkv);
   dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units);
   if (tiling >= 3) {
-#define LAUNCH(N_, TPL_)                                                                                        \
-  hipLaunchKernelGGL((qk_wave_kernel<N_, TPL_>), grid, dim3(64), 0, st, tb, (const half_t *)q, (half_t *)scores, \
+#define LAUNCH(N_, TPL_, MF_)                                                                                        \
+  hipLaunchKernelGGL((qk_wave_kernel<N_, TPL_, MF_>), grid, dim3(64), 0, st, tb, (const half_t *)q, (half_t *)scores, \
                      (int)Hq, (int)Hkv, Tall, fz)
 #define LAUNCH_DS(N_) \
-  if (tiling == 3) LAUNCH(N_, 8); else LAUNCH(N_, 4)
+  if (tiling == 3) LAUNCH(N_, 8, false); else LAUNCH(N_, 4, false)
     switch (nrep) {
       case 1: LAUNCH_DS(1); break;
       case 2: LAUNCH_DS(2); break;
-      case 4: LAUNCH_DS(4); break;
+      case 4:
+        if (!mf) LAUNCH_DS(4);
+        else if (tiling == 3) LAUNCH(4, 8, true);
+        else LAUNCH(4, 4, true);
+        break;
       default: LAUNCH_DS(8);
     }
 #undef LAUNCH_DS
@@ -1772,15 +2106,19 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
   dim3 block((unsigned)waves * 64);
   const int rh = waves == 4 ? (nrep < 4 ? nrep : 4) : (nrep < 2 ? nrep : 2);  // QkReduce::RH
   const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
-#define LAUNCH(N_, W_)                                                                                        \
-  hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
+#define LAUNCH(N_, W_, MF_)                                                                                        \
+  hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_, MF_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
                      (int)Hq, (int)Hkv, (int)D, Tall, fz, tpw)
 #define LAUNCH_W(N_) \
-  if (waves == 8) LAUNCH(N_, 8); else LAUNCH(N_, 4)
+  if (waves == 8) LAUNCH(N_, 8, false); else LAUNCH(N_, 4, false)
   switch (nrep) {
     case 1: LAUNCH_W(1); break;
     case 2: LAUNCH_W(2); break;
-    case 4: LAUNCH_W(4); break;
+    case 4:
+      if (!mf) LAUNCH_W(4);
+      else if (waves == 8) LAUNCH(4, 8, true);
+      else LAUNCH(4, 4, true);
+      break;
     default: LAUNCH_W(8);
   }
 #undef LAUNCH_W
@@ -1790,7 +2128,10 @@ static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B,
 
 // chunk length for the p.V split-K: aim for a few workgroups per CU, never below 64 tokens
 static int64_t pv_chunk_tokens(int64_t total_tokens, int64_t BHkv) {
-  const int64_t target_wgs = 256 * 4;
+  // Chunks hold equal token counts, so their byte counts differ by class (an fp16 row is eight 2-bit rows): a long
+  // launch evens that out over two resident rounds of shorter chunks (B=8 at 64k context: 108 -> 101 us), a short
+  // one keeps one round.
+  const int64_t target_wgs = total_tokens * BHkv >= CB_FOLD_MIN_TOKEN_ROWS ? 256 * 8 : 256 * 4;
   int64_t chunks_per_bh = (target_wgs + BHkv - 1) / BHkv;
   if (chunks_per_bh < 1) chunks_per_bh = 1;
   int64_t c = (total_tokens + chunks_per_bh - 1) / chunks_per_bh;
@@ -1808,19 +2149,22 @@ static int64_t seg_total_tokens(const hqekv_seg *segs, int nseg) {
 
 static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, float *partial, int64_t B,
                      int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st,
-                     int stages = 3) {
+                     bool mf, int stages = 3) {
   const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
   if (tb.total_units > 0 && (stages & 1)) {
     dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units), block(PV_THREADS);
-#define LAUNCH(N_, D_)                                                                                   \
-  hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
+#define LAUNCH(N_, D_, MF_)                                                                                   \
+  hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_, MF_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
                      (int)Hkv, Tall, chunk, n_bhq, fz)
-#define LAUNCH_D(N_) LAUNCH(N_, 128)
+#define LAUNCH_D(N_) LAUNCH(N_, 128, false)
     switch (nrep) {
       case 1: LAUNCH_D(1); break;
       case 2: LAUNCH_D(2); break;
-      case 4: LAUNCH_D(4); break;
+      case 4:
+        if (mf) LAUNCH(4, 128, true);
+        else LAUNCH_D(4);
+        break;
       default: LAUNCH_D(8);
     }
 #undef LAUNCH_D
@@ -1850,7 +2194,8 @@ extern "C" int hqekv_qk_hybrid(const hqekv_seg *segs, int nseg, const void *q, v
   SegTable tb{};
   rc = build_table(segs, nseg, true, D, qk_tile_of(tiling), Tall, &tb, "qk_hybrid");
   if (rc) return rc;
-  return launch_qk(tb, q, scores, B, Hq, Hkv, D, Tall, FuseArgs{}, (hipStream_t)stream, tiling);
+  return launch_qk(tb, q, scores, B, Hq, Hkv, D, Tall, FuseArgs{}, (hipStream_t)stream, tiling,
+                   dot_on_matrix_cores(0, Hq / Hkv));
 }
 
 extern "C" int hqekv_scale_softmax(void *scores, const void *mask, int64_t mask_row_stride, int64_t n_rows,
@@ -1902,7 +2247,7 @@ extern "C" int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, v
                 (long long)need);
   if ((uintptr_t)workspace & 15) return fail(HQEKV_E_ALIGN, "pv_hybrid: workspace not 16-byte aligned");
   return launch_pv(tb, chunk, const_cast<void *>(p), out, (float *)workspace, B, Hq, Hkv, D, Tall, FuseArgs{},
-                   (hipStream_t)stream);
+                   (hipStream_t)stream, dot_on_matrix_cores(0, Hq / Hkv));
 }
 
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -1993,10 +2338,15 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
     fz.arrive = (uint32_t *)(ws + L.arrive_off);
     fz.out = (half_t *)attn_out;
   }
+  if ((flags & HQEKV_DOT_MFMA) && (flags & HQEKV_DOT_VALU))
+    return fail(HQEKV_E_ARG, "decode_attn: HQEKV_DOT_MFMA and HQEKV_DOT_VALU exclude each other");
+  if ((flags & HQEKV_DOT_MFMA) && Hq / Hkv != 4)
+    return fail(HQEKV_E_UNSUPPORTED, "decode_attn: the matrix-core dot products need Hq/Hkv == 4 (got %lld)", (long long)(Hq / Hkv));
+  const bool mf = dot_on_matrix_cores(flags, Hq / Hkv);
   const int only = flags & (HQEKV_ONLY_QK | HQEKV_ONLY_PV | HQEKV_ONLY_COMBINE);
   const bool only_qk = only == HQEKV_ONLY_QK;
   if (only == 0 || only_qk) {
-    rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st, tiling);
+    rc = launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, fz, st, tiling, mf);
     if (rc) return rc;
     if (!fuse) {
       rc = hqekv_scale_softmax(attn_weights, mask, mask_row_stride, B * Hq, Tall, 1.0f / (float)sqrt((double)D), stream);
@@ -2005,7 +2355,7 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
   }
   if (only_qk) return HQEKV_OK;
   const int stages = only == HQEKV_ONLY_PV ? 1 : (only == HQEKV_ONLY_COMBINE ? 2 : 3);
-  return launch_pv(vt, L.chunk, attn_weights, attn_out, (float *)ws, B, Hq, Hkv, D, Tall, fz, st, stages);
+  return launch_pv(vt, L.chunk, attn_weights, attn_out, (float *)ws, B, Hq, Hkv, D, Tall, fz, st, mf, stages);
 }
 
 // ------------------------------------------------------------------ per-class GEMV on the same kernels

@@ -248,6 +248,14 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
 #define HQEKV_ONLY_QK 0x100
 #define HQEKV_ONLY_PV 0x200
 #define HQEKV_ONLY_COMBINE 0x400
+/* Form of the inner products of both GEMV launches.  With four query heads per KV head (Hq/Hkv == 4) the products of
+ * the dequantised values with the query (or with the probabilities) can run on the matrix cores: one 4x4x4 fp16 matrix
+ * instruction per four elements of the reduction axis and lane, in place of eight two-element dot products on the
+ * vector ALU.  The dequantised values are the same bits either way, products are exact and accumulation is fp32 in
+ * both; only the order of the additions differs.  Neither flag: the library's default for the shape.
+ * HQEKV_DOT_MFMA with another head ratio returns HQEKV_E_UNSUPPORTED. */
+#define HQEKV_DOT_MFMA 0x800
+#define HQEKV_DOT_VALU 0x1000
 int64_t hqekv_decode_workspace_bytes(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
                                      int64_t B, int64_t Hq, int64_t Hkv, int64_t D);
 int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
