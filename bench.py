@@ -421,6 +421,152 @@ def bench_end_to_end(args):
     print(json.dumps(out))
 
 
+def measure_decode(workload: str, n_layers: int, K: int, W: int, args, dev):
+    """Build ``n_layers`` distinct layer caches of ``workload`` and time the decode-attention layer-step on them.
+
+    W untimed warm-up steps, then timed regions of EXACTLY K steps each (a barrier-free single process: synchronise on
+    both sides), five of them; the figure is the median region.  Step i works on layer cache i mod n_layers, and the
+    first timed step follows the last warm-up step's layer, so a timed step never finds its cache warm from the
+    warm-up; between two regions a 512 MiB buffer is rewritten (untimed), which also empties the 256 MB memory-side
+    cache.  Launches are replayed from HIP graphs (one of a whole cycle over the layers, one of the K mod n_layers
+    steps that remain) unless --no-graph."""
+    from hqekv_amd import _lib, synth
+    from hqekv_amd.attention import DecodePlan, default_flags
+    layers = build_layers(workload, n_layers, dev)
+    plan_flags = default_flags() | _lib.qk_tiling(_lib.QK_TILINGS.get(args.qk_tiling, 0))
+    plan_flags |= {"auto": 0, "mfma": _lib.DOT_MFMA, "valu": _lib.DOT_VALU}[args.dot]
+    plans = [DecodePlan(q, cache, flags=plan_flags) for q, cache in layers]
+    qs = [q.contiguous() for q, _ in layers]
+    cfg = synth.CONFIGS[workload]
+    pkv0 = layers[0][1]
+    alg_bytes = synth.algorithmic_bytes(pkv0, cfg["Hq"])
+    k_bytes, v_bytes = side_bytes(pkv0, True), side_bytes(pkv0, False)
+    sync = torch.cuda.synchronize
+
+    def step(i):
+        plans[i % n_layers].run(qs[i % n_layers])
+
+    for i in range(W):
+        step(i)
+    sync()
+    first = W % n_layers                    # the timed steps start where the warm-up stopped
+    rounds, rem = divmod(K, n_layers)
+
+    def graph_of(lo, n):
+        if n == 0:
+            return None
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(lo, lo + n):
+                step(i)
+        return g
+
+    use_graph = not args.no_graph
+    g_cycle = graph_of(first, n_layers) if use_graph and rounds else None
+    g_rest = graph_of(first, rem) if use_graph and rem else None
+    if use_graph:
+        for g in (g_cycle, g_rest):
+            if g is not None:
+                g.replay()
+        sync()
+
+    def timed():
+        if use_graph:
+            for _ in range(rounds):
+                g_cycle.replay()
+            if g_rest is not None:
+                g_rest.replay()
+        else:
+            for i in range(first, first + K):
+                step(i)
+
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    regions, regions_host = [], []
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(5):
+        # the rewrite of the flush buffer is queued right ahead of the timed steps, so they start on a busy GPU with
+        # cold caches -- what a decode loop sees between two layers -- and not on one that has gone idle in a wait
+        sync()
+        flush.fill_(1)
+        e0.record()
+        timed()
+        e1.record()
+        sync()
+        regions.append(e0.elapsed_time(e1) * 1e3 / K)
+    for _ in range(5):   # the same K steps on the host's clock, synchronised on both sides
+        regions_host.append(time_region(timed, sync) / K * 1e6)
+    del flush
+    # the figure is the GPU's time for the K steps (HIP events on the launch stream around exactly those steps);
+    # the host's clock around a synchronised region adds the launch and wake-up latency of one graph replay, which
+    # K = 20 steps do not amortise
+    us_per_step = statistics.median(regions)
+    us_per_step_host = statistics.median(regions_host)
+
+    # per-kernel averages (HIP events on the launch stream), one kind of kernel back-to-back over all layers;
+    # replayed from a HIP graph (unless --no-graph) so that the host's launch rate does not show in the
+    # figure of a short kernel
+    reps = 5
+    fused = bool(plans[0].flags & _lib.FUSE_SOFTMAX)
+
+    def part_us(launch_all, n=n_layers):
+        if args.no_graph:
+            return event_avg_us(launch_all, n, reps)
+        launch_all()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            launch_all()
+        return event_avg_us(g.replay, n, reps)
+
+    qk_us = part_us(lambda: [p.run(q, only=_lib.ONLY_QK) for p, q in zip(plans, qs)])
+    sm_us = 0.0
+    if not fused:  # the general path has a softmax launch of its own; time it and take it out of the q.K^T figure
+        sm_us = part_us(lambda: [p.run_softmax() for p in plans])
+        qk_us -= sm_us
+    pv_us = part_us(lambda: [p.run(q, only=_lib.ONLY_PV) for p, q in zip(plans, qs)])
+    cb_us = part_us(lambda: [p.run(q, only=_lib.ONLY_COMBINE) for p, q in zip(plans, qs)])
+    for p, q in zip(plans, qs):  # leave consistent outputs behind
+        p.run(q)
+    dominant = "qk_hybrid_kernel" if qk_us >= pv_us else "pv_hybrid_kernel"
+    dom_us, dom_bytes = (qk_us, k_bytes) if qk_us >= pv_us else (pv_us, v_bytes)
+    achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+
+    # the yardstick: a launch that only reads as many bytes as the dominant kernel must, from buffers as distinct as
+    # the layer caches (1024 workgroups of 256 threads, 16-byte loads, eight in flight per lane), timed the same way
+    lib = _lib.load()
+    nb = (dom_bytes + 15) // 16 * 16
+    bufs = [torch.empty(nb, dtype=torch.uint8, device=dev).fill_(i + 1) for i in range(n_layers)]
+    sums = torch.zeros(1024, dtype=torch.int32, device=dev)
+
+    def read_all():
+        st = _lib.stream_ptr(dev)   # torch's current stream: the capture stream while a graph is recorded
+        for b in bufs:
+            _lib.check(lib.hqekv_selftest_stream_read(b.data_ptr(), nb, sums.data_ptr(), 1024, st), "stream_read")
+
+    floor_us = part_us(read_all)
+    del bufs
+    traffic, traffic_source = recorded_traffic(workload, dominant)
+    return dict(
+        us_per_step=us_per_step, us_per_step_host=us_per_step_host, regions=[round(r, 3) for r in regions],
+        alg_bytes=alg_bytes, cfg=cfg, layers=layers,
+        plans=plans, qs=qs,
+        config={"workload": f"{workload}: {WORKLOADS[workload]}", "B": cfg["B"], "Hq": cfg["Hq"],
+                "Hkv": cfg["Hkv"], "head_dim": cfg["D"], "context": cfg["T"], "kept_tokens": pkv0[41],
+                "layers_cycled": n_layers, "launch": "hip-graph replay" if use_graph else "eager",
+                "timing": "median of 5 regions of `steps` steps, HIP events around the steps; 512 MiB rewritten "
+                          "on the stream right before each region",
+                "qk_tiling": args.qk_tiling, "dot": args.dot,
+                "softmax": "fused into the two GEMV launches" if fused else "separate launch",
+                "algorithmic_bytes_per_step": alg_bytes},
+        kernels_us={"qk_hybrid_kernel": round(qk_us, 3), "scale_softmax_kernel": round(sm_us, 3),
+                    "pv_hybrid_kernel": round(pv_us, 3), "pv_combine_kernel": round(cb_us, 3)},
+        roofline={"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                  "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                  "traffic_source": traffic_source, "bytes_per_launch": dom_bytes, "avg_us": round(dom_us, 3),
+                  "launch_floor_us": round(floor_us, 3),
+                  "launch_floor": "a launch that only reads bytes_per_launch bytes (hqekv_selftest_stream_read), same timing"})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -434,6 +580,8 @@ def main():
                     help="form of the inner products: matrix cores, vector ALU, or the library's default")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="workload c2 only: skip the short configuration-4 measurement printed under 'extra'")
     ap.add_argument("--end-to-end", action="store_true",
                     help="workload c5 only: prompt pass + greedy decode of a random-init Llama-3.1-8B (takes minutes)")
     ap.add_argument("--prompt-len", type=int, default=131072)
@@ -471,109 +619,45 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     n_layers = args.layers or {"c1": 64, "c2": 32, "c4": 4, "c5": 32}[args.workload]
-    layers = build_layers(args.workload, n_layers, dev)
-    from hqekv_amd import _lib as _L
-    from hqekv_amd.attention import default_flags
-    plan_flags = default_flags() | _L.qk_tiling(_L.QK_TILINGS.get(args.qk_tiling, 0))
-    plan_flags |= {"auto": 0, "mfma": _L.DOT_MFMA, "valu": _L.DOT_VALU}[args.dot]
-    plans = [DecodePlan(q, cache, flags=plan_flags) for q, cache in layers]
-    qs = [q.contiguous() for q, _ in layers]
-    cfg = synth.CONFIGS[args.workload]
-    pkv0 = layers[0][1]
-    alg_bytes = synth.algorithmic_bytes(pkv0, cfg["Hq"])
-    k_bytes, v_bytes = side_bytes(pkv0, True), side_bytes(pkv0, False)
-
-    def step(i):
-        plans[i % n_layers].run(qs[i % n_layers])
-
-    sync = torch.cuda.synchronize
-    for i in range(args.warmup):
-        step(i)
-    sync()
-
-    K = args.steps
-    rounds, rem = divmod(K, n_layers)
-    graph = None
-    if not args.no_graph and rounds > 0:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            for i in range(n_layers):
-                step(i)
-        graph.replay()
-        sync()
-
-    def timed():
-        if graph is not None:
-            for _ in range(rounds):
-                graph.replay()
-            for i in range(rem):
-                step(i)
-        else:
-            for i in range(K):
-                step(i)
-
-    elapsed = time_region(timed, sync)
-    us_per_step = elapsed / K * 1e6
-
-    # per-kernel averages (HIP events on the launch stream), one kind of kernel back-to-back over all layers;
-    # replayed from a HIP graph (unless --no-graph) so that the host's launch rate does not show in the
-    # figure of a short kernel
-    from hqekv_amd import _lib
-    reps = 5
-    fused = bool(plans[0].flags & _lib.FUSE_SOFTMAX)
-
-    def part_us(launch_all):
-        if args.no_graph:
-            return event_avg_us(launch_all, n_layers, reps)
-        launch_all()
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            launch_all()
-        return event_avg_us(g.replay, n_layers, reps)
-
-    qk_us = part_us(lambda: [p.run(q, only=_lib.ONLY_QK) for p, q in zip(plans, qs)])
-    sm_us = 0.0
-    if not fused:  # the general path has a softmax launch of its own; time it and take it out of the q.K^T figure
-        sm_us = part_us(lambda: [p.run_softmax() for p in plans])
-        qk_us -= sm_us
-    pv_us = part_us(lambda: [p.run(q, only=_lib.ONLY_PV) for p, q in zip(plans, qs)])
-    cb_us = part_us(lambda: [p.run(q, only=_lib.ONLY_COMBINE) for p, q in zip(plans, qs)])
-    for p, q in zip(plans, qs):  # leave consistent outputs behind
-        p.run(q)
-    dominant = "qk_hybrid_kernel" if qk_us >= pv_us else "pv_hybrid_kernel"
-    dom_us, dom_bytes = (qk_us, k_bytes) if qk_us >= pv_us else (pv_us, v_bytes)
-    achieved = dom_bytes / (dom_us * 1e-6) / 1e9
-
-    traffic, traffic_source = recorded_traffic(args.workload, dominant)
-
+    m = measure_decode(args.workload, n_layers, args.steps, args.warmup, args, dev)
     out = {
         "metric": METRIC,
-        "value": round(us_per_step, 3),
+        "value": round(m["us_per_step"], 3),
         "unit": "us/layer",
         "n_gpus": 1,
-        "steps": K,
+        "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(us_per_step / 1e3, 6),
+        "ms_per_step": round(m["us_per_step"] / 1e3, 6),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {WORKLOADS[args.workload]}", "B": cfg["B"], "Hq": cfg["Hq"],
-                   "Hkv": cfg["Hkv"], "head_dim": cfg["D"], "context": cfg["T"], "kept_tokens": pkv0[41],
-                   "layers_cycled": n_layers, "launch": "eager" if graph is None else "hip-graph replay",
-                   "qk_tiling": args.qk_tiling, "dot": args.dot,
-                   "softmax": "fused into the two GEMV launches" if fused else "separate launch",
-                   "algorithmic_bytes_per_step": alg_bytes},
-        "achieved_GBps": round(alg_bytes / (us_per_step * 1e-6) / 1e9, 1),
-        "pct_of_hbm_peak": round(alg_bytes / (us_per_step * 1e-6) / 1e9 / HBM_PEAK_GBPS * 100, 2),
-        "kernels_us": {"qk_hybrid_kernel": round(qk_us, 3), "scale_softmax_kernel": round(sm_us, 3),
-                       "pv_hybrid_kernel": round(pv_us, 3), "pv_combine_kernel": round(cb_us, 3)},
-        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "traffic_source": traffic_source, "bytes_per_launch": dom_bytes, "avg_us": round(dom_us, 3)},
+        "config": m["config"],
+        "timed_regions_us_per_step": m["regions"],
+        "host_clock_us_per_step": round(m["us_per_step_host"], 3),
+        "achieved_GBps": round(m["alg_bytes"] / (m["us_per_step"] * 1e-6) / 1e9, 1),
+        "pct_of_hbm_peak": round(m["alg_bytes"] / (m["us_per_step"] * 1e-6) / 1e9 / HBM_PEAK_GBPS * 100, 2),
+        "kernels_us": m["kernels_us"],
+        "roofline": m["roofline"],
     }
+    us_per_step, cfg, layers, plans, qs = m["us_per_step"], m["cfg"], m["layers"], m["plans"], m["qs"]
+    sync = torch.cuda.synchronize
+    if args.workload == "c2" and not args.no_extra:
+        # the large-launch regime beside the headline: configuration 4's shape on a few layer caches
+        del m
+        try:
+            x = measure_decode("c4", 3, 12, 3, args, dev)
+            out["extra"] = {"workload": x["config"]["workload"], "layers_cycled": 3, "steps": 12, "warmup": 3,
+                            "us_per_layer_step": round(x["us_per_step"], 2),
+                            "timed_regions_us_per_step": x["regions"],
+                            "achieved_GBps": round(x["alg_bytes"] / (x["us_per_step"] * 1e-6) / 1e9, 1),
+                            "pct_of_hbm_peak": round(x["alg_bytes"] / (x["us_per_step"] * 1e-6) / 1e9 / HBM_PEAK_GBPS * 100, 2),
+                            "kernels_us": x["kernels_us"], "roofline": x["roofline"]}
+            del x
+            torch.cuda.empty_cache()
+        except torch.OutOfMemoryError as e:   # a smaller GPU: the headline stands on its own
+            out["extra"] = {"skipped": f"configuration 4 does not fit: {e}"}
 
     if args.workload == "c5":
         # one generated token passes through every resident layer once

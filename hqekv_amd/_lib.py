@@ -25,6 +25,7 @@ ONLY_PV = 0x200
 ONLY_COMBINE = 0x400
 DOT_MFMA = 0x800    # inner products on the matrix cores (Hq/Hkv == 4 only)
 DOT_VALU = 0x1000   # inner products on the vector ALU
+ONLY_RAW_QK = 0x2000   # the q.K^T launch alone, raw fp16 scores
 QK_TILINGS = {"8waves": 1, "4waves": 2, "wave512": 3, "wave256": 4}   # HQEKV_QK_TILING_*: tilings a call may force
 
 
@@ -40,7 +41,7 @@ LAYOUT_NORMAL1 = 2       # 1-bit segment in normal-quantile coding (scale = std,
 EXPORTS = (
     "hqekv_version", "hqekv_last_error",
     "hqekv_quant_pack_rows", "hqekv_quant_pack_k_tokenmajor", "hqekv_dequant_unpack_rows", "hqekv_pack_i32",
-    "hqekv_selftest_quant_division", "hqekv_selftest_wave_reduce",
+    "hqekv_selftest_quant_division", "hqekv_selftest_wave_reduce", "hqekv_selftest_stream_read",
     "hqekv_normal1_quant_pack_rows", "hqekv_normal1_quant_pack_k_tokenmajor", "hqekv_normal1_dequant_unpack_rows",
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group", "hqekv_gemv_normal_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
@@ -92,6 +93,7 @@ _PROTOS = {
     "hqekv_pack_i32": (C.c_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "hqekv_selftest_quant_division": (C.c_int, [_vp, _vp]),
     "hqekv_selftest_wave_reduce": (C.c_int, [_vp, _vp, _i64, _vp]),
+    "hqekv_selftest_stream_read": (C.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hqekv_normal1_quant_pack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "hqekv_normal1_quant_pack_k_tokenmajor": (C.c_int, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "hqekv_normal1_dequant_unpack_rows": (C.c_int, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
@@ -105,7 +107,7 @@ _PROTOS = {
     "hqekv_decode_workspace_bytes": (_i64, [_SEGP, _int, _SEGP, _int, _i64, _i64, _i64, _i64]),
     "hqekv_decode_attn": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _int, _vp]),
     "hqekv_decode_attn_static": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
-    "hqekv_cache_migrate": (C.c_int, [_int, _CCP, _int, _CCP, _int, _vp, _i64, _i64, _vp]),
+    "hqekv_cache_migrate": (C.c_int, [_int, _CCP, _int, _CCP, _int, _vp, _i64, _i64, _vp, _vp]),
 }
 STATIC_SCRATCH_BYTES = 8 << 20   # HQEKV_STATIC_SCRATCH_BYTES
 

@@ -540,8 +540,9 @@ def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, counts, s
     plan_h[nb:2 * nb] = pos
     plan = _to_dev(plan_h[:(2 * nb + 1) // 2 * 2].view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
     with _lib.on_device(dev):
+        # (no status word: this plan was made a few lines up from the classes it names; the kernel still checks it)
         rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src, _SRC_NEW + 1, dst, n_dst, plan.data_ptr(), B * H, D,
-                                             _lib.stream_ptr(dev))
+                                             None, _lib.stream_ptr(dev))
     _lib.check(rc, "cache_migrate")
     # the kernel writes the position arrays behind torch's back: the version stamps taken above still hold, and the
     # host copies describe exactly what the kernel wrote

@@ -2343,6 +2343,11 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
   if ((flags & HQEKV_DOT_MFMA) && Hq / Hkv != 4)
     return fail(HQEKV_E_UNSUPPORTED, "decode_attn: the matrix-core dot products need Hq/Hkv == 4 (got %lld)", (long long)(Hq / Hkv));
   const bool mf = dot_on_matrix_cores(flags, Hq / Hkv);
+  if (flags & HQEKV_ONLY_RAW_QK) {   // the q.K^T launch alone, raw fp16 scores: no scaling, no statistics, no softmax
+    FuseArgs raw{};
+    raw.two_step = fz.two_step;
+    return launch_qk(kt, q, attn_weights, B, Hq, Hkv, D, Tall, raw, st, tiling, mf);
+  }
   const int only = flags & (HQEKV_ONLY_QK | HQEKV_ONLY_PV | HQEKV_ONLY_COMBINE);
   const bool only_qk = only == HQEKV_ONLY_QK;
   if (only == 0 || only_qk) {

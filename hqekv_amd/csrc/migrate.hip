@@ -37,9 +37,24 @@ struct MigArgs {
   MigClass dst[HQEKV_MAX_SEGS];
   int32_t dst_begin[HQEKV_MAX_SEGS + 1];  // first plan entry of every destination class; [n_dst] = total
   int32_t n_dst;
+  int32_t n_src;
   const int32_t *plan_src;  // (source slot << 24) | source block, per destination block
   const int32_t *plan_pos;  // new position of the block's first token / 32
+  int32_t *status;          // optional: set to non-zero when a plan entry is refused
 };
+
+// The plan lives in device memory and is read by the kernel only, so the kernel is what checks it: an entry must name
+// a populated source class, a block inside it and a position inside the new sequence.  An entry that does not is
+// skipped (its destination block keeps whatever the buffer held) and flagged; nothing is read or written out of range.
+__device__ __forceinline__ bool plan_entry_ok(const MigArgs &a, int32_t code, int32_t pos, int total) {
+  const uint32_t slot = (uint32_t)code >> 24, blk = (uint32_t)code & 0xffffffu;
+  if (slot >= (uint32_t)a.n_src) return false;
+  const int64_t n = a.src[slot].n_tokens;
+  return n > 0 && a.src[slot].data != nullptr && (int64_t)blk < (n >> 5) && pos >= 0 && pos < total;
+}
+__device__ __forceinline__ void plan_refused(const MigArgs &a) {
+  if (a.status) atomicOr(a.status, 1);
+}
 
 // where one lane's group lives: fp16 values (with the element stride) or packed words + scale + zero
 struct GroupRef {
@@ -266,23 +281,29 @@ __global__ __launch_bounds__(MIG_THREADS) void cache_migrate_kernel(MigArgs a, i
     const MigClass dc = a.dst[dst_class_of(a, u)];
     const int64_t db = u - a.dst_begin[dst_class_of(a, u)];
     const int32_t code = a.plan_src[u];
+    if (!plan_entry_ok(a, code, a.plan_pos[u], total)) {   // uniform: the whole workgroup serves this entry
+      if (threadIdx.x == 0) plan_refused(a);
+      return;
+    }
     if (bh == 0 && threadIdx.x < 32 && dc.idx) dc.idx[db * 32 + threadIdx.x] = (int64_t)a.plan_pos[u] * 32 + threadIdx.x;
     for (int lane = threadIdx.x; lane < D; lane += MIG_THREADS)
       migrate_group<false>(a.src[code >> 24], dc, bh, code & 0xffffff, db, lane, D);
   } else {
     const int u0 = blockIdx.x * MIG_KB;
     const int u = u0 + (int)(threadIdx.x % MIG_KB);
-    const bool live = u < total;
-    const int uc = live ? u : u0;   // (u0 < total by the grid size)
+    const int uc = u < total ? u : u0;   // (u0 < total by the grid size)
     const int ci = dst_class_of(a, uc);
     const int64_t db = uc - a.dst_begin[ci];
     const int32_t code = a.plan_src[uc];
-    const int si = code >> 24;
-    const bool token_major = a.src[si].bits == 16 && a.src[si].layout == HQEKV_LAYOUT_TOKEN_MAJOR;
+    const bool entry_ok = plan_entry_ok(a, code, a.plan_pos[uc], total);
+    const bool live = u < total && entry_ok;
+    if (u < total && !entry_ok && threadIdx.x < MIG_KB) plan_refused(a);
+    const int si = entry_ok ? (int)((uint32_t)code >> 24) : 0;
+    const bool token_major = entry_ok && a.src[si].bits == 16 && a.src[si].layout == HQEKV_LAYOUT_TOKEN_MAJOR;
     if (bh == 0) {  // positions of the blocks' tokens
       for (int e = threadIdx.x; e < MIG_KB * 32; e += MIG_THREADS) {
         const int ue = u0 + e / 32;
-        if (ue < total) {
+        if (ue < total && plan_entry_ok(a, a.plan_src[ue], a.plan_pos[ue], total)) {
           const int ce = dst_class_of(a, ue);
           int64_t *idx = a.dst[ce].idx;
           if (idx) idx[(int64_t)(ue - a.dst_begin[ce]) * 32 + e % 32] = (int64_t)a.plan_pos[ue] * 32 + e % 32;
@@ -293,6 +314,7 @@ __global__ __launch_bounds__(MIG_THREADS) void cache_migrate_kernel(MigArgs a, i
       for (int j = 0; j < MIG_KB && u0 + j < total; ++j) {
         const int cj = dst_class_of(a, u0 + j);
         const int32_t code_j = a.plan_src[u0 + j];
+        if (!plan_entry_ok(a, code_j, a.plan_pos[u0 + j], total)) continue;   // uniform
         for (int lane = threadIdx.x; lane < D; lane += MIG_THREADS)
           migrate_group<true>(a.src[code_j >> 24], a.dst[cj], bh, code_j & 0xffffff, u0 + j - a.dst_begin[cj], lane, D);
       }
@@ -323,7 +345,7 @@ static int check_class(const hqekv_cache_class &c, bool is_src, int k, int64_t D
 using namespace hq;
 
 extern "C" int hqekv_cache_migrate(int is_k, const hqekv_cache_class *src, int n_src, const hqekv_cache_class *dst,
-                                   int n_dst, const int32_t *plan, int64_t BH, int64_t D, void *stream) {
+                                   int n_dst, const int32_t *plan, int64_t BH, int64_t D, int32_t *status, void *stream) {
   if (n_src < 0 || n_src > HQEKV_MAX_SEGS || n_dst < 0 || n_dst > HQEKV_MAX_SEGS || (n_src && !src) || (n_dst && !dst))
     return fail(HQEKV_E_ARG, "cache_migrate: bad class tables");
   if (BH <= 0 || BH > 65535 || D <= 0 || D % 32 != 0 || D > 1024)
@@ -355,6 +377,8 @@ extern "C" int hqekv_cache_migrate(int is_k, const hqekv_cache_class *src, int n
   if (total >= (1 << 24)) return fail(HQEKV_E_UNSUPPORTED, "cache_migrate: %lld blocks (limit 2^24)", (long long)total);
   if (!plan) return fail(HQEKV_E_ARG, "cache_migrate: null plan");
   a.n_dst = n_dst;
+  a.n_src = n_src;
+  a.status = status;
   a.plan_src = plan;
   a.plan_pos = plan + total;
   const dim3 block(MIG_THREADS);

@@ -582,6 +582,40 @@ extern "C" int hqekv_selftest_wave_reduce(const void *in, void *out, int64_t n_w
   return check_launch("selftest_wave_reduce_kernel");
 }
 
+// Yardstick: a launch that does nothing but read `bytes` bytes, as wide and as deep as the hardware likes them
+// (16 bytes per lane, eight requests in flight per lane, every CU busy).  What this takes, launch included, is the
+// floor for any kernel that has to read the same bytes once.  `sum` receives one word per workgroup (so that the
+// loads cannot be dropped).
+namespace hq {
+constexpr int SR_THREADS = 256, SR_UNROLL = 8;
+__global__ __launch_bounds__(SR_THREADS) void stream_read_kernel(const uint4 *__restrict__ p, int64_t n16, uint32_t *__restrict__ sum) {
+  uint32_t acc = 0;
+  const int64_t stride = (int64_t)gridDim.x * SR_THREADS * SR_UNROLL;
+  for (int64_t i = (int64_t)blockIdx.x * SR_THREADS * SR_UNROLL + threadIdx.x; i < n16; i += stride) {
+    uint4 v[SR_UNROLL];
+#pragma unroll
+    for (int k = 0; k < SR_UNROLL; ++k) {
+      const int64_t j = i + (int64_t)k * SR_THREADS;
+      v[k] = j < n16 ? p[j] : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int k = 0; k < SR_UNROLL; ++k) acc ^= v[k].x ^ v[k].y ^ v[k].z ^ v[k].w;
+  }
+  for (int o = 32; o; o >>= 1) acc ^= (uint32_t)__shfl_xor((int)acc, o, HQ_WAVE);
+  if ((threadIdx.x & 63) == 0) atomicXor(sum + blockIdx.x, acc);
+}
+}  // namespace hq
+
+extern "C" int hqekv_selftest_stream_read(const void *src, int64_t bytes, void *sum, int64_t n_workgroups, void *stream) {
+  if (!src || !sum || bytes < 0 || n_workgroups <= 0 || n_workgroups > 65535)
+    return fail(HQEKV_E_ARG, "selftest_stream_read: null pointer, negative size or 0 / more than 65535 workgroups");
+  if (((uintptr_t)src & 15) || (bytes & 15)) return fail(HQEKV_E_ALIGN, "selftest_stream_read: 16-byte granularity");
+  if (bytes == 0) return HQEKV_OK;
+  hipLaunchKernelGGL(hq::stream_read_kernel, dim3((unsigned)n_workgroups), dim3(hq::SR_THREADS), 0, (hipStream_t)stream,
+                     (const uint4 *)src, bytes / 16, (uint32_t *)sum);
+  return check_launch("stream_read_kernel");
+}
+
 extern "C" int hqekv_selftest_quant_division(void *counts, void *stream) {
   if (!counts) return fail(HQEKV_E_ARG, "selftest_quant_division: null pointer");
   if ((uintptr_t)counts & 7) return fail(HQEKV_E_ALIGN, "selftest_quant_division: counts must be 8-byte aligned");

@@ -119,6 +119,14 @@ int hqekv_selftest_quant_division(void *counts, void *stream);
  */
 int hqekv_selftest_wave_reduce(const void *in, void *out, int64_t n_waves, void *stream);
 
+/* No counterpart in the reference: the measurement yardstick.  One launch of `n_workgroups` workgroups that only reads
+ * `bytes` bytes at `src` (16-byte loads, eight in flight per lane) and XORs them into `sum` (n_workgroups uint32,
+ * device, so the reads cannot be elided).  Its duration, launch included, is the floor for any kernel that must read
+ * the same bytes once; the benchmark prints it beside the decode kernels' figures.  src 16-byte aligned, bytes a
+ * multiple of 16, n_workgroups in [1, 65535].
+ */
+int hqekv_selftest_stream_read(const void *src, int64_t bytes, void *sum, int64_t n_workgroups, void *stream);
+
 /* Replaces pack_along_last_dim (quant/pack_unpack.py:16-70): q is (n_rows, L) int32 codes,
  * code is (n_rows, L/pf) int32, both contiguous. */
 int hqekv_pack_i32(const void *q, void *code, int64_t n_rows, int64_t L, int bits, void *stream);
@@ -256,6 +264,10 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
  * HQEKV_DOT_MFMA with another head ratio returns HQEKV_E_UNSUPPORTED. */
 #define HQEKV_DOT_MFMA 0x800
 #define HQEKV_DOT_VALU 0x1000
+/* Run the q.K^T launch alone and leave the RAW fp16 scores in attn_weights (no scaling, no softmax), with the tiling
+ * and the form of the dot products the other flags name: what gemv_forward_cuda_qk_group_hq returns
+ * (quant/csrc/gemv_cuda.h:78-109), for callers and tests that want the scores of one particular tiling. */
+#define HQEKV_ONLY_RAW_QK 0x2000
 int64_t hqekv_decode_workspace_bytes(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
                                      int64_t B, int64_t Hq, int64_t Hkv, int64_t D);
 int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
@@ -279,6 +291,10 @@ int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs,
  * destination is dropped (evicted).  Same width: the packed bytes are copied; fp16 -> b bits: quantised; a -> b < a
  * bits: dequantised with the two fp16 roundings, then quantised; never the other way round.
  * is_k != 0: classes are (B,H,D,*) with groups of 32 tokens per channel; else (B,H,T,*) with groups of 32 channels.
+ * The plan is device memory the host never sees, so the kernel checks every entry it reads: a source slot that is
+ * not populated, a source block past the end of its class or a position outside the new sequence makes the kernel
+ * skip that destination block (nothing out of range is touched) and, when `status` (device, one int32 the caller has
+ * zeroed; may be NULL) is given, set it to a non-zero value.
  */
 typedef struct hqekv_cache_class {
   int32_t bits;      /* 16, 8, 4, 2 or 1                       */
@@ -292,7 +308,7 @@ typedef struct hqekv_cache_class {
   int64_t *idx;      /* destination only: (n_tokens) or NULL   */
 } hqekv_cache_class;
 int hqekv_cache_migrate(int is_k, const hqekv_cache_class *src, int n_src, const hqekv_cache_class *dst,
-                        int n_dst, const int32_t *plan, int64_t BH, int64_t D, void *stream);
+                        int n_dst, const int32_t *plan, int64_t BH, int64_t D, int32_t *status, void *stream);
 
 /* No counterpart in the reference: hqekv_decode_attn for callers that cannot allocate (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  Same arguments minus the workspace: the split-K

@@ -52,15 +52,18 @@ def test_argument_validation_without_a_gpu():
     assert rc == -1 and b"null" in lib.hqekv_last_error()
     assert lib.hqekv_selftest_wave_reduce(None, None, 4, None) == -1
     assert lib.hqekv_selftest_quant_division(None, None) == -1
+    assert lib.hqekv_selftest_stream_read(None, 16, None, 1, None) == -1
+    assert lib.hqekv_selftest_stream_read(16, 16, 16, 0, None) == -1
+    assert lib.hqekv_selftest_stream_read(16, 24, 16, 1, None) == -2
     # cache migration: class tables are checked before anything is launched
     cc = (_lib.CacheClass * 2)()
     cc[0].bits, cc[0].n_tokens, cc[0].data = 16, 48, 256
-    assert lib.hqekv_cache_migrate(1, cc, 1, cc, 1, None, 4, 128, None) == -1 and b"whole blocks" in lib.hqekv_last_error()
+    assert lib.hqekv_cache_migrate(1, cc, 1, cc, 1, None, 4, 128, None, None) == -1 and b"whole blocks" in lib.hqekv_last_error()
     cc[0].n_tokens = 64
-    assert lib.hqekv_cache_migrate(1, cc, 1, cc, 1, None, 4, 128, None) == -1 and b"null plan" in lib.hqekv_last_error()
+    assert lib.hqekv_cache_migrate(1, cc, 1, cc, 1, None, 4, 128, None, None) == -1 and b"null plan" in lib.hqekv_last_error()
     cc[0].bits = 3
-    assert lib.hqekv_cache_migrate(0, cc, 1, cc, 1, None, 4, 128, None) == -1
-    assert lib.hqekv_cache_migrate(0, cc, 9, cc, 1, None, 4, 128, None) == -1
+    assert lib.hqekv_cache_migrate(0, cc, 1, cc, 1, None, 4, 128, None, None) == -1
+    assert lib.hqekv_cache_migrate(0, cc, 9, cc, 1, None, 4, 128, None, None) == -1
     # a segment table with an unknown bit width
     segs = _lib.make_segs([dict(bits=3, n_tokens=32, data=None)])
     segs[0].data = 16

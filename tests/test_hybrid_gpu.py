@@ -536,3 +536,41 @@ def test_random_configurations(dev):
         assert torch.allclose(o.float(), o_stage, rtol=RTOL, atol=ATOL), what
         checked += 1
     assert checked >= 150
+
+
+@pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave256"])
+@pytest.mark.parametrize("dot", ["mfma", "valu"])
+def test_score_scaling_matches_torch_division_on_device(dev, tiling, dot):
+    """``attn_weights /= math.sqrt(head_dim)`` (quant/quant_matmul_hq.py:100) pinned on the device: the scaled fp16
+    logits the fused q.K^T launch stores must equal, bit for bit, the raw fp16 scores of the same launch (same tiling,
+    same form of the dot products) followed by torch's own in-place division executed on the GPU, which multiplies by
+    the fp32 reciprocal and rounds to fp16.  Data like configuration 2: hybrid classes, K outlier channels, logits of
+    a hundred and more, where one fp16 place is 0.06."""
+    import math
+    from hqekv_amd import _lib
+    from hqekv_amd.attention import DecodePlan
+    B, Hq, Hkv, T, D = 2, 32, 8, 4096, 128
+    q, K, V = synth.make_qkv(B, Hq, Hkv, T, D, 4242)
+    classes = synth.split_blocks(T, (0.05, 0.15, 0.30, 0.30, 0.20), 4242)
+    cache = synth.cache_to(synth.build_cache(K, V, classes, 0, O.uniform_group_quantize_pack_last_dim), dev)
+    form = _lib.DOT_MFMA if dot == "mfma" else _lib.DOT_VALU
+    plan = DecodePlan(q.to(dev), cache, flags=_lib.FUSE_SOFTMAX | _lib.qk_tiling(_lib.QK_TILINGS[tiling]) | form)
+    assert plan.flags & _lib.FUSE_SOFTMAX
+    qd = q.to(dev).contiguous()
+    plan.run(qd, only=_lib.ONLY_QK)
+    scaled = plan.weights.clone()
+    plan.run(qd, only=_lib.ONLY_RAW_QK)
+    raw = plan.weights.clone()
+    torch.cuda.synchronize()
+    assert float(raw.float().abs().max()) > 100.0
+    expect = raw.clone()
+    expect /= math.sqrt(D)                                  # torch's own op, on the device
+    assert torch.equal(scaled.view(torch.int16), expect.view(torch.int16))
+    # and the rule itself on every fp16 bit pattern: x / sqrt(128) on the device == rnd16(x * fp32(1 / sqrt(128)))
+    allx = torch.arange(0, 65536, dtype=torch.int32, device=dev).to(torch.int16).view(torch.float16)
+    finite = torch.isfinite(allx)
+    by_torch = allx.clone()
+    by_torch /= math.sqrt(D)
+    inv = torch.tensor(1.0, dtype=torch.float32, device=dev) / torch.tensor(float(D), dtype=torch.float32, device=dev).sqrt()
+    by_rule = (allx.float() * inv).half()
+    assert torch.equal(by_torch[finite].view(torch.int16), by_rule[finite].view(torch.int16))

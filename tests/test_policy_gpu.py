@@ -260,10 +260,53 @@ def test_cache_migrate_random_plans(dev, is_k, low_normal, D):
             d.layout = _lib.LAYOUT_NORMAL1 if (b == 1 and low_normal) else 0
         got[b] = (oc, os_, oz, oi)
     plan = torch.tensor(plan_src + plan_pos, dtype=torch.int32).to(dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
     rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src, 6, dst, n_dst, plan.data_ptr(), B * H, D,
-                                         _lib.stream_ptr(torch.device(dev)))
+                                         status.data_ptr(), _lib.stream_ptr(torch.device(dev)))
     _lib.check(rc, "cache_migrate")
     torch.cuda.synchronize()
+    assert int(status) == 0
     for b in want:
         for name, a, w in zip(("code", "scale", "zero", "idx"), got[b], want[b]):
             _same(a, w, f"{b}-bit class {name}")
+    # A plan that is wrong in every way the kernel can be told: a slot past the table, an empty slot, a block past
+    # the end of its class, a position outside the new sequence.  Those entries are refused -- their destination
+    # blocks keep the sentinel, the status word is set -- and every other entry is served as before.
+    n_all = len(plan_src)
+    bad_src, bad_pos = list(plan_src), list(plan_pos)
+    victims = [0, n_all // 3, n_all // 2, n_all - 1]
+    bad_src[victims[0]] = (7 << 24) | 0                       # slot 7 of a table of 7 entries (6 populated + 1 empty)
+    bad_src[victims[1]] = (6 << 24) | 0                       # the empty slot
+    bad_src[victims[2]] = (1 << 24) | (n_src[1] + 3)          # past the end of the 8-bit class
+    bad_pos[victims[3]] = n_all + 5                           # position outside the new sequence
+    src7 = (_lib.CacheClass * 7)()
+    for i in range(6):
+        C_ = src[i]
+        for f, _t in _lib.CacheClass._fields_:
+            setattr(src7[i], f, getattr(C_, f))
+    sent_i, sent_h = -1234567, -3.0
+    for b in got:
+        oc, os_, oz, oi = got[b]
+        oc.fill_(sent_i if oc.dtype == torch.int32 else sent_h)
+        oi.fill_(-7)
+        if os_ is not None:
+            os_.fill_(sent_h)
+            oz.fill_(sent_h)
+    plan_bad = torch.tensor(bad_src + bad_pos, dtype=torch.int32).to(dev)
+    rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src7, 7, dst, n_dst, plan_bad.data_ptr(), B * H, D,
+                                         status.data_ptr(), _lib.stream_ptr(torch.device(dev)))
+    _lib.check(rc, "cache_migrate")
+    torch.cuda.synchronize()
+    assert int(status) != 0
+    u = 0
+    for b in bits_of:
+        if b not in want:
+            continue
+        oi, wi = got[b][3].cpu(), want[b][3]
+        for k in range(wi.numel() // 32):
+            sl = slice(32 * k, 32 * k + 32)
+            if u + k in victims:
+                assert bool((oi[sl] == -7).all()), f"{b}-bit class: refused block {k} was written"
+            else:
+                assert torch.equal(oi[sl], wi[sl]), f"{b}-bit class: block {k} of a plan with refused entries"
+        u += wi.numel() // 32
