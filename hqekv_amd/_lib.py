@@ -45,7 +45,7 @@ EXPORTS = (
     "hqekv_normal1_quant_pack_rows", "hqekv_normal1_quant_pack_k_tokenmajor", "hqekv_normal1_dequant_unpack_rows",
     "hqekv_gemv_workspace_bytes", "hqekv_gemv_uniform_group", "hqekv_gemv_normal_group",
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
-    "hqekv_decode_workspace_bytes", "hqekv_decode_attn", "hqekv_decode_attn_static",
+    "hqekv_decode_workspace_bytes", "hqekv_decode_attn", "hqekv_decode_attn_static", "hqekv_decode_step", "hqekv_ring_row",
     "hqekv_cache_migrate",
 )
 
@@ -61,6 +61,22 @@ class Seg(C.Structure):
         ("scale", C.c_void_p),
         ("zero", C.c_void_p),
         ("idx", C.c_void_p),
+        ("slab_tokens", C.c_int64),
+    ]
+
+
+class StepExtra(C.Structure):
+    """Mirror of ``struct hqekv_step_extra``."""
+    _fields_ = [
+        ("ring_line", C.c_void_p),
+        ("ring_order", C.c_int32),
+        ("append_rows", C.c_int32),
+        ("new_k", C.c_void_p),
+        ("new_v", C.c_void_p),
+        ("k_dst", C.c_void_p),
+        ("v_dst", C.c_void_p),
+        ("k_dst_slab_tokens", C.c_int64),
+        ("v_dst_slab_tokens", C.c_int64),
     ]
 
 
@@ -106,6 +122,8 @@ _PROTOS = {
     "hqekv_pv_hybrid": (C.c_int, [_SEGP, _int, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "hqekv_decode_workspace_bytes": (_i64, [_SEGP, _int, _SEGP, _int, _i64, _i64, _i64, _i64]),
     "hqekv_decode_attn": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _int, _vp]),
+    "hqekv_decode_step": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _int, _vp, C.POINTER(StepExtra)]),
+    "hqekv_ring_row": (C.c_int, [_vp, _i64, _i64, _i64, _vp, _int, _vp]),
     "hqekv_decode_attn_static": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "hqekv_cache_migrate": (C.c_int, [_int, _CCP, _int, _CCP, _int, _vp, _i64, _i64, _vp, _vp]),
 }
@@ -192,4 +210,5 @@ def make_segs(items) -> "C.Array[Seg]":
         s.scale = ptr(it.get("scale"))
         s.zero = ptr(it.get("zero"))
         s.idx = ptr(it.get("idx"))
+        s.slab_tokens = int(it.get("slab_tokens", 0))
     return arr

@@ -37,6 +37,32 @@ def _idx(t: Optional[torch.Tensor], n: int, dev) -> Optional[torch.Tensor]:
     return t
 
 
+def token_major_window(t: torch.Tensor):
+    """An fp16 (B,H,n,D) tensor as the kernels read it: -> (tensor whose data_ptr is the first row, token rows between
+    two (b, h) slabs or 0 when dense).  The head of a longer buffer -- ``buf[:, :, :n]`` of a capacity-sized residual
+    buffer -- is read where it lies; anything else that is not dense is copied."""
+    if t.is_contiguous():
+        return t, 0
+    B, H, n, D = t.shape
+    sb, sh, st, sd = t.stride()
+    if sd == 1 and st == D and sh % D == 0 and sh >= n * D and (B == 1 or sb == H * sh):
+        return t, sh // D
+    return t.contiguous(), 0
+
+
+def ring_order(T: int, weights: torch.Tensor) -> int:
+    """How torch's GPU reduction deals the 32 head rows of ``weights`` (B,32,1,T) to threads when it sums them: to two
+    threads when rows are a multiple of 4 long, at least 256, and 8-byte aligned, else to one (measured on the
+    device; ``hqekv_ring_row`` and the decode step reproduce either order bit for bit)."""
+    return 2 if (T % 4 == 0 and T >= 256 and weights.data_ptr() % 8 == 0) else 1
+
+
+def ring_row_on_device_applies(weights: torch.Tensor) -> bool:
+    """Shapes for which the ring row's order is pinned against torch on the device."""
+    return (weights.dtype == torch.float16 and weights.dim() == 4 and weights.shape[2] == 1 and weights.shape[1] == 32
+            and weights.shape[0] <= 8 and weights.shape[3] >= 256 and weights.is_contiguous())
+
+
 def _f16_k_item(k16: torch.Tensor, idx, keep: list) -> dict:
     """fp16 K class (B,Hkv,D,T): read channel-major, or token-major if it is a transposed view."""
     B, H, D, T = k16.shape
@@ -74,11 +100,11 @@ def key_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = Tru
             items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx, layout=layout))
     new_K = pkv[NEW_K]
     if residual and new_K is not None and new_K.shape[2] > 0:
-        nk = new_K.contiguous()
+        nk, slab = token_major_window(new_K)
         keep.append(nk)
         nh_kv, D = nk.shape[1], nk.shape[3]
         n = nk.shape[2]
-        items.append(dict(bits=16, n_tokens=n, data=nk, idx=None, pos_base=Tall - n, token_major=1))
+        items.append(dict(bits=16, n_tokens=n, data=nk, idx=None, pos_base=Tall - n, token_major=1, slab_tokens=slab))
     return items, nh_kv, D
 
 
@@ -106,11 +132,11 @@ def value_segments(pkv: tuple, dev, Tall: int, keep: list, low_uniform: bool = T
             items.append(dict(bits=b, n_tokens=n, data=code, scale=sc, zero=zr, idx=idx, layout=layout))
     new_V = pkv[NEW_V]
     if residual and new_V is not None and new_V.shape[2] > 0:
-        nv = new_V.contiguous()
+        nv, slab = token_major_window(new_V)
         keep.append(nv)
         nh_kv, D = nv.shape[1], nv.shape[3]
         n = nv.shape[2]
-        items.append(dict(bits=16, n_tokens=n, data=nv, idx=None, pos_base=Tall - n))
+        items.append(dict(bits=16, n_tokens=n, data=nv, idx=None, pos_base=Tall - n, slab_tokens=slab))
     return items, nh_kv, D
 
 
@@ -244,6 +270,7 @@ class SegmentMemo:
         self.Hkv = None
         self.dims = (None, None)
         self.partition = False                 # the classes' position arrays cover [0, kept) once per side
+        self._step = None                      # what step_call keeps between steps
 
     def lookup(self, pkv: tuple, dev, low_uniform: bool) -> bool:
         held = self.held
@@ -272,14 +299,15 @@ class SegmentMemo:
         self.held = tuple(pkv[:NEW_K])
         self.key = (dev, low_uniform)
         self.partition = classes_partition_positions(pkv)
+        self._step = None
 
     @staticmethod
     def _fill(s, t: torch.Tensor, end: int, layout: int, keep: list):
         """Table entry of an fp16 token-major block (B,Hkv,n,D) whose last token sits at position end - 1."""
-        tc = t.contiguous()
+        tc, slab = token_major_window(t)
         keep.append(tc)
         n = tc.shape[2]
-        s.bits, s.layout, s.n_tokens, s.pos_base, s.data = 16, layout, n, end - n, tc.data_ptr()
+        s.bits, s.layout, s.n_tokens, s.pos_base, s.data, s.slab_tokens = 16, layout, n, end - n, tc.data_ptr(), slab
         return tc.shape[1], tc.shape[3]
 
     def tables(self, pkv: tuple, Tall: int, keep: list, tail=None):
@@ -308,9 +336,78 @@ class SegmentMemo:
             self.ws = torch.empty(max(need + need // 8, 256) // 4, dtype=torch.float32, device=dev)
         return self.ws
 
+    def step_call(self, q: torch.Tensor, pkv: tuple, Tall: int, k: torch.Tensor, v: torch.Tensor, res, n: int,
+                  ring_store: Optional[torch.Tensor], ring_row: int, low_uniform: bool):
+        """One decode step of a layer as one C call (``hqekv_decode_step``) with as little host work as the call
+        allows: the class entries of the tables are the memo's, the residual is the first ``n`` token rows of the
+        capacity buffers ``res`` = (K, V), this step's ``k`` / ``v`` (B,Hkv,L,D, dense) are read as a segment of
+        their own and copied to row ``n`` of the buffers, and -- when ``ring_store`` (rows x max_length, fp16) is
+        given -- row ``ring_row`` of it receives the ring row.  -> (attn_weights, attn_output)."""
+        dev = q.device
+        if not self.lookup(pkv, dev, low_uniform):
+            self.build(pkv, dev, low_uniform)
+        B, Hq, _, D = q.shape
+        Hkv, L = k.shape[1], k.shape[2]
+        kbuf, vbuf = res
+        st = self._step
+        if st is None or st[0] is not kbuf:
+            # entries that stay the same from step to step: the residual's (bits, layout, data, slab), the tail's
+            # (bits, layout), and the appends' slab lengths
+            for arr, base, buf, layout in ((self.k_arr, self.n_k, kbuf, _lib.LAYOUT_TOKEN_MAJOR), (self.v_arr, self.n_v, vbuf, 0)):
+                for j in (0, 1):
+                    e = arr[base + j]
+                    e.bits, e.layout, e.scale, e.zero, e.idx, e.slab_tokens = 16, layout, None, None, None, 0
+            x = _lib.StepExtra()
+            x.k_dst_slab_tokens, x.v_dst_slab_tokens = kbuf.shape[2], vbuf.shape[2]
+            st = self._step = (kbuf, x, kbuf.data_ptr(), vbuf.data_ptr(), kbuf.shape[2])
+        _, x, kptr, vptr, cap = st
+        n_k, n_v = self.n_k, self.n_v
+        ka, va = self.k_arr, self.v_arr
+        if n:
+            e = ka[n_k]
+            e.n_tokens, e.pos_base, e.data, e.slab_tokens = n, Tall - L - n, kptr, cap
+            e = va[n_v]
+            e.n_tokens, e.pos_base, e.data, e.slab_tokens = n, Tall - L - n, vptr, cap
+            n_k += 1
+            n_v += 1
+        e = ka[n_k]
+        e.n_tokens, e.pos_base, e.data, e.slab_tokens = L, Tall - L, k.data_ptr(), 0
+        e = va[n_v]
+        e.n_tokens, e.pos_base, e.data, e.slab_tokens = L, Tall - L, v.data_ptr(), 0
+        n_k += 1
+        n_v += 1
+        # (positions nobody writes must read as zero when the classes do not cover every position)
+        weights = (torch.empty if self.partition else torch.zeros)(B, Hq, 1, Tall, dtype=torch.float16, device=dev)
+        out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev)
+        if ring_store is not None:
+            x.ring_line = ring_store.data_ptr() + 2 * ring_row * ring_store.shape[1]
+            x.ring_order = 2 if (Tall % 4 == 0 and Tall >= 256 and weights.data_ptr() % 8 == 0) else 1
+        else:
+            x.ring_line = None
+        row_bytes = 2 * D
+        x.append_rows, x.new_k, x.new_v = L, k.data_ptr(), v.data_ptr()
+        x.k_dst, x.v_dst = kptr + n * row_bytes, vptr + n * row_bytes
+        flags = default_flags() if self.partition else 0
+        lib = _lib.load()
+        ws = self.ws
+        with _lib.on_device(dev):
+            for attempt in (0, 1):
+                if ws is None or attempt:
+                    need = lib.hqekv_decode_workspace_bytes(ka, n_k, va, n_v, B, Hq, Hkv, D)
+                    if need < 0:
+                        raise ValueError("invalid segment table")
+                    ws = self.workspace(2 * need, dev)   # room for the residual to grow without asking again
+                rc = lib.hqekv_decode_step(ka, n_k, va, n_v, q.data_ptr(), None, 0, weights.data_ptr(), out.data_ptr(),
+                                           B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4, flags,
+                                           _lib.stream_ptr(dev), C.byref(x))
+                if rc != -3:   # HQEKV_E_WORKSPACE: the cache has outgrown the workspace kept from earlier steps
+                    break
+        _lib.check(rc, "decode_step")
+        return weights, out
+
 
 def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bool, flags: Optional[int] = None,
-                     low_uniform: bool = True, memo: Optional[SegmentMemo] = None, tail=None):
+                     low_uniform: bool = True, memo: Optional[SegmentMemo] = None, tail=None, step=None):
     """q (B,Hq,1,D) fp16 -> (attn_weights (B,Hq,1,Tall) fp16 probabilities, attn_output (B,Hq,1,D) fp16).
 
     One q.K^T launch over all K classes and one p.V launch over all V classes with the softmax fused
@@ -321,6 +418,10 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
     ``tail`` = (k, v), each (B,Hkv,L,D) fp16: tokens that follow the tuple's residual without being part of it yet
     (``Tall`` counts them).  The kernels read them as one more fp16 segment per side, so a caller can start the
     attention of a decode step before it appends the step's key and value to the residual.
+    ``step``: what the caller's decode step does around the attention, folded into the call's last launch
+    (``hqekv_decode_step``): ``step["ring_line"]`` = a (Tall,) fp16 view that receives ``attn_weights.sum(0).sum(0)``
+    in torch's order (only for shapes ``ring_row_on_device_applies`` covers; the caller checks), ``step["append"]`` =
+    (K buffer, V buffer, n): the rows of ``tail`` are copied to token row n of the (B,Hkv,cap,D) buffers.
     """
     _lib.require_gpu(q, "q")
     if q.dtype != torch.float16:
@@ -374,10 +475,28 @@ def decode_attention(q: torch.Tensor, pkv: tuple, mask, Tall: int, zero_init: bo
             ws = memo.workspace(need, dev)
         else:
             ws = decode_workspace(k_segs, n_k, v_segs, n_v, B, Hq, Hkv, D, dev)
-        rc = lib.hqekv_decode_attn(
-            k_segs, n_k, v_segs, n_v, qc.data_ptr(), mptr, mstride,
-            weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4,
-            use_flags, _lib.stream_ptr(dev))
+        if step is None:
+            rc = lib.hqekv_decode_attn(
+                k_segs, n_k, v_segs, n_v, qc.data_ptr(), mptr, mstride,
+                weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4,
+                use_flags, _lib.stream_ptr(dev))
+        else:
+            x = _lib.StepExtra()
+            line = step.get("ring_line")
+            if line is not None:
+                x.ring_line, x.ring_order = line.data_ptr(), ring_order(Tall, weights)
+            app = step.get("append")
+            if app is not None:
+                kbuf, vbuf, n = app
+                tk, tv = tail[0].contiguous(), tail[1].contiguous()
+                keep += [tk, tv]
+                x.append_rows, x.new_k, x.new_v = tk.shape[2], tk.data_ptr(), tv.data_ptr()
+                x.k_dst, x.v_dst = kbuf[0, 0, n].data_ptr(), vbuf[0, 0, n].data_ptr()
+                x.k_dst_slab_tokens, x.v_dst_slab_tokens = kbuf.shape[2], vbuf.shape[2]
+            rc = lib.hqekv_decode_step(
+                k_segs, n_k, v_segs, n_v, qc.data_ptr(), mptr, mstride,
+                weights.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, Tall, ws.data_ptr(), ws.numel() * 4,
+                use_flags, _lib.stream_ptr(dev), C.byref(x))
     _lib.check(rc, "decode_attention")
     return weights, out
 

@@ -48,6 +48,7 @@ struct SegDev {
   int32_t layout;      // HQEKV_LAYOUT_*: 1 = fp16 K stored token-major, 2 = 1-bit normal-quantile coding
   int32_t unit_begin;  // first chunk of this segment in the p.V partial buffer
   int32_t n_units;     // tiles (q.K^T) or chunks (p.V) of this segment
+  int64_t slab_tokens; // token rows between two (b, kv head) slabs of a token-major fp16 segment (>= n_tokens)
 };
 
 struct SegTable {
@@ -94,6 +95,25 @@ struct FuseArgs {
   uint32_t *arrive;
   half_t *out;         // (B*Hq, D) attention output, written by the last workgroup of each (b, kv head)
   int32_t two_step;    // never fold the bias removal of a code into its multiply (HQEKV_TWO_STEP_DEQUANT)
+};
+
+// What the caller of a decode step does next to the attention (model/llama_hqe.py:131-133, 200), folded into the
+// step's last launch: the row of the importance ring -- the probabilities summed over the batch, rounded to fp16,
+// then summed over the heads and rounded again (model/public_func.py:243-257: attn_weights.sum(0).sum(0)) -- and
+// the copies that append the step's key and value rows to the fp16 residual.
+struct StepEpilogue {
+  const half_t *weights;   // (B, Hq, Tall) probabilities
+  half_t *ring_line;       // (Tall) or nullptr
+  int64_t Tall;
+  int32_t B, Hq;
+  int32_t ring_by;         // threads torch's reduction deals the head rows to for this shape: 1 or 2
+  int32_t app_rows;        // token rows to append per (b, kv head); 0 = none
+  int32_t app_row_elems;   // head_dim
+  int32_t app_bh;          // B * Hkv
+  const half_t *app_src[2];
+  half_t *app_dst[2];          // first destination row of slab 0
+  int64_t app_src_slab[2];     // elements between two (b, kv head) slabs
+  int64_t app_dst_slab[2];
 };
 
 // A workgroup learns its segment and its tile/chunk from its block id with two scalar loads at the top of
@@ -578,7 +598,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
                                                int Hq, int64_t Tall, int wave, int lane, const half2_t *q2s,
                                                half_t *__restrict__ scores, const FuseArgs &fz, float *red) {
   const int64_t n = sg.n_tokens;
-  const half_t *kb = (const half_t *)sg.data + (int64_t)bh * n * D;
+  const half_t *kb = (const half_t *)sg.data + (int64_t)bh * sg.slab_tokens * D;
   const int DP = D >> 1;
   constexpr int TPW = 64 / QK_WAVES;  // tokens per wave
   float m_run[NREP], l_run[NREP];  // running softmax statistics of this wave's tokens (fused mode)
@@ -1615,7 +1635,8 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
   const int g = cl >> 2;
   const int sh2 = (BITS == 2) ? (cl & 1) * 16 : (BITS == 1) ? (cl & 3) * 8 : 0;
   const uint32_t wofs = (BITS == 1 ? (cl >> 2) : BITS == 2 ? (cl >> 1) : cl * WPL) * 4u;  // byte offset inside a token row
-  const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * sg.n_tokens * ROWB, (uint32_t)(sg.n_tokens * ROWB));
+  const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * (BITS == 16 ? sg.slab_tokens : sg.n_tokens) * ROWB,
+                              (uint32_t)(sg.n_tokens * ROWB));
   const uint32_t lane_off = (uint32_t)(2 * tl) * ROWB + wofs;   // this lane's first token of a step + word
 
   struct Words {
@@ -1924,13 +1945,84 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   if (threadIdx.x == 0) __hip_atomic_store(&fz.arrive[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---- the importance ring's row, in the order torch's GPU reduction adds fp16 rows in (fp32 accumulators):
+// a thread of that reduction walks its rows with FOUR interleaved accumulators (its k-th row goes to accumulator
+// k mod 4, each starting from zero) and adds them up as ((a0 + a1) + a2) + a3; the rows of one output are dealt
+// round-robin to `by` threads whose results are added in a halving tree.  by is 1 for the sum over the batch, and for
+// the sum over the 32 heads it is 2 when the row length is a multiple of 4 of at least 256 on an 8-byte aligned
+// input, else 1 (measured against torch.sum on the device; the caller passes the value for its shape).
+template <int NBY, typename Load>
+__device__ __forceinline__ float torch_row_sum(int n_rows, Load &&load) {
+  float v[NBY];
+#pragma unroll
+  for (int y = 0; y < NBY; ++y) {
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int r = y;
+    for (; r + 3 * NBY < n_rows; r += 4 * NBY) {
+      a0 += load(r);
+      a1 += load(r + NBY);
+      a2 += load(r + 2 * NBY);
+      a3 += load(r + 3 * NBY);
+    }
+    if (r < n_rows) a0 += load(r);
+    if (r + NBY < n_rows) a1 += load(r + NBY);
+    if (r + 2 * NBY < n_rows) a2 += load(r + 2 * NBY);
+    v[y] = ((a0 + a1) + a2) + a3;
+  }
+  if constexpr (NBY == 2) return v[0] + v[1];
+  return v[0];
+}
+
+// columns [c0, c0 + n) of the ring row; one column per thread
+__device__ __forceinline__ void ring_row_columns(const StepEpilogue &e, int64_t c0, int64_t c1) {
+  for (int64_t t = c0 + threadIdx.x; t < c1; t += blockDim.x) {
+    const half_t *col = e.weights + t;
+    const int64_t hs = e.Tall, bs = (int64_t)e.Hq * e.Tall;
+    auto head = [&](int h) -> float {   // the batch sum of head h, rounded to fp16 as the first reduction stores it
+      if (e.B == 1) return (float)col[(int64_t)h * hs];
+      const float sb = torch_row_sum<1>(e.B, [&](int b) { return (float)col[(int64_t)b * bs + (int64_t)h * hs]; });
+      return (float)(half_t)sb;
+    };
+    const float sum = e.ring_by == 2 ? torch_row_sum<2>(e.Hq, head) : torch_row_sum<1>(e.Hq, head);
+    e.ring_line[t] = (half_t)sum;
+  }
+}
+
+// block `blk` of `nblk` of the epilogue: a share of the ring row's columns, and of the appended rows
+__device__ __forceinline__ void step_epilogue_block(const StepEpilogue &e, int64_t blk, int64_t nblk) {
+  if (e.ring_line) {
+    const int64_t per = (e.Tall + nblk - 1) / nblk;
+    ring_row_columns(e, blk * per, min(e.Tall, (blk + 1) * per));
+  }
+  if (e.app_rows > 0) {   // 16-byte pieces of the appended rows, dealt over the blocks
+    const int64_t row16 = e.app_row_elems / 8;   // pieces per row (head_dim is a multiple of 32)
+    const int64_t per_side = (int64_t)e.app_bh * e.app_rows * row16;
+    for (int64_t i = blk * blockDim.x + threadIdx.x; i < 2 * per_side; i += nblk * blockDim.x) {
+      const int side = i >= per_side ? 1 : 0;
+      const int64_t j = i - side * per_side;
+      const int64_t bh = j / (e.app_rows * row16), rem = j % (e.app_rows * row16);
+      const uint4 *src = reinterpret_cast<const uint4 *>(e.app_src[side] + bh * e.app_src_slab[side]) + rem;
+      uint4 *dst = reinterpret_cast<uint4 *>(e.app_dst[side] + bh * e.app_dst_slab[side]) + rem;
+      *dst = *src;
+    }
+  }
+}
+
 // fixed-order sum over chunks: deterministic replacement for the reference's half atomics
 // (quant/csrc/gemv_cuda_wv_uniform.cu:110).  One workgroup per (b, hq) row and 128 channels; CB_SLICES
 // slices of the chunk list are summed in parallel (strided, ascending within a slice, eight requests in
-// flight per thread), then the slices in order.
+// flight per thread), then the slices in order.  Workgroups with blockIdx.z > 0 (or all of them, when there is
+// nothing to combine) run the step epilogue instead.
 __global__ __launch_bounds__(CB_CH * CB_SLICES) void pv_combine_kernel(const float *__restrict__ partial,
                                                                       half_t *__restrict__ out, int n_chunks,
-                                                                      int64_t n_bhq, int D) {
+                                                                      int64_t n_bhq, int D, StepEpilogue ep, int combine) {
+  const int z0 = combine ? 1 : 0;
+  if ((int)blockIdx.z >= z0) {
+    const int64_t per_z = (int64_t)gridDim.x * gridDim.y;
+    step_epilogue_block(ep, ((int64_t)blockIdx.z - z0) * per_z + (int64_t)blockIdx.y * gridDim.x + blockIdx.x,
+                        per_z * (gridDim.z - z0));
+    return;
+  }
   __shared__ float sh[CB_SLICES / 2][CB_CH];
   const int64_t r = blockIdx.x;
   const int d = threadIdx.x % CB_CH, sl = threadIdx.x / CB_CH;  // a wave holds two slices of the 32 channels
@@ -1993,6 +2085,9 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
       return fail(HQEKV_E_ALIGN, "%s: segment %d fp16 data must be 16-byte aligned", who, k);
     if (s.n_tokens * D >= (1LL << 31))
       return fail(HQEKV_E_UNSUPPORTED, "%s: segment %d: n_tokens * D must stay below 2^31 per (b, head) slab", who, k);
+    const bool token_major_f16 = s.bits == 16 && (is_k ? s.layout == HQEKV_LAYOUT_TOKEN_MAJOR : true);
+    if (s.slab_tokens != 0 && (s.slab_tokens < s.n_tokens || !token_major_f16))
+      return fail(HQEKV_E_ARG, "%s: segment %d: slab_tokens applies to token-major fp16 segments and must be >= n_tokens", who, k);
     SegDev &d = tb->seg[m++];
     d.data = s.data;
     d.scale = (const half_t *)s.scale;
@@ -2004,6 +2099,7 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
     d.layout = (is_k && s.bits == 16 && s.layout == HQEKV_LAYOUT_TOKEN_MAJOR) ? HQEKV_LAYOUT_TOKEN_MAJOR
                : (s.bits == 1 && s.layout == HQEKV_LAYOUT_NORMAL1)              ? HQEKV_LAYOUT_NORMAL1
                                                                                 : 0;
+    d.slab_tokens = s.slab_tokens > 0 ? s.slab_tokens : s.n_tokens;
     d.unit_begin = (int32_t)units;
     const int64_t per = (is_k && d.layout == HQEKV_LAYOUT_TOKEN_MAJOR) ? 64 : unit_tokens;
     const int64_t nu = (s.n_tokens + per - 1) / per;
@@ -2149,7 +2245,7 @@ static int64_t seg_total_tokens(const hqekv_seg *segs, int nseg) {
 
 static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, float *partial, int64_t B,
                      int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st,
-                     bool mf, int stages = 3) {
+                     bool mf, int stages = 3, const StepEpilogue *ep = nullptr) {
   const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
   if (tb.total_units > 0 && (stages & 1)) {
@@ -2172,9 +2268,20 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
     int rc = check_launch("pv_hybrid_kernel");
     if (rc) return rc;
   }
-  if (!(stages & 2) || fz.arrive) return HQEKV_OK;   // folded: the last p.V workgroups have written the output
-  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)n_bhq, (unsigned)((D + CB_CH - 1) / CB_CH)), dim3(CB_CH * CB_SLICES), 0, st, partial,
-                     (half_t *)out, (int)tb.total_units, n_bhq, (int)D);
+  const bool combine = (stages & 2) && !fz.arrive;   // folded: the last p.V workgroups have written the output
+  const bool epilogue = ep && (ep->ring_line || ep->app_rows > 0) && stages == 3;
+  if (!combine && !epilogue) return HQEKV_OK;
+  // The epilogue rides in the combine launch as extra workgroups (grid.z); one workgroup per 4096 columns of the
+  // ring row.  Without a combine (folded into p.V) the launch holds the epilogue alone.
+  const dim3 base((unsigned)n_bhq, (unsigned)((D + CB_CH - 1) / CB_CH));
+  unsigned z = combine ? 1u : 0u;
+  if (epilogue) {
+    const int64_t want = ep->ring_line ? (Tall + 4095) / 4096 : 1;
+    z += (unsigned)((want + (int64_t)base.x * base.y - 1) / ((int64_t)base.x * base.y));
+  }
+  StepEpilogue none{};
+  hipLaunchKernelGGL(pv_combine_kernel, dim3(base.x, base.y, z), dim3(CB_CH * CB_SLICES), 0, st, partial, (half_t *)out,
+                     (int)tb.total_units, n_bhq, (int)D, epilogue ? *ep : none, combine ? 1 : 0);
   return check_launch("pv_combine_kernel");
 }
 
@@ -2292,10 +2399,86 @@ extern "C" int64_t hqekv_decode_workspace_bytes(const hqekv_seg *k_segs, int n_k
   return L.total;
 }
 
+static int fill_epilogue(const hqekv_step_extra *x, const void *attn_weights, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                         int64_t Tall, StepEpilogue *e) {
+  *e = StepEpilogue{};
+  if (!x) return HQEKV_OK;
+  e->weights = (const half_t *)attn_weights;
+  e->Tall = Tall;
+  e->B = (int32_t)B;
+  e->Hq = (int32_t)Hq;
+  if (x->ring_line) {
+    if (x->ring_order != 1 && x->ring_order != 2) return fail(HQEKV_E_ARG, "decode_step: ring_order must be 1 or 2");
+    if ((uintptr_t)x->ring_line & 1) return fail(HQEKV_E_ALIGN, "decode_step: ring_line not 2-byte aligned");
+    e->ring_line = (half_t *)x->ring_line;
+    e->ring_by = x->ring_order;
+  }
+  if (x->append_rows < 0) return fail(HQEKV_E_ARG, "decode_step: negative append_rows");
+  if (x->append_rows > 0) {
+    if (!x->new_k || !x->new_v || !x->k_dst || !x->v_dst) return fail(HQEKV_E_ARG, "decode_step: append without source or destination");
+    if (x->k_dst_slab_tokens < x->append_rows || x->v_dst_slab_tokens < x->append_rows)
+      return fail(HQEKV_E_ARG, "decode_step: destination slabs shorter than the appended rows");
+    if (((uintptr_t)x->new_k | (uintptr_t)x->new_v | (uintptr_t)x->k_dst | (uintptr_t)x->v_dst) & 15)
+      return fail(HQEKV_E_ALIGN, "decode_step: appended rows and their destinations must be 16-byte aligned");
+    e->app_rows = x->append_rows;
+    e->app_row_elems = (int32_t)D;
+    e->app_bh = (int32_t)(B * Hkv);
+    e->app_src[0] = (const half_t *)x->new_k;
+    e->app_src[1] = (const half_t *)x->new_v;
+    e->app_dst[0] = (half_t *)x->k_dst;
+    e->app_dst[1] = (half_t *)x->v_dst;
+    e->app_src_slab[0] = e->app_src_slab[1] = (int64_t)x->append_rows * D;
+    e->app_dst_slab[0] = x->k_dst_slab_tokens * D;
+    e->app_dst_slab[1] = x->v_dst_slab_tokens * D;
+  }
+  return HQEKV_OK;
+}
+
+extern "C" int hqekv_ring_row(const void *attn_weights, int64_t B, int64_t Hq, int64_t Tall, void *line, int order,
+                              void *stream) {
+  if (!attn_weights || !line || B <= 0 || Hq <= 0 || Tall <= 0 || B > 0x7fffffffLL || Hq > 0x7fffffffLL)
+    return fail(HQEKV_E_ARG, "ring_row: null pointer or empty shape");
+  hqekv_step_extra x{};
+  x.ring_line = line;
+  x.ring_order = order;
+  StepEpilogue e;
+  const int rc = fill_epilogue(&x, attn_weights, B, Hq, 1, 32, Tall, &e);
+  if (rc) return rc;
+  const int64_t blocks = (Tall + 4095) / 4096;
+  if (blocks > 65535) return fail(HQEKV_E_UNSUPPORTED, "ring_row: Tall too large");
+  hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)blocks, 1, 1), dim3(CB_CH * CB_SLICES), 0, (hipStream_t)stream,
+                     (const float *)nullptr, (half_t *)nullptr, 0, (int64_t)0, 0, e, 0);
+  return check_launch("ring_row");
+}
+
+static int decode_impl(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
+                       const void *q, const void *mask, int64_t mask_row_stride, void *attn_weights,
+                       void *attn_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall,
+                       void *workspace, int64_t workspace_bytes, int flags, void *stream, const hqekv_step_extra *extra);
+
 extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
                                  const void *q, const void *mask, int64_t mask_row_stride, void *attn_weights,
                                  void *attn_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall,
                                  void *workspace, int64_t workspace_bytes, int flags, void *stream) {
+  return decode_impl(k_segs, n_k, v_segs, n_v, q, mask, mask_row_stride, attn_weights, attn_out, B, Hq, Hkv, D, Tall,
+                     workspace, workspace_bytes, flags, stream, nullptr);
+}
+
+extern "C" int hqekv_decode_step(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
+                                 const void *q, const void *mask, int64_t mask_row_stride, void *attn_weights,
+                                 void *attn_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall,
+                                 void *workspace, int64_t workspace_bytes, int flags, void *stream,
+                                 const hqekv_step_extra *extra) {
+  if (flags & (HQEKV_ONLY_QK | HQEKV_ONLY_PV | HQEKV_ONLY_COMBINE | HQEKV_ONLY_RAW_QK))
+    return fail(HQEKV_E_ARG, "decode_step: the single-stage flags belong to hqekv_decode_attn");
+  return decode_impl(k_segs, n_k, v_segs, n_v, q, mask, mask_row_stride, attn_weights, attn_out, B, Hq, Hkv, D, Tall,
+                     workspace, workspace_bytes, flags, stream, extra);
+}
+
+static int decode_impl(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
+                       const void *q, const void *mask, int64_t mask_row_stride, void *attn_weights,
+                       void *attn_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall,
+                       void *workspace, int64_t workspace_bytes, int flags, void *stream, const hqekv_step_extra *extra) {
   int rc = check_heads("decode_attn", B, Hq, Hkv, D);
   if (rc) return rc;
   if (D != 128) return fail(HQEKV_E_UNSUPPORTED, "decode_attn: head_dim %lld (supported: 128)", (long long)D);
@@ -2360,7 +2543,10 @@ extern "C" int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_s
   }
   if (only_qk) return HQEKV_OK;
   const int stages = only == HQEKV_ONLY_PV ? 1 : (only == HQEKV_ONLY_COMBINE ? 2 : 3);
-  return launch_pv(vt, L.chunk, attn_weights, attn_out, (float *)ws, B, Hq, Hkv, D, Tall, fz, st, mf, stages);
+  StepEpilogue ep;
+  rc = fill_epilogue(extra, attn_weights, B, Hq, Hkv, D, Tall, &ep);
+  if (rc) return rc;
+  return launch_pv(vt, L.chunk, attn_weights, attn_out, (float *)ws, B, Hq, Hkv, D, Tall, fz, st, mf, stages, &ep);
 }
 
 // ------------------------------------------------------------------ per-class GEMV on the same kernels

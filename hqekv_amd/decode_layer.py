@@ -20,7 +20,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .attention import SegmentMemo
+from .attention import SegmentMemo, value_length
 from .hqe_2 import KV_cache_hqe_2
 from .hqe_matmul import qkv_matmul_hqe_2
 from .public_func import get_block_token_idx, last_attn_weights, make_sum_equal
@@ -82,6 +82,9 @@ class HqeAttentionLayer:
         self.token_num = 0
         self.last_weights = last_attn_weights(last_length=last_length)
         self._memo = SegmentMemo()   # segment tables of the classes, rebuilt after each compression
+        self._res = None             # (K buffer, V buffer): the fp16 residual in capacity-sized storage
+        self.fused_step = True       # ring row and residual appends inside the attention call (False: separate launches)
+        self._own_tuple = False      # the tuple handed in carries the class tensors this layer built its tables from
 
     def reset(self) -> None:
         """What the reference's ``generate`` does per layer before a new prompt [555-557]."""
@@ -91,6 +94,7 @@ class HqeAttentionLayer:
         self.ratio_e = self.ratio_e_0.clone()
         self.last_weights.reset()
         self._memo = SegmentMemo()
+        self._res = None
 
     def set_max_length(self, max_length: int) -> None:
         """Prompt length + new tokens: the width of the importance ring [691-695]."""
@@ -112,6 +116,34 @@ class HqeAttentionLayer:
             scale=self.scaling)
         return attn_weights, attn_output
 
+    # ------------------------------------------------------------------ residual storage
+    def _residual_in_buffers(self, pkv: tuple, key_states: torch.Tensor) -> tuple:
+        """The tuple with its fp16 residual held as the head of this layer's capacity-sized buffers (B,Hkv,cap,D), so
+        that a decode step appends a row in place instead of re-allocating ``cat(residual, k)`` [131-133].  A residual
+        that is not there yet -- after the prompt, after a compression, or a tuple from elsewhere -- is copied in
+        once; the fields of the tuple are views of the same shape and content as the reference's tensors."""
+        res_K, res_V = pkv[-3], pkv[-2]
+        B, H, L, D = key_states.shape
+        n = res_K.shape[2] if res_K is not None else 0
+        buf = self._res
+        held = self._memo.held
+        self._own_tuple = held is not None and all(a is b for a, b in zip(held, pkv))
+        fits = (buf is not None and buf[0].shape[0] == B and buf[0].shape[1] == H and buf[0].shape[3] == D
+                and buf[0].device == key_states.device and buf[0].dtype == key_states.dtype and n + L <= buf[0].shape[2])
+        if fits and (n == 0 or (res_K.data_ptr() == buf[0].data_ptr() and res_V.data_ptr() == buf[1].data_ptr()
+                                and res_K.stride() == buf[0].stride() and res_V.stride() == buf[1].stride())):
+            return pkv
+        cap = max(2 * BLOCK, (n + L + BLOCK - 1) // BLOCK * BLOCK + BLOCK)
+        kb = torch.empty(B, H, cap, D, dtype=key_states.dtype, device=key_states.device)
+        vb = torch.empty_like(kb)
+        if n:
+            kb[:, :, :n].copy_(res_K)
+            vb[:, :, :n].copy_(res_V)
+        self._res = (kb, vb)
+        if n == 0:
+            return pkv
+        return pkv[:-3] + (kb[:, :, :n], vb[:, :, :n], pkv[-1])
+
     # ------------------------------------------------------------------ one call
     def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
                 attention_mask: Optional[torch.Tensor] = None, past_key_value: Optional[tuple] = None,
@@ -125,12 +157,40 @@ class HqeAttentionLayer:
             # The attention reads this step's key and value where they are, as a segment behind the residual, and
             # is queued first; the copies that append them to the residual [131-133] follow it on the stream, off
             # the step's critical path.
-            attn_weights, attn_output = qkv_matmul_hqe_2(query_states, past_key_value, attention_mask,
-                                                         self.head_dim, self.quant_strategy, memo=self._memo,
-                                                         tail=(key_states, value_states))
-            self.last_weights.update(attn_weights)
-            new_K = torch.cat((past_key_value[-3], key_states), dim=2) if past_key_value[-3] is not None else key_states
-            new_V = torch.cat((past_key_value[-2], value_states), dim=2) if past_key_value[-2] is not None else value_states
+            past_key_value = self._residual_in_buffers(past_key_value, key_states)
+            n = past_key_value[-3].shape[2] if past_key_value[-3] is not None else 0
+            # tokens the classes hold = the history this layer has kept; a tuple from elsewhere is counted
+            Tall = (self.history_reserve_length if self._own_tuple else value_length(past_key_value) - n) + n + L
+            lw = self.last_weights
+            # shapes for which the ring row's summation order is pinned against torch's on the device
+            on_device = (self.fused_step and L == 1 and Tall >= 256 and query_states.shape[1] == 32
+                         and query_states.shape[0] <= 8 and query_states.dtype == torch.float16
+                         and (lw.weights is None or lw.weights.dtype == torch.float16) and lw.max_length >= Tall)
+            plain_inputs = (self.fused_step and attention_mask is None and query_states.shape[2] == 1
+                            and query_states.is_contiguous() and key_states.is_contiguous() and value_states.is_contiguous()
+                            and query_states.dtype == torch.float16 and query_states.is_cuda
+                            and self.quant_strategy in ("uniform_group", "high_uniform_group_low_normal_group"))
+            if plain_inputs:
+                # One call: attention, the ring row (in torch's own summation order) and the two residual appends
+                # [131-133, 200]; the kernels read this step's key and value where they are, as a segment behind the
+                # residual, and copy them into the residual buffers in the call's last launch.
+                if on_device and lw.weights is None:
+                    lw.decode_row(query_states, Tall)   # creates the store
+                attn_weights, attn_output = self._memo.step_call(
+                    query_states, past_key_value, Tall, key_states, value_states, self._res, n,
+                    lw.weights if on_device else None, lw.next_line, self.quant_strategy == "uniform_group")
+            else:
+                attn_weights, attn_output = qkv_matmul_hqe_2(query_states, past_key_value, attention_mask,
+                                                             self.head_dim, self.quant_strategy, memo=self._memo,
+                                                             tail=(key_states, value_states))
+            if plain_inputs and on_device:
+                lw.advance(Tall)
+            else:
+                lw.update(attn_weights)
+            if not plain_inputs:   # the plain sequence of the reference: two copies after the attention
+                self._res[0][:, :, n:n + L].copy_(key_states)
+                self._res[1][:, :, n:n + L].copy_(value_states)
+            new_K, new_V = self._res[0][:, :, :n + L], self._res[1][:, :, :n + L]
             past_key_value = past_key_value[:-3] + (new_K, new_V, kv_seq_len)
         else:
             attn_weights, attn_output = self._prefill(query_states, key_states, value_states, attention_mask)

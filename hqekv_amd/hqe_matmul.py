@@ -13,11 +13,12 @@ from .attention import decode_attention, value_length
 
 
 def qkv_matmul_hqe_2(q: torch.Tensor, past_key_value: Tuple, attention_mask, head_dim: int,
-                     quant_strategy: str, block_size: int = 32, group_size: int = 32, memo=None, tail=None):
+                     quant_strategy: str, block_size: int = 32, group_size: int = 32, memo=None, tail=None, step=None):
     """-> (attn_weights (B,Hq,1,real_len) fp16, attn_output (B,Hq,1,D) fp16).
     Not in the reference's signature, both optional: ``memo``, an ``attention.SegmentMemo`` kept per layer, and
     ``tail`` = (k, v), the step's new key and value rows (B,Hkv,L,D) when the caller has not appended them to the
-    tuple's residual yet; they count into ``real_len``."""
+    tuple's residual yet; they count into ``real_len``; ``step``: the ring row and the residual appends of the
+    caller's decode step, folded into the call (``attention.decode_attention``)."""
     if quant_strategy not in ("uniform_group", "high_uniform_group_low_normal_group"):
         # upstream accepts only these two here (quant/hqe_matmul.py:370-377)
         raise ValueError('invalid quant_strategy')
@@ -27,7 +28,7 @@ def qkv_matmul_hqe_2(q: torch.Tensor, past_key_value: Tuple, attention_mask, hea
     if real_len == 0:
         raise ValueError('invalid past_key_value')
     return decode_attention(q, past_key_value, None, real_len, zero_init=False,
-                            low_uniform=quant_strategy == "uniform_group", memo=memo, tail=tail)
+                            low_uniform=quant_strategy == "uniform_group", memo=memo, tail=tail, step=step)
 
 
 def qkv_matmul_hqe(q: torch.Tensor, past_key_value: Tuple, attention_mask, head_dim: int,

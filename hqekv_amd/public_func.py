@@ -112,6 +112,18 @@ class last_attn_weights:
         kept = torch.index_select(self.weights, 1, reserve_idx)
         self.weights.narrow(1, 0, kept.shape[1]).copy_(kept)
 
+    def decode_row(self, like: torch.Tensor, T: int) -> torch.Tensor:
+        """The (T,) slot the next decode row belongs in, for a caller that has the row written by the kernels
+        (``hqekv_decode_step`` / ``hqekv_ring_row``) instead of calling ``update``; follow it with ``advance(T)``."""
+        if self.weights is None:
+            self.weights = like.new_zeros(self.last_length, self.max_length)
+        return self.weights[self.next_line, :T]
+
+    def advance(self, T: int) -> None:
+        """Bookkeeping of ``update`` for one decode row that has been written in place."""
+        self.kv_seq_len = T
+        self.next_line = (self.next_line + 1) % self.last_length
+
     def update(self, attn_weights: torch.Tensor) -> None:
         """attn_weights (B, H, L, T): a prompt (L > 1) stores its last rows, a decode step (L == 1) one ring row.
         The sums run over the batch first and over the heads second, each rounded to the store's dtype."""
@@ -123,6 +135,19 @@ class last_attn_weights:
             self.weights[:rows, :T] = attn_weights[:, :, L - rows:, :].sum(0).sum(0)
         else:
             rows = 1
+            if attn_weights.is_cuda and self.weights.dtype == attn_weights.dtype:
+                from .attention import ring_order, ring_row_on_device_applies
+                if ring_row_on_device_applies(attn_weights):
+                    # one launch for any batch size, in the order torch's own reduction adds the rows
+                    from . import _lib
+                    line = self.weights[self.next_line, :T]
+                    with _lib.on_device(attn_weights.device):
+                        rc = _lib.load().hqekv_ring_row(attn_weights.data_ptr(), attn_weights.shape[0], attn_weights.shape[1], T,
+                                                        line.data_ptr(), ring_order(T, attn_weights),
+                                                        _lib.stream_ptr(attn_weights.device))
+                    _lib.check(rc, "ring_row")
+                    self.advance(T)
+                    return
             per_head = attn_weights[0] if attn_weights.shape[0] == 1 else attn_weights.sum(0)
             line = self.weights[self.next_line:self.next_line + 1, :T]
             if line.dtype == per_head.dtype:

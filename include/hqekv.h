@@ -183,6 +183,9 @@ typedef struct hqekv_seg {
   const void *scale;     /* NULL when bits == 16                                       */
   const void *zero;
   const int64_t *idx;    /* (n_tokens) or NULL                                         */
+  int64_t slab_tokens;   /* token-major fp16 segments only (the residual, the fp16 V class): token rows between two
+                            (b, kv head) slabs in memory when the segment is the head of a longer, capacity-sized
+                            buffer; 0 = n_tokens (dense)                                */
 } hqekv_seg;
 
 /* Replaces gemv_forward_cuda_qk_group_hq (quant/csrc/gemv_cuda.h:78-109; kernel
@@ -275,6 +278,39 @@ int hqekv_decode_attn(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs,
                       void *attn_weights, void *attn_out, int64_t B, int64_t Hq, int64_t Hkv,
                       int64_t D, int64_t Tall, void *workspace, int64_t workspace_bytes, int flags,
                       void *stream);
+
+/* The decode step of the reference's attention layer as ONE call: hqekv_decode_attn plus what the layer does around it
+ * on every generated token (model/llama_hqe.py:131-136, 200) --
+ *   new_K = cat(residual, k), new_V = cat(residual, v)     two rows copied behind the residual, which the caller keeps
+ *                                                          in capacity-sized buffers (see hqekv_seg.slab_tokens)
+ *   last_weights.update(attn_weights)                      one row of the importance ring:
+ *                                                          attn_weights.sum(0).sum(0), model/public_func.py:243-257
+ * -- folded into the call's last launch (extra workgroups of the split-K combine, or a launch of their own when the
+ * combine runs inside p.V).  The ring row follows the order in which torch's GPU reduction adds the rows (fp32
+ * accumulation, one rounding to fp16 per reduction): ring_order is the number of threads that reduction deals the
+ * head rows to for the shape at hand -- 2 when Tall is a multiple of 4, at least 256, and attn_weights is 8-byte
+ * aligned; else 1 -- pinned against torch.sum on the device for 32 heads and batch sizes 1..8.
+ * The appended rows are not read by this call's attention: the caller names this step's key and value as segments of
+ * their own.  `extra` may be NULL (then the call is hqekv_decode_attn); single-stage flags are refused.
+ */
+typedef struct hqekv_step_extra {
+  void *ring_line;             /* (Tall) fp16, any 2-byte alignment; NULL = no ring row                    */
+  int32_t ring_order;          /* 1 or 2, see above                                                        */
+  int32_t append_rows;         /* token rows of new_k / new_v per (b, kv head); 0 = nothing to append      */
+  const void *new_k, *new_v;   /* (B,Hkv,append_rows,D) fp16, dense, 16-byte aligned                       */
+  void *k_dst, *v_dst;         /* where slab 0's first appended row goes (16-byte aligned)                 */
+  int64_t k_dst_slab_tokens;   /* token rows between two (b, kv head) slabs of the destination buffers     */
+  int64_t v_dst_slab_tokens;
+} hqekv_step_extra;
+int hqekv_decode_step(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs, int n_v,
+                      const void *q, const void *mask, int64_t mask_row_stride,
+                      void *attn_weights, void *attn_out, int64_t B, int64_t Hq, int64_t Hkv,
+                      int64_t D, int64_t Tall, void *workspace, int64_t workspace_bytes, int flags,
+                      void *stream, const hqekv_step_extra *extra);
+/* The ring row alone: line[t] = rnd16(sum_h rnd16(sum_b attn_weights[b,h,t])) in torch's order (`order` as
+ * ring_order above).  Replaces last_attn_weights.update for one decode row (model/public_func.py:250-254). */
+int hqekv_ring_row(const void *attn_weights, int64_t B, int64_t Hq, int64_t Tall, void *line, int order,
+                   void *stream);
 
 /* ------------------------------------------------------------------ cache maintenance (one launch per side)
  * Replaces the per-(source, target) gathers, dequantise / re-quantise calls and torch.cat re-copies of one

@@ -1,0 +1,113 @@
+"""The importance ring's decode row on the device (hqekv_ring_row, and the same code inside hqekv_decode_step) against
+torch's own ``attn_weights.sum(0).sum(0)`` executed on the GPU, bit for bit -- the row's last place decides block
+rankings (model/public_func.py:92-106, 243-257), so the kernels follow the order in which torch's reduction adds the
+rows.  Shapes: 32 heads, batch 1..8, rows from 256 tokens up, every residue of the length modulo 4, aligned and
+unaligned slots of the ring store."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _order_sensitive(B, H, T, g):
+    """Small values everywhere plus, in every column, big values that cancel exactly in pairs: what is left depends on
+    which small values met a big partial sum before its partner arrived -- any other order of additions shows."""
+    m = torch.randint(1024, 2048, (B * H, T), generator=g).float() / 1024.0
+    e = torch.randint(8, 15, (B * H, T), generator=g).float()
+    X = m * torch.exp2(-e)
+    order = torch.rand(B * H, T, generator=g).argsort(0)
+    cols = torch.arange(T)
+    for k in range(max(1, B * H // 8)):
+        big = (torch.randint(1024, 2048, (T,), generator=g).float() / 1024.0) * 1024.0
+        X[order[2 * k], cols] = big
+        X[order[2 * k + 1], cols] = -big
+    return X.half().view(B, H, 1, T)
+
+
+def _probabilities(B, H, T, g):
+    return torch.softmax(torch.randn(B, H, 1, T, generator=g) * 4.0, dim=-1).half()
+
+
+@pytest.mark.parametrize("B", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("kind", ["order_sensitive", "probabilities"])
+def test_ring_row_equals_torch_sum_on_device(dev, B, kind):
+    from hqekv_amd import _lib
+    from hqekv_amd.attention import ring_order, ring_row_on_device_applies
+    H = 32
+    g = torch.Generator().manual_seed(100 * B + len(kind))
+    lib = _lib.load()
+    for T in (256, 257, 258, 259, 260, 1000, 1023, 4096, 4099, 8200, 26208, 26209, 26210, 26211, 52449, 104864):
+        w = (_order_sensitive if kind == "order_sensitive" else _probabilities)(B, H, T, g).to(dev)
+        assert ring_row_on_device_applies(w)
+        expect = w.sum(0).sum(0).reshape(T)                       # torch's own reductions, on the device
+        for max_len, row in ((T + 8, 0), (T + 9, 1), (T + 10, 3), (T + 11, 7)):   # slots of every alignment
+            store = torch.full((20, max_len), -5.0, dtype=torch.float16, device=dev)
+            line = store[row, :T]
+            rc = lib.hqekv_ring_row(w.data_ptr(), B, H, T, line.data_ptr(), ring_order(T, w), _lib.stream_ptr(dev))
+            _lib.check(rc, "ring_row")
+            torch.cuda.synchronize()
+            assert torch.equal(line.view(torch.int16), expect.view(torch.int16)), (B, T, max_len, row)
+            assert bool((store[row, T:] == -5.0).all()) and bool((store[row - 1] == -5.0).all())   # nothing else written
+    # the class that keeps the ring takes this route for such rows, and torch's for the others
+    from hqekv_amd.public_func import last_attn_weights
+    ring = last_attn_weights()
+    ring.set_max_length(5000)
+    for T in (100, 255, 256, 4099):
+        w = _probabilities(B, H, T, g).to(dev)
+        slot = ring.next_line
+        ring.update(w)
+        assert torch.equal(ring.weights[slot, :T].view(torch.int16), w.sum(0).sum(0).reshape(T).view(torch.int16)), T
+
+
+def test_ring_row_rejects_bad_arguments(dev):
+    from hqekv_amd import _lib
+    lib = _lib.load()
+    w = torch.zeros(1, 32, 1, 256, dtype=torch.float16, device=dev)
+    line = torch.zeros(256, dtype=torch.float16, device=dev)
+    assert lib.hqekv_ring_row(w.data_ptr(), 1, 32, 256, line.data_ptr(), 3, None) == -1
+    assert lib.hqekv_ring_row(None, 1, 32, 256, line.data_ptr(), 1, None) == -1
+    assert lib.hqekv_ring_row(w.data_ptr(), 1, 32, 0, line.data_ptr(), 1, None) == -1
+
+
+@pytest.mark.parametrize("B,T0", [(1, 300), (2, 257), (4, 512)])
+def test_layer_step_in_one_call_equals_the_separate_launches(dev, B, T0):
+    """Two layers in lockstep over a prompt and 70 decode steps (two compressions): one runs a decode step as ONE call
+    (attention + ring row + residual appends, hqekv_decode_step), the other as the reference's sequence of separate
+    operations.  Every field of the cache tuples, the ring stores, the probabilities and the outputs are identical
+    bit for bit, and each ring row equals torch's own attn_weights.sum(0).sum(0) on the device."""
+    from hqekv_amd.decode_layer import HqeAttentionLayer
+    Hq, Hkv, D, steps = 32, 8, 128, 70
+    ratios = dict(bit_0=0.2, bit_4=0.3, bit_2=0.5, bit_1=0.0)
+    one, sep = HqeAttentionLayer(D, **ratios), HqeAttentionLayer(D, **ratios)
+    sep.fused_step = False
+    for l in (one, sep):
+        l.set_max_length(T0 + steps)
+    g = torch.Generator().manual_seed(7 + B)
+    pkv1 = pkv2 = None
+    compressions = 0
+    for step in range(steps + 1):
+        L = T0 if step == 0 else 1
+        q = torch.randn(B, Hq, L, D, generator=g).half().to(dev)
+        k = torch.randn(B, Hkv, L, D, generator=g).half().to(dev)
+        v = torch.randn(B, Hkv, L, D, generator=g).half().to(dev)
+        mask = None
+        if step == 0:
+            mask = torch.triu(torch.full((T0, T0), torch.finfo(torch.float16).min, dtype=torch.float16), diagonal=1)[None, None].to(dev)
+        slot = one.last_weights.next_line
+        o1, w1, pkv1, aux1 = one(q, k, v, mask, pkv1, None)
+        o2, w2, pkv2, aux2 = sep(q, k, v, mask, pkv2, None)
+        where = f"step {step}"
+        assert torch.equal(w1, w2) and torch.equal(o1, o2), where
+        if step and aux1 is None:   # (a compression moves the ring's columns afterwards)
+            T = w1.shape[-1]
+            assert torch.equal(one.last_weights.weights[slot, :T].view(torch.int16),
+                               w1.sum(0).sum(0).reshape(T).view(torch.int16)), where
+        assert torch.equal(one.last_weights.weights.view(torch.int16), sep.last_weights.weights.view(torch.int16)), where
+        assert (aux1 is None) == (aux2 is None), where
+        compressions += aux1 is not None
+        for i, (a, b) in enumerate(zip(pkv1, pkv2)):
+            if torch.is_tensor(a):
+                assert a.shape == b.shape and torch.equal(a, b), (where, i)
+            else:
+                assert a == b, (where, i)
+    assert compressions >= 2
