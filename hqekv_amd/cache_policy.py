@@ -15,7 +15,8 @@ survivors (quant/hqe_2.py:661-670).
 
 Two engines produce the same bytes.  ``gather`` (the default wherever it applies): everything the reference
 moves is a whole block of 32 tokens and every block ends in exactly one place, so the host works out, per
-block, where each class's blocks come from (numpy over a few thousand entries), and ONE kernel launch per side
+block, where each class's blocks come from (``hqekv_plan_side``, the library's host-side planner: one C call
+per side over a few thousand entries), and ONE kernel launch per side
 (``hqekv_cache_migrate``) rebuilds all classes from the old ones and the new tokens -- survivors copied, demoted
 blocks dequantised and re-quantised, new blocks quantised, evicted blocks left out, positions re-ranked; the
 device is waited for once, to fetch the two block rankings.  ``steps``: the general engine for selections that
@@ -382,54 +383,38 @@ def _migrate(side: Dict[int, _Cls], new: torch.Tensor, targets: List[Optional[np
 _SRC_NEW = 5   # source slot of the new fp16 tokens (slots 0..4: the old fp16, 8, 4, 2, 1-bit classes)
 
 
-def _block_labels(sorted_idx: torch.Tensor, bit_num, total_blocks: int, order_h: Optional[np.ndarray]) -> Optional[np.ndarray]:
-    """label[b] = index of the target (fp16, 8, 4, 2, 1[, evict]) block b is ranked into, or None when the ranking
-    or the counts are not made of whole blocks covering every block once."""
-    counts = [int(v) for v in (bit_num.tolist() if torch.is_tensor(bit_num) else bit_num)]
-    if any(c % BLOCK or c < 0 for c in counts) or sum(counts) != total_blocks * BLOCK:
-        return None
-    if order_h is None:
-        order_h = _host_blocks(sorted_idx)
-    if order_h is None or order_h.shape[0] != total_blocks:
-        return None
-    label = np.full(total_blocks, -1, dtype=np.int8)
-    start = 0
-    for ti, c in enumerate(counts):
-        nb = c // BLOCK
-        label[order_h[start:start + nb]] = ti
-        start += nb
-    if (label < 0).any():   # a block ranked twice and another one never
-        return None
-    return label
-
-
-def _plan_side(old_blocks: Dict[int, np.ndarray], hist_blocks: int, n_new_blocks: int, label: np.ndarray):
-    """-> (blocks per new class (5,), source slot / source block / old position of every new block, all classes
-    back to back in class order).
-
-    Normative order inside a class (quant/hqe_2.py:552-659): the members that stay, in their order; then the new
-    tokens ranked into it; then what comes down from the fp16, 8, 4 and 2-bit classes, each in source order.  A
-    block only ever moves to a lower precision; a block ranked into a higher one stays where it is.  With the
-    classes numbered 0..4 from fp16 down, evicted = 5 and a new block's own class taken as -1, a block lands in
-    max(own class, ranked class); one three-key sort over all blocks (class, origin, place in the source) lays
-    every class out in that order."""
+def _plan_side_c(old_blocks: Dict[int, np.ndarray], hist_blocks: int, n_new_blocks: int, order_h: np.ndarray, bit_num):
+    """The block-level plan of one side from the library's host-side planner (``hqekv_plan_side``): which new class
+    every block lands in, in which order, and its new position.  -> (blocks per new class (5,), plan words -- source entries then
+    new block numbers, ready for the kernel --, surviving old block numbers ascending, or None when nothing was
+    evicted), or None when the ranking or the counts are not made of whole blocks covering every block once."""
+    from . import _lib
+    import ctypes as C
     total = hist_blocks + n_new_blocks
-    cls_of = np.empty(total, dtype=np.int64)     # class a block is in now (5: the new tokens)
-    idx_in = np.empty(total, dtype=np.int64)     # its place inside that class
+    counts_t = [int(v) for v in (bit_num.tolist() if torch.is_tensor(bit_num) else bit_num)]
+    if order_h is None or order_h.shape[0] != total:
+        return None
+    order64 = np.ascontiguousarray(order_h, dtype=np.int64)
+    ptrs = (C.c_void_p * 5)()
+    cnts = (C.c_int32 * 5)()
+    hold = []
     for ci, bits in enumerate(CLASS_BITS):
         b = old_blocks.get(bits)
         if b is not None and b.size:
-            cls_of[b] = ci
-            idx_in[b] = np.arange(b.size)
-    cls_of[hist_blocks:] = _SRC_NEW
-    idx_in[hist_blocks:] = np.arange(n_new_blocks)
-    own = np.where(cls_of == _SRC_NEW, -1, cls_of)
-    dest = np.maximum(own, label)
-    origin = np.where(own == dest, 0, own + 2)   # stays: 0; new: 1; moved down from class c: c + 2
-    order = np.lexsort((idx_in, origin, dest))
-    counts = np.bincount(dest, minlength=6)
-    order = order[:total - counts[5]]            # the evicted blocks sort last
-    return counts[:5], cls_of[order], idx_in[order], order
+            b32 = np.ascontiguousarray(b, dtype=np.int32)
+            hold.append(b32)
+            ptrs[ci], cnts[ci] = b32.ctypes.data, b32.size
+    targets = (C.c_int64 * len(counts_t))(*counts_t)
+    counts = np.empty(5, dtype=np.int32)
+    plan = np.empty(2 * total + 2, dtype=np.int32)
+    alive = np.empty(max(total, 1), dtype=np.int32)
+    n_alive = C.c_int32(0)
+    rc = _lib.load().hqekv_plan_side(ptrs, cnts, hist_blocks, n_new_blocks, order64.ctypes.data, targets, len(counts_t),
+                                     counts.ctypes.data, plan.ctypes.data, alive.ctypes.data, C.byref(n_alive))
+    if rc:
+        return None
+    u = n_alive.value
+    return counts, plan[:2 * u], (alive[:u].astype(np.int64) if u < total else None)
 
 
 _CLASS_SHAPES_K = {b: (lambda B, H, D, n, b=b: [(B, H, D, n)] if b == 16 else [(B, H, D, n * b // 32), (B, H, D, n // 32), (B, H, D, n // 32)]) for b in CLASS_BITS}
@@ -443,11 +428,13 @@ def _numel(shape) -> int:
     return n
 
 
-def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, counts, slots, srcs, pos,
+def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, counts, plan_words: np.ndarray,
                  strategy: str) -> Dict[int, _Cls]:
     """Allocate the new classes of one side (one buffer per element type, the tensors are views of it) and fill
-    them with one launch of the migration kernel.  ``slots`` / ``srcs`` / ``pos``: source slot, source block and
-    new block number of every new block, the classes back to back."""
+    them with one launch of the migration kernel.  ``plan_words`` (int32): per new block, the classes back to
+    back, (source slot << 24) | source block, then every block's new block number."""
+    nb = plan_words.size // 2
+    pos = plan_words[nb:].astype(np.int64)
     from . import _lib
     B, H, n_new, D = new.shape
     dev = new.device
@@ -534,11 +521,7 @@ def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, counts, s
         idx_t._hq_host_version = idx_t._version
         blk0 += n // BLOCK
         out[bits] = _Cls(data, idx_t, sc, zr)
-    nb = slots.size
-    plan_h = np.empty(2 * nb + (2 * nb) % 2 + 2, dtype=np.int32)
-    plan_h[:nb] = (slots << 24) | srcs
-    plan_h[nb:2 * nb] = pos
-    plan = _to_dev(plan_h[:(2 * nb + 1) // 2 * 2].view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
+    plan = _to_dev(np.ascontiguousarray(plan_words).view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
     with _lib.on_device(dev):
         # (no status word: this plan was made a few lines up from the classes it names; the kernel still checks it)
         rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src, _SRC_NEW + 1, dst, n_dst, plan.data_ptr(), B * H, D,
@@ -588,23 +571,19 @@ def _compress_gather(pkv: tuple, new_K, new_V, res_K, res_V, history: int, compr
         k_order_h, v_order_h = both[0], both[1]
     elif v_ord is not None and v_ord[0].numel() == total_blocks:
         v_order_h = v_ord[0].to("cpu", torch.int64).numpy()
-    k_label = _block_labels(K_sorted_idx, K_bit_num, total_blocks, k_order_h)
-    v_label = _block_labels(V_sorted_idx, V_bit_num, total_blocks, v_order_h)
-    if k_label is None or v_label is None:
+    if k_order_h is None:
+        k_order_h = _host_blocks(K_sorted_idx)
+    if v_order_h is None:
+        v_order_h = _host_blocks(V_sorted_idx)
+    k_plan = _plan_side_c(old["k"], hist_blocks, n_new_blocks, k_order_h, K_bit_num)
+    v_plan = _plan_side_c(old["v"], hist_blocks, n_new_blocks, v_order_h, V_bit_num)
+    if k_plan is None or v_plan is None:
         return None
     dev = new_V.device
     sides = {}
-    for name, is_k, side, new, label in (("k", True, k_side, new_K, k_label), ("v", False, v_side, new_V, v_label)):
-        counts, slots, srcs, old_pos = _plan_side(old[name], hist_blocks, n_new_blocks, label)
-        pos = old_pos
-        evicted = old_pos.size < total_blocks
-        if evicted:   # survivors keep their order; a block's new number is its rank among them
-            alive = np.sort(old_pos)
-            rank_of = np.empty(total_blocks, dtype=np.int64)
-            rank_of[alive] = np.arange(alive.size)
-            pos = rank_of[old_pos]
-        sides[name] = _gather_side(is_k, side, new, counts, slots, srcs, pos, strategy)
-        if name == "v" and evicted:
+    for name, is_k, side, new, (counts, words, alive) in (("k", True, k_side, new_K, k_plan), ("v", False, v_side, new_V, v_plan)):
+        sides[name] = _gather_side(is_k, side, new, counts, words, strategy)
+        if name == "v" and alive is not None:   # evicted tokens leave the token ranges and the ring as well
             keep_tok = (alive[:, None] * BLOCK + np.arange(BLOCK, dtype=np.int64)).reshape(-1)
             keep_t = _to_dev(keep_tok, dev)
             V_norm = V_norm[keep_t]

@@ -11,8 +11,9 @@ Per call (model/llama_hqe.py, line numbers in brackets):
             update for the next 32-token increment [233-239].
 
 Decode attention, quantisation, demotion and eviction run on the HIP kernels of this package.  The prompt
-attention (outside the quantised path) uses torch: ``scaled_dot_product_attention`` for the output and a
-matmul for the last 20 rows of probabilities, the only rows the ring keeps [146-170].
+attention (outside the quantised path) uses torch: ``scaled_dot_product_attention`` with grouped query heads for
+the output and one batched matmul for the last 20 rows of probabilities, the only rows the ring keeps [146-170];
+neither materialises ``repeat_kv`` copies of K or V.
 """
 from __future__ import annotations
 
@@ -34,6 +35,26 @@ def _repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
         return x
     B, H, T, D = x.shape
     return x[:, :, None, :, :].expand(B, H, n_rep, T, D).reshape(B, H * n_rep, T, D)
+
+
+_GQA_SDPA = [True]   # torch's fused attention takes grouped query heads directly (no repeat_kv copies) until it says no
+
+
+def gqa_prompt_attention(q, k, v, attention_mask, scaling):
+    """softmax(q k^T * scaling + mask) v over a whole prompt with grouped query heads, through torch's fused attention
+    (the prompt is outside the quantised path; the reference calls flash-attention here, model/llama_hqe.py:146-154).
+    K and V are handed over as they are, (B,Hkv,T,D); only when the fused kernel refuses grouped heads are they
+    expanded."""
+    n_rep = q.shape[1] // k.shape[1]
+    causal = attention_mask is None and k.shape[-2] > 1
+    if n_rep > 1 and _GQA_SDPA[0]:
+        try:
+            return torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=attention_mask, is_causal=causal,
+                                                                    scale=scaling, enable_gqa=True)
+        except (TypeError, RuntimeError):
+            _GQA_SDPA[0] = False
+    return torch.nn.functional.scaled_dot_product_attention(q, _repeat_kv(k, n_rep), _repeat_kv(v, n_rep),
+                                                            attn_mask=attention_mask, is_causal=causal, scale=scaling)
 
 
 def class_token_counts(total_length: int, ratio_q: torch.Tensor, ratio_e: torch.Tensor):
@@ -102,18 +123,20 @@ class HqeAttentionLayer:
 
     # ------------------------------------------------------------------ prompt
     def _prefill(self, q, k, v, attention_mask):
-        n_rep = q.shape[1] // k.shape[1]
-        T = k.shape[-2]
+        """Prompt attention [141-188]: the output over all rows, and the probabilities of the last 20 rows only (what
+        the ring keeps).  K and V are read once per KV head: the query heads that share a KV head are folded into the
+        row dimension of one batched product instead of materialising ``repeat_kv`` copies of K and V."""
+        B, Hq, T, D = q.shape
+        Hkv = k.shape[1]
+        n_rep = Hq // Hkv
         rows = min(T, LAST_TOKEN_NUM)
-        kr = _repeat_kv(k, n_rep)
-        w = torch.matmul(q[:, :, -rows:, :], kr.transpose(2, 3)) * self.scaling
+        q_last = q[:, :, T - rows:, :].reshape(B, Hkv, n_rep * rows, D)          # (b, kv head, [rep, row], d)
+        w = (torch.matmul(q_last, k.transpose(2, 3)) * self.scaling).view(B, Hq, rows, T)
         if attention_mask is not None:
             w = w + attention_mask[:, :, -rows:, :]
             w = torch.max(w, torch.tensor(torch.finfo(w.dtype).min, dtype=w.dtype, device=w.device))
         attn_weights = torch.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
-        attn_output = torch.nn.functional.scaled_dot_product_attention(
-            q, kr, _repeat_kv(v, n_rep), attn_mask=attention_mask, is_causal=attention_mask is None and T > 1,
-            scale=self.scaling)
+        attn_output = gqa_prompt_attention(q, k, v, attention_mask, self.scaling)
         return attn_weights, attn_output
 
     # ------------------------------------------------------------------ residual storage

@@ -21,14 +21,8 @@ import torch
 
 from . import _lib
 from .attention import K_BASE, NEW_K, NEW_V, V_BASE, SegmentMemo, decode_attention, default_flags
+from .decode_layer import gqa_prompt_attention
 from .pack_unpack import uniform_group_quantize_pack_last_dim
-
-
-def _repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
-    if n_rep == 1:
-        return x
-    B, H, T, D = x.shape
-    return x[:, :, None, :, :].expand(B, H, n_rep, T, D).reshape(B, H * n_rep, T, D)
 
 
 class KiviAttentionLayer:
@@ -55,9 +49,7 @@ class KiviAttentionLayer:
     def _prefill(self, q, k, v, attention_mask):
         n_rep = q.shape[1] // k.shape[1]
         T, R = k.shape[-2], self.residual_length
-        out = torch.nn.functional.scaled_dot_product_attention(
-            q, _repeat_kv(k, n_rep), _repeat_kv(v, n_rep), attn_mask=attention_mask,
-            is_causal=attention_mask is None and T > 1, scale=self.scaling)
+        out = gqa_prompt_attention(q, k, v, attention_mask, self.scaling)   # grouped heads: no repeat_kv copies
         tail = T % R
         k_quant = k if tail == 0 else (k[:, :, :T - tail, :] if T >= R else None)
         k_full = None if tail == 0 else k[:, :, T - tail:, :].contiguous()

@@ -346,6 +346,27 @@ typedef struct hqekv_cache_class {
 int hqekv_cache_migrate(int is_k, const hqekv_cache_class *src, int n_src, const hqekv_cache_class *dst,
                         int n_dst, const int32_t *plan, int64_t BH, int64_t D, int32_t *status, void *stream);
 
+/* The plan for hqekv_cache_migrate, worked out on the HOST (every pointer here is a host pointer; nothing is launched).
+ * Replaces the class-by-class selection of one compression (quant/hqe_2.py:552-659 for K, :672-836 for V: torch.isin
+ * masks per (source, target) pair) and the re-ranking of the positions after an eviction (:661-670) by their outcome.
+ *   old_blocks[c], old_counts[c]  c = 0..4 (fp16, 8, 4, 2, 1 bit): block numbers (first position / 32) of class c's
+ *                                 blocks in stored order; together they are 0 .. hist_blocks-1
+ *   n_new_blocks                  blocks of new fp16 tokens; they are numbered hist_blocks ..
+ *   order                         all hist_blocks + n_new_blocks block numbers, most important first
+ *   target_tokens[n_targets]      tokens the ranking is cut into: fp16, 8, 4, 2, 1 bit [, evicted]; multiples of 32
+ * A block moves only to a lower precision (ranked higher, it stays); inside a new class: the members that stay, the
+ * new tokens, then what comes down from fp16, 8, 4, 2 bit, each in source order.
+ *   counts_out[5]                 blocks of every new class
+ *   plan_out[2 * total]           room for every block; filled: per new block (n_alive of them, classes back to
+ *                                 back) (source slot << 24) | block inside the source (slot 5 = the new tokens), then
+ *                                 -- from plan_out[n_alive] on -- its new block number (its rank among the survivors):
+ *                                 the 2 * n_alive words hqekv_cache_migrate reads
+ *   alive_out[total], n_alive_out the surviving blocks' old numbers, ascending
+ */
+int hqekv_plan_side(const int32_t *const *old_blocks, const int32_t *old_counts, int32_t hist_blocks,
+                    int32_t n_new_blocks, const int64_t *order, const int64_t *target_tokens, int32_t n_targets,
+                    int32_t *counts_out, int32_t *plan_out, int32_t *alive_out, int32_t *n_alive_out);
+
 /* No counterpart in the reference: hqekv_decode_attn for callers that cannot allocate (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  Same arguments minus the workspace: the split-K
  * partials and softmax statistics go to a fixed buffer of HQEKV_STATIC_SCRATCH_BYTES inside the library's device

@@ -110,19 +110,27 @@ def test_oracle_policy_invariants_every_step():
 
 
 def test_block_planner_against_the_move_sequence_by_brute_force():
-    """The product's block-level planner (one three-key sort) against the reference's sequence of moves written out
-    with plain loops (quant/hqe_2.py:552-659): for every target from 1 bit up -- its members that stay, the new
-    tokens ranked into it, then what comes down from the fp16, 8, 4 and 2-bit classes in source order; a block
-    ranked into a higher precision stays; evicted blocks appear nowhere."""
+    """The library's host-side planner (hqekv_plan_side, through the product's wrapper) against the reference's
+    sequence of moves written out with plain loops (quant/hqe_2.py:552-659): for every target from 1 bit up -- its
+    members that stay, the new tokens ranked into it, then what comes down from the fp16, 8, 4 and 2-bit classes in
+    source order; a block ranked into a higher precision stays; evicted blocks appear nowhere, and the survivors'
+    new block numbers are their ranks among the survivors (quant/hqe_2.py:661-670)."""
     import numpy as np
     from hqekv_amd import cache_policy as cp
     rng = np.random.default_rng(0)
     for trial in range(300):
         hist, n_new = int(rng.integers(0, 40)), int(rng.integers(1, 8))
+        total = hist + n_new
         parts = np.split(rng.permutation(hist), np.sort(rng.integers(0, hist + 1, 4)))
         old = {b: parts[i].astype(np.int64) for i, b in enumerate(cp.CLASS_BITS) if parts[i].size}
-        label = rng.integers(0, 6, hist + n_new).astype(np.int8)
-        counts, slots, srcs, pos = cp._plan_side(old, hist, n_new, label)
+        n_targets = 6 if trial % 3 else 5
+        label = rng.integers(0, n_targets, total).astype(np.int8)
+        # a ranking and token counts that produce exactly these labels
+        order = np.concatenate([rng.permutation(np.flatnonzero(label == t)) for t in range(n_targets)]).astype(np.int64)
+        bit_num = [int((label == t).sum()) * 32 for t in range(n_targets)]
+        got = cp._plan_side_c(old, hist, n_new, order, bit_num)
+        assert got is not None, trial
+        counts, words, alive = got
         want = []
         for ti, bits in enumerate(cp.CLASS_BITS):
             for j, p in enumerate(old.get(bits, [])):
@@ -135,6 +143,23 @@ def test_block_planner_against_the_move_sequence_by_brute_force():
                 for j, p in enumerate(old.get(cp.CLASS_BITS[si], [])):
                     if label[p] == ti:
                         want.append((ti, si, j, p))
-        assert [w[1] for w in want] == slots.tolist() and [w[2] for w in want] == srcs.tolist(), trial
-        assert [w[3] for w in want] == pos.tolist(), trial
-        assert counts.tolist() == [sum(1 for w in want if w[0] == t) for t in range(5)]
+        u = len(want)
+        assert words.size == 2 * u, trial
+        assert [(w[1] << 24) | w[2] for w in want] == words[:u].tolist(), trial
+        survivors = sorted(w[3] for w in want)
+        rank = {p: r for r, p in enumerate(survivors)}
+        assert [rank[w[3]] for w in want] == words[u:].tolist(), trial
+        assert counts.tolist() == [sum(1 for w in want if w[0] == t) for t in range(5)], trial
+        if u < total:
+            assert alive.tolist() == survivors, trial
+        else:
+            assert alive is None, trial
+    # what the planner refuses: counts that are not whole blocks, a ranking that names a block twice, classes that do
+    # not partition the history
+    old = {16: np.array([0, 1], dtype=np.int64)}
+    order = np.array([0, 1, 2], dtype=np.int64)
+    assert cp._plan_side_c(old, 2, 1, order, [32, 0, 0, 0, 64]) is not None
+    assert cp._plan_side_c(old, 2, 1, order, [33, 0, 0, 0, 63]) is None
+    assert cp._plan_side_c(old, 2, 1, np.array([0, 0, 2], dtype=np.int64), [32, 0, 0, 0, 64]) is None
+    assert cp._plan_side_c({16: np.array([0, 0], dtype=np.int64)}, 2, 1, order, [32, 0, 0, 0, 64]) is None
+    assert cp._plan_side_c(old, 2, 1, order, [32, 0, 0, 0, 32]) is None
