@@ -1973,26 +1973,133 @@ __device__ __forceinline__ float torch_row_sum(int n_rows, Load &&load) {
   return v[0];
 }
 
-// columns [c0, c0 + n) of the ring row; one column per thread
-__device__ __forceinline__ void ring_row_columns(const StepEpilogue &e, int64_t c0, int64_t c1) {
-  for (int64_t t = c0 + threadIdx.x; t < c1; t += blockDim.x) {
-    const half_t *col = e.weights + t;
-    const int64_t hs = e.Tall, bs = (int64_t)e.Hq * e.Tall;
-    auto head = [&](int h) -> float {   // the batch sum of head h, rounded to fp16 as the first reduction stores it
-      if (e.B == 1) return (float)col[(int64_t)h * hs];
-      const float sb = torch_row_sum<1>(e.B, [&](int b) { return (float)col[(int64_t)b * bs + (int64_t)h * hs]; });
-      return (float)(half_t)sb;
-    };
-    const float sum = e.ring_by == 2 ? torch_row_sum<2>(e.Hq, head) : torch_row_sum<1>(e.Hq, head);
-    e.ring_line[t] = (half_t)sum;
+// torch_row_sum<1> for a row count known at compile time, fully unrolled (row k goes to accumulator k mod 4)
+template <int N, typename Load>
+__device__ __forceinline__ float torch_row_sum_n(Load &&load) {
+  float a[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < N; ++r) a[r & 3] += load(r);
+  return ((a[0] + a[1]) + a[2]) + a[3];
+}
+
+constexpr int RING_V = 4;                 // adjacent columns of the ring row a lane loads at a time (8 bytes)
+constexpr int RING_SPAN = 64 * RING_V;    // columns a workgroup covers per pass
+constexpr int RING_LDS_HEADS = 64;        // most heads whose batch sums a pass parks in LDS
+
+// The probabilities as a pointer into global memory: the pointer arrives inside a by-value struct, where the
+// compiler cannot tell its address space and would fall back to generic (flat) loads.
+typedef const __attribute__((address_space(1))) half_t *ring_src_t;
+struct __attribute__((packed, aligned(2))) ring_quad_t { uint64_t v; };   // RING_V probabilities at an element's alignment
+static_assert(sizeof(half_t) * RING_V == sizeof(uint64_t), "a quad is one 64-bit word");
+typedef const __attribute__((address_space(1))) ring_quad_t *ring_quad_src_t;
+
+// what the ring row needs from the epilogue's description, by value (nothing here lives in memory)
+struct RingShape {
+  ring_src_t w;      // (B, Hq, Tall)
+  int64_t Tall;
+  int B, Hq, by;
+};
+
+// heads g, g + waves, ... of a lane's RING_V columns into the LDS tile, for a batch of NB rows known at compile
+// time: the loads of HU heads are issued before the first sum is formed (the additions keep torch_row_sum's order)
+// `shift` > 0 marks the row's last, ragged quad: its loads start `shift` columns early, so that they end with the
+// row, and the wanted columns are moved down afterwards.
+template <int NB>
+__device__ __forceinline__ void ring_heads_to_lds(const RingShape r, ring_src_t col, int shift, int g, int waves,
+                                                  half_t *tile_lane) {
+  constexpr int HU = 8 / NB;   // heads in flight per thread: about eight loads
+  const int64_t hs = r.Tall, bs = (int64_t)r.Hq * r.Tall;
+  for (int h0 = g; h0 < r.Hq; h0 += waves * HU) {
+    uint64_t raw[HU][NB];   // a quad is loaded, shifted and stored as one 64-bit word
+#pragma unroll
+    for (int u = 0; u < HU; ++u) {
+      const int h = min(h0 + u * waves, r.Hq - 1);
+#pragma unroll
+      for (int b = 0; b < NB; ++b)   // 8 bytes at the alignment of an element: the target reads unaligned
+        raw[u][b] = reinterpret_cast<ring_quad_src_t>(col + (int64_t)b * bs + (int64_t)h * hs)->v >> (16 * shift);
+    }
+#pragma unroll
+    for (int u = 0; u < HU; ++u) {
+      const int h = h0 + u * waves;
+      uint64_t v = raw[u][0];
+      if constexpr (NB > 1) {
+        v = 0;
+#pragma unroll
+        for (int i = 0; i < RING_V; ++i) {
+          const half_t s = (half_t)torch_row_sum_n<NB>(
+              [&](int b) { return (float)__builtin_bit_cast(half_t, (uint16_t)(raw[u][b] >> (16 * i))); });
+          v |= (uint64_t)__builtin_bit_cast(uint16_t, s) << (16 * i);
+        }
+      }
+      if (h < r.Hq) *reinterpret_cast<uint64_t *>(tile_lane + h * RING_SPAN) = v;   // 8-byte aligned: lane * RING_V halves
+    }
+  }
+}
+
+// Column t for any batch size and head count, one load at a time: for the shapes the tiled path does not take.
+// Kept out of line so that its registers do not add to the tiled path's.
+__device__ __noinline__ float ring_column_alone(const RingShape r, int64_t t) {
+  ring_src_t col = r.w + t;
+  const int64_t hs = r.Tall, bs = (int64_t)r.Hq * r.Tall;
+  auto head = [&](int h) -> float {
+    if (r.B == 1) return (float)col[(int64_t)h * hs];
+    return (float)(half_t)torch_row_sum<1>(r.B, [&](int b) { return (float)col[(int64_t)b * bs + (int64_t)h * hs]; });
+  };
+  return r.by == 2 ? torch_row_sum<2>(r.Hq, head) : torch_row_sum<1>(r.Hq, head);
+}
+
+// Columns [c0, c1) of the ring row, RING_SPAN per pass (c0 a multiple of RING_SPAN).  The loads are spread over the
+// whole workgroup -- lane l of every wave looks at columns 4 l .. 4 l + 3 of the pass, wave g at heads g, g + waves,
+// ... -- so every load is independent of the others and 8 bytes wide; the head values (fp16 by construction) meet
+// in LDS, where the first RING_SPAN threads add them up in torch's order, one column each.  Every thread of the
+// workgroup must call this with the same arguments; blockDim.x is a multiple of 64 and at least RING_SPAN.
+__device__ __forceinline__ void ring_row_columns(const StepEpilogue &e, int64_t c0, int64_t c1, half_t *tile) {
+  const RingShape r{(ring_src_t)(uintptr_t)e.weights, e.Tall, e.B, e.Hq, e.ring_by};
+  half_t *const line = e.ring_line;
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const bool lds = r.Hq <= RING_LDS_HEADS && r.B <= 8;
+  for (int64_t t0 = c0; t0 < c1; t0 += RING_SPAN) {
+    const int64_t t = t0 + threadIdx.x;   // the column this thread sums in the end (threads below RING_SPAN)
+    if (lds) {
+      const int64_t c = t0 + lane * RING_V;
+      // the row's last quad may stick out by `shift` columns (the passes of all workgroups but the last end on a
+      // multiple of RING_SPAN): it is loaded from `shift` columns earlier, which needs a row of RING_V columns at least
+      const int shift = (int)max((int64_t)0, c + RING_V - c1);
+      const bool mine = shift < RING_V && c - shift >= 0;
+      ring_src_t col = r.w + (mine ? c - shift : 0);
+      half_t *tile_lane = tile + lane * RING_V;
+      switch (mine ? r.B : 0) {
+        case 1: ring_heads_to_lds<1>(r, col, shift, g, waves, tile_lane); break;
+        case 2: ring_heads_to_lds<2>(r, col, shift, g, waves, tile_lane); break;
+        case 3: ring_heads_to_lds<3>(r, col, shift, g, waves, tile_lane); break;
+        case 4: ring_heads_to_lds<4>(r, col, shift, g, waves, tile_lane); break;
+        case 5: ring_heads_to_lds<5>(r, col, shift, g, waves, tile_lane); break;
+        case 6: ring_heads_to_lds<6>(r, col, shift, g, waves, tile_lane); break;
+        case 7: ring_heads_to_lds<7>(r, col, shift, g, waves, tile_lane); break;
+        case 8: ring_heads_to_lds<8>(r, col, shift, g, waves, tile_lane); break;
+        default: break;
+      }
+      __syncthreads();
+    }
+    if (threadIdx.x < RING_SPAN && t < c1) {
+      float sum;
+      if (lds && c1 >= RING_V) {
+        auto head = [&](int h) -> float { return (float)tile[h * RING_SPAN + threadIdx.x]; };
+        sum = r.by == 2 ? torch_row_sum<2>(r.Hq, head) : torch_row_sum<1>(r.Hq, head);
+      } else {   // outside what the LDS tile covers: the thread walks its column alone
+        sum = ring_column_alone(r, t);
+      }
+      line[t] = (half_t)sum;
+    }
+    if (lds) __syncthreads();
   }
 }
 
 // block `blk` of `nblk` of the epilogue: a share of the ring row's columns, and of the appended rows
-__device__ __forceinline__ void step_epilogue_block(const StepEpilogue &e, int64_t blk, int64_t nblk) {
+__device__ __forceinline__ void step_epilogue_block(const StepEpilogue &e, int64_t blk, int64_t nblk, half_t *sh) {
   if (e.ring_line) {
-    const int64_t per = (e.Tall + nblk - 1) / nblk;
-    ring_row_columns(e, blk * per, min(e.Tall, (blk + 1) * per));
+    const int64_t per = ((e.Tall + nblk - 1) / nblk + RING_SPAN - 1) / RING_SPAN * RING_SPAN;
+    ring_row_columns(e, min(e.Tall, blk * per), min(e.Tall, (blk + 1) * per), sh);
   }
   if (e.app_rows > 0) {   // 16-byte pieces of the appended rows, dealt over the blocks
     const int64_t row16 = e.app_row_elems / 8;   // pieces per row (head_dim is a multiple of 32)
@@ -2016,14 +2123,17 @@ __device__ __forceinline__ void step_epilogue_block(const StepEpilogue &e, int64
 __global__ __launch_bounds__(CB_CH * CB_SLICES) void pv_combine_kernel(const float *__restrict__ partial,
                                                                       half_t *__restrict__ out, int n_chunks,
                                                                       int64_t n_bhq, int D, StepEpilogue ep, int combine) {
+  static_assert(RING_LDS_HEADS * RING_SPAN * sizeof(half_t) >= (CB_SLICES / 2) * CB_CH * sizeof(float) &&
+                    CB_CH * CB_SLICES >= RING_SPAN, "one LDS array serves both roles");
+  __shared__ __align__(16) half_t sh_all[RING_LDS_HEADS * RING_SPAN];
   const int z0 = combine ? 1 : 0;
   if ((int)blockIdx.z >= z0) {
     const int64_t per_z = (int64_t)gridDim.x * gridDim.y;
     step_epilogue_block(ep, ((int64_t)blockIdx.z - z0) * per_z + (int64_t)blockIdx.y * gridDim.x + blockIdx.x,
-                        per_z * (gridDim.z - z0));
+                        per_z * (gridDim.z - z0), sh_all);
     return;
   }
-  __shared__ float sh[CB_SLICES / 2][CB_CH];
+  float (*sh)[CB_CH] = reinterpret_cast<float (*)[CB_CH]>(sh_all);
   const int64_t r = blockIdx.x;
   const int d = threadIdx.x % CB_CH, sl = threadIdx.x / CB_CH;  // a wave holds two slices of the 32 channels
   const int d0 = blockIdx.y * CB_CH;
@@ -2271,12 +2381,12 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
   const bool combine = (stages & 2) && !fz.arrive;   // folded: the last p.V workgroups have written the output
   const bool epilogue = ep && (ep->ring_line || ep->app_rows > 0) && stages == 3;
   if (!combine && !epilogue) return HQEKV_OK;
-  // The epilogue rides in the combine launch as extra workgroups (grid.z); one workgroup per 4096 columns of the
-  // ring row.  Without a combine (folded into p.V) the launch holds the epilogue alone.
+  // The epilogue rides in the combine launch as extra workgroups (grid.z); one workgroup per RING_SPAN columns of
+  // the ring row.  Without a combine (folded into p.V) the launch holds the epilogue alone.
   const dim3 base((unsigned)n_bhq, (unsigned)((D + CB_CH - 1) / CB_CH));
   unsigned z = combine ? 1u : 0u;
   if (epilogue) {
-    const int64_t want = ep->ring_line ? (Tall + 4095) / 4096 : 1;
+    const int64_t want = ep->ring_line ? (Tall + RING_SPAN - 1) / RING_SPAN : 1;
     z += (unsigned)((want + (int64_t)base.x * base.y - 1) / ((int64_t)base.x * base.y));
   }
   StepEpilogue none{};
@@ -2444,8 +2554,8 @@ extern "C" int hqekv_ring_row(const void *attn_weights, int64_t B, int64_t Hq, i
   StepEpilogue e;
   const int rc = fill_epilogue(&x, attn_weights, B, Hq, 1, 32, Tall, &e);
   if (rc) return rc;
-  const int64_t blocks = (Tall + 4095) / 4096;
-  if (blocks > 65535) return fail(HQEKV_E_UNSUPPORTED, "ring_row: Tall too large");
+  const int64_t blocks = (Tall + RING_SPAN - 1) / RING_SPAN;
+  if (blocks > 0x7fffffffLL) return fail(HQEKV_E_UNSUPPORTED, "ring_row: Tall too large");
   hipLaunchKernelGGL(pv_combine_kernel, dim3((unsigned)blocks, 1, 1), dim3(CB_CH * CB_SLICES), 0, (hipStream_t)stream,
                      (const float *)nullptr, (half_t *)nullptr, 0, (int64_t)0, 0, e, 0);
   return check_launch("ring_row");

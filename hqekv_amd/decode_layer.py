@@ -189,6 +189,11 @@ class HqeAttentionLayer:
             on_device = (self.fused_step and L == 1 and Tall >= 256 and query_states.shape[1] == 32
                          and query_states.shape[0] <= 8 and query_states.dtype == torch.float16
                          and (lw.weights is None or lw.weights.dtype == torch.float16) and lw.max_length >= Tall)
+            if self.fused_step and attention_mask is None and L == 1 and query_states.is_cuda:
+                # slices of a fused projection's output arrive with a batch stride of their own: one small copy each
+                # buys the one-call step
+                query_states, key_states, value_states = (x if x.is_contiguous() else x.contiguous()
+                                                          for x in (query_states, key_states, value_states))
             plain_inputs = (self.fused_step and attention_mask is None and query_states.shape[2] == 1
                             and query_states.is_contiguous() and key_states.is_contiguous() and value_states.is_contiguous()
                             and query_states.dtype == torch.float16 and query_states.is_cuda

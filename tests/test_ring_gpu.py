@@ -59,6 +59,36 @@ def test_ring_row_equals_torch_sum_on_device(dev, B, kind):
         assert torch.equal(ring.weights[slot, :T].view(torch.int16), w.sum(0).sum(0).reshape(T).view(torch.int16)), T
 
 
+def _row_sum_in_kernel_order(rows, by):
+    """The documented order on the host in float32: the rows are dealt round-robin to ``by`` walkers, a walker adds its
+    k-th row to accumulator k mod 4 and closes with ((a0 + a1) + a2) + a3, two walkers are added at the end."""
+    parts = []
+    for y in range(by):
+        acc = [torch.zeros(rows.shape[1], dtype=torch.float32) for _ in range(4)]
+        for k, r in enumerate(range(y, rows.shape[0], by)):
+            acc[k % 4] = acc[k % 4] + rows[r].float()
+        parts.append(((acc[0] + acc[1]) + acc[2]) + acc[3])
+    return parts[0] if by == 1 else parts[0] + parts[1]
+
+
+@pytest.mark.parametrize("B,H,T", [(9, 32, 300), (2, 80, 300), (2, 32, 3), (1, 32, 2), (3, 7, 1031)])
+@pytest.mark.parametrize("by", [1, 2])
+def test_ring_row_shapes_outside_the_tiled_path(dev, B, H, T, by):
+    """More than 8 batch rows, more than 64 heads, rows shorter than one 4-column load: the kernel walks such columns
+    one load at a time.  torch's order is not pinned for these shapes, so the check is the documented order itself."""
+    from hqekv_amd import _lib
+    g = torch.Generator().manual_seed(B * 1000 + H + T)
+    w = _order_sensitive(B, H, T, g)
+    per_head = w[0, :, 0] if B == 1 else torch.stack([_row_sum_in_kernel_order(w[:, h, 0], 1).half() for h in range(H)])
+    expect = _row_sum_in_kernel_order(per_head, by).half()
+    line = torch.full((T + 3,), -5.0, dtype=torch.float16, device=dev)
+    wd = w.to(dev)
+    _lib.check(_lib.load().hqekv_ring_row(wd.data_ptr(), B, H, T, line.data_ptr(), by, _lib.stream_ptr(dev)), "ring_row")
+    torch.cuda.synchronize()
+    assert torch.equal(line[:T].cpu().view(torch.int16), expect.view(torch.int16))
+    assert bool((line[T:] == -5.0).all())
+
+
 def test_ring_row_rejects_bad_arguments(dev):
     from hqekv_amd import _lib
     lib = _lib.load()
