@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+import weakref
 from typing import List, Optional, Tuple
 
 import numpy as np
@@ -164,9 +165,12 @@ def idx_cover_once(idx_list, n: int) -> bool:
         return False
     if not idx_list:
         return True
-    key = tuple((id(t), t._version) for t in idx_list) + (n,)
-    hit = getattr(idx_list[0], "_hq_cover", None)   # rides on the first array, like the cache policy's host copies
-    if hit is not None and hit[0] == key:
+    # The verdict rides on the first array and names the others by weak reference: it holds while these very tensor
+    # objects are alive, sit where they sat and have not been written through torch since.  (A kernel that writes an
+    # array through its raw pointer does not show here: whoever launches one drops `_hq_cover` from the array.)
+    key = tuple((t.data_ptr(), int(t.numel()), t._version) for t in idx_list) + (n,)
+    hit = getattr(idx_list[0], "_hq_cover", None)
+    if hit is not None and hit[0] == key and len(hit[2]) == len(idx_list) and all(r() is t for r, t in zip(hit[2], idx_list)):
         return hit[1]
     trusted = [getattr(t, "_hq_host_version", None) == t._version for t in idx_list]
     blocks = [getattr(t, "_hq_blocks", None) if ok_ else None for t, ok_ in zip(idx_list, trusted)]
@@ -182,7 +186,7 @@ def idx_cover_once(idx_list, n: int) -> bool:
         c = torch.cat([t.reshape(-1).to(torch.int64) for t in idx_list])
         inside = (c >= 0) & (c < n)
         ok = bool(inside.all() & (torch.bincount(c.clamp(0, n - 1), minlength=n) == 1).all())
-    idx_list[0]._hq_cover = (key, ok)
+    idx_list[0]._hq_cover = (key, ok, [weakref.ref(t) for t in idx_list])
     return ok
 
 

@@ -564,13 +564,17 @@ def _compress_gather(pkv: tuple, new_K, new_V, res_K, res_V, history: int, compr
     k_ord = getattr(K_sorted_idx, "_hq_block_order", None)
     v_ord = getattr(V_sorted_idx, "_hq_block_order", None)
     k_order_h = v_order_h = None
-    if (k_ord is not None and v_ord is not None and k_ord[0].numel() == total_blocks == v_ord[0].numel()
-            and getattr(K_sorted_idx, "_hq_block_order_version", None) == K_sorted_idx._version
-            and k_ord[0].device == v_ord[0].device):
+
+    def fresh(idx, ord_):   # the ranking that rides on a token list counts only while nobody has written into the list
+        return (ord_ is not None and ord_[0].numel() == total_blocks
+                and getattr(idx, "_hq_block_order_version", None) == idx._version)
+    if fresh(K_sorted_idx, k_ord) and fresh(V_sorted_idx, v_ord) and k_ord[0].device == v_ord[0].device:
         both = torch.stack((k_ord[0], v_ord[0])).to("cpu", torch.int64).numpy()
         k_order_h, v_order_h = both[0], both[1]
-    elif v_ord is not None and v_ord[0].numel() == total_blocks:
+    elif fresh(V_sorted_idx, v_ord):
         v_order_h = v_ord[0].to("cpu", torch.int64).numpy()
+    elif fresh(K_sorted_idx, k_ord):
+        k_order_h = k_ord[0].to("cpu", torch.int64).numpy()
     if k_order_h is None:
         k_order_h = _host_blocks(K_sorted_idx)
     if v_order_h is None:

@@ -370,7 +370,10 @@ int hqekv_plan_side(const int32_t *const *old_blocks, const int32_t *old_counts,
 /* No counterpart in the reference: hqekv_decode_attn for callers that cannot allocate (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  Same arguments minus the workspace: the split-K
  * partials and softmax statistics go to a fixed buffer of HQEKV_STATIC_SCRATCH_BYTES inside the library's device
- * image, one copy per GPU, held until the process ends; its address is looked up on the first call on a device.
+ * image, one copy per GPU, held until the process ends; its address is looked up on the first call on a device
+ * (hipGetSymbolAddress, which may make the runtime load the library's device image): make that first call on every
+ * device BEFORE a stream capture begins -- a call with the real shapes or any small one -- since a runtime that loads
+ * code inside a capture may refuse the capture.  Later calls only launch kernels.
  * The call allocates and frees nothing.  A call whose hqekv_decode_workspace_bytes() exceeds the buffer returns
  * HQEKV_E_WORKSPACE (use hqekv_decode_attn then).  All calls on one GPU share the buffer: calls that overlap in
  * time on one GPU (two streams, two threads) race; calls ordered on one stream are fine.

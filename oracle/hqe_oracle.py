@@ -35,8 +35,12 @@ ATen evaluates as multiply-by-reciprocal.  ``scalar_div='recip'`` restates that 
 torch's own on-device op chain to close the gap.  The accumulation order of ``torch.std_mean`` on the GPU
 (last fp16 place of std / mean of the normal-quantile class) is restated in ``std_mean_gpu_tree`` and pinned by
 the GPU suite, which compares the HIP quantiser with ``torch.std_mean`` run on the device bit for bit, plus a
-known answer recorded from such a run (tests/test_oracle.py).  Also unpinned: the order of equal scores in
-``torch.sort`` (block ranking; restated with a stable sort).
+known answer recorded from such a run (tests/test_oracle.py).  That pin is to torch on ROCm (MI355X) only: which
+order ``torch.std_mean`` takes on the reference's own CUDA platform is covered by no fixture the reference holds, so
+the last place of std / mean -- and the sign codes of values next to the mean -- are PARITY UNPINNED against the
+reference as its authors ran it.  The CPU order (``NORMAL1_STAT_ORDER = "torch_cpu"``, the default) stays exercised
+by the CPU suite.  Also unpinned: the order of equal scores in ``torch.sort`` (block ranking; restated with a stable
+sort).
 """
 from __future__ import annotations
 

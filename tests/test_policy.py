@@ -163,3 +163,25 @@ def test_block_planner_against_the_move_sequence_by_brute_force():
     assert cp._plan_side_c(old, 2, 1, np.array([0, 0, 2], dtype=np.int64), [32, 0, 0, 0, 64]) is None
     assert cp._plan_side_c({16: np.array([0, 0], dtype=np.int64)}, 2, 1, order, [32, 0, 0, 0, 64]) is None
     assert cp._plan_side_c(old, 2, 1, order, [32, 0, 0, 0, 32]) is None
+
+
+def test_cover_once_verdict_is_not_reused_for_other_tensors():
+    """The remembered verdict of ``idx_cover_once`` belongs to the very tensors it was formed on, in the state they
+    were in: an array written in place, or another array in the place of one that has been freed, is checked again."""
+    from hqekv_amd.attention import idx_cover_once
+    a = torch.arange(0, 64, dtype=torch.int32)
+    b = torch.arange(64, 128, dtype=torch.int32)
+    assert idx_cover_once([a, b], 128) and idx_cover_once([a, b], 128)
+    assert a._hq_cover[1] is True
+    del b
+    for _ in range(8):   # new arrays of the same size, one of which may well land where b was
+        c = torch.arange(60, 124, dtype=torch.int32)          # overlaps a: not a partition
+        assert not idx_cover_once([a, c], 128)
+        del c
+    b = torch.arange(64, 128, dtype=torch.int32)
+    assert idx_cover_once([a, b], 128)
+    b[5] = 3                                                   # written through torch: the version moves
+    assert not idx_cover_once([a, b], 128)
+    b[5] = 69
+    assert idx_cover_once([a, b], 128)
+    assert not idx_cover_once([a, b], 129) and not idx_cover_once([a], 128)

@@ -55,8 +55,10 @@ def _cache(B, Hq, Hkv, T, residual, seed, dev):
     return q, cache, q.to(dev), synth.cache_to(cache, dev)
 
 
-@pytest.mark.parametrize("flags", [1, 0], ids=["fused", "general"])
+@pytest.mark.parametrize("flags", [1, 0, 1 | 4], ids=["fused", "general", "fused_folded_combine"])
 def test_static_scratch_entry_matches_workspace_entry(dev, flags):
+    """The third case forces the folded combine (HQEKV_FOLD_COMBINE), whose arrival counters live in the shared
+    buffer too: they must be back at zero for the second call."""
     big = _cache(2, 8, 2, 4096 + 21, 21, 31, dev)
     small = _cache(1, 8, 2, 640 + 3, 3, 32, dev)
     for q, cache, qd, cd in (big, small):   # the second call is the smaller one, on the buffer the first one used
@@ -65,6 +67,32 @@ def test_static_scratch_entry_matches_workspace_entry(dev, flags):
         w_ref, o_ref = O.qkv_matmul(q, cache, None, 128, use_mask=False, round_per_class=False)
         torch.testing.assert_close(w1.float().cpu(), w_ref.float(), rtol=1e-3, atol=2e-3)
         torch.testing.assert_close(o1.float().cpu(), o_ref.float(), rtol=1e-3, atol=2e-3)
+
+
+def test_static_scratch_entry_leaves_device_memory_alone(dev):
+    """Free device memory, as the driver reports it, is the same before and after calls of the static entry (the first
+    call on the device, which looks up the buffer's address, has been made before the measurement starts)."""
+    from hqekv_amd import _lib
+    lib = _lib.load()
+    q, cache, qd, cd = _cache(2, 8, 2, 2048 + 5, 5, 33, dev)
+    B, Hq, _, D = qd.shape
+    k_segs, n_k, v_segs, n_v, Hkv, Tall, keep = _tables(qd, cd, dev)
+    w = torch.zeros(B, Hq, 1, Tall, dtype=torch.float16, device=dev)
+    o = torch.zeros(B, Hq, 1, D, dtype=torch.float16, device=dev)
+    st = _lib.stream_ptr(dev)
+
+    def call(flags):
+        _lib.check(lib.hqekv_decode_attn_static(k_segs, n_k, v_segs, n_v, qd.data_ptr(), None, 0, w.data_ptr(),
+                                                o.data_ptr(), B, Hq, Hkv, D, Tall, flags, st), "decode_attn_static")
+    call(1)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(dev)
+    reserved_before = torch.cuda.memory_reserved(dev)
+    for flags in (1, 0, 1 | 4, 1):
+        call(flags)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(dev)
+    assert free_after == free_before and torch.cuda.memory_reserved(dev) == reserved_before
 
 
 def test_static_scratch_entry_rejects_what_does_not_fit(dev):
