@@ -33,7 +33,7 @@ import numpy as np
 import torch
 
 from . import pack_unpack as PU
-from .public_func import calculate_token_range, get_block_token_idx
+from .public_func import RankedBlocks, calculate_token_range, get_block_token_idx, rank_blocks
 
 BLOCK = 32
 CLASS_BITS = (16, 8, 4, 2, 1)
@@ -76,6 +76,8 @@ def _host_idx(t: torch.Tensor) -> np.ndarray:
 
 def _host_blocks(t: torch.Tensor) -> Optional[np.ndarray]:
     """Block numbers (first position / 32) of a position tensor made of whole aligned blocks, else None."""
+    if isinstance(t, RankedBlocks):
+        t = t.tokens()
     if getattr(t, "_hq_host_version", None) == t._version:
         blocks = getattr(t, "_hq_blocks", None)
         if blocks is not None and blocks.shape[0] * BLOCK == t.numel():
@@ -391,26 +393,29 @@ def _plan_side_c(old_blocks: Dict[int, np.ndarray], hist_blocks: int, n_new_bloc
     from . import _lib
     import ctypes as C
     total = hist_blocks + n_new_blocks
-    counts_t = [int(v) for v in (bit_num.tolist() if torch.is_tensor(bit_num) else bit_num)]
+    counts_t = bit_num.tolist() if torch.is_tensor(bit_num) else [int(v) for v in bit_num]
     if order_h is None or order_h.shape[0] != total:
         return None
-    order64 = np.ascontiguousarray(order_h, dtype=np.int64)
+
+    def addr(a: np.ndarray) -> int:   # (cheaper than a.ctypes.data, which builds a ctypes object per call)
+        return a.__array_interface__["data"][0]
+    order64 = order_h if order_h.dtype == np.int64 and order_h.flags.c_contiguous else np.ascontiguousarray(order_h, dtype=np.int64)
     ptrs = (C.c_void_p * 5)()
     cnts = (C.c_int32 * 5)()
     hold = []
     for ci, bits in enumerate(CLASS_BITS):
         b = old_blocks.get(bits)
         if b is not None and b.size:
-            b32 = np.ascontiguousarray(b, dtype=np.int32)
+            b32 = b if b.dtype == np.int32 and b.flags.c_contiguous else np.ascontiguousarray(b, dtype=np.int32)
             hold.append(b32)
-            ptrs[ci], cnts[ci] = b32.ctypes.data, b32.size
+            ptrs[ci], cnts[ci] = addr(b32), b32.size
     targets = (C.c_int64 * len(counts_t))(*counts_t)
-    counts = np.empty(5, dtype=np.int32)
-    plan = np.empty(2 * total + 2, dtype=np.int32)
-    alive = np.empty(max(total, 1), dtype=np.int32)
+    out = np.empty(3 * total + 8, dtype=np.int32)   # counts (5, padded to 6), plan words (2 * total), survivors (total)
+    counts, plan, alive = out[:5], out[6:6 + 2 * total], out[6 + 2 * total:6 + 3 * total]
     n_alive = C.c_int32(0)
-    rc = _lib.load().hqekv_plan_side(ptrs, cnts, hist_blocks, n_new_blocks, order64.ctypes.data, targets, len(counts_t),
-                                     counts.ctypes.data, plan.ctypes.data, alive.ctypes.data, C.byref(n_alive))
+    base = addr(out)
+    rc = _lib.load().hqekv_plan_side(ptrs, cnts, hist_blocks, n_new_blocks, addr(order64), targets, len(counts_t),
+                                     base, base + 24, base + 4 * (6 + 2 * total), C.byref(n_alive))
     if rc:
         return None
     u = n_alive.value
@@ -429,10 +434,11 @@ def _numel(shape) -> int:
 
 
 def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, counts, plan_words: np.ndarray,
-                 strategy: str) -> Dict[int, _Cls]:
+                 strategy: str, plan_dev: Optional[torch.Tensor] = None) -> Dict[int, _Cls]:
     """Allocate the new classes of one side (one buffer per element type, the tensors are views of it) and fill
     them with one launch of the migration kernel.  ``plan_words`` (int32): per new block, the classes back to
-    back, (source slot << 24) | source block, then every block's new block number."""
+    back, (source slot << 24) | source block, then every block's new block number; ``plan_dev``: the same words on
+    the device when the caller has sent them already."""
     nb = plan_words.size // 2
     pos = plan_words[nb:].astype(np.int64)
     from . import _lib
@@ -521,7 +527,8 @@ def _gather_side(is_k: bool, side: Dict[int, _Cls], new: torch.Tensor, counts, p
         idx_t._hq_host_version = idx_t._version
         blk0 += n // BLOCK
         out[bits] = _Cls(data, idx_t, sc, zr)
-    plan = _to_dev(np.ascontiguousarray(plan_words).view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
+    plan = plan_dev if plan_dev is not None else \
+        _to_dev(np.ascontiguousarray(plan_words).view(np.int64), dev).view(torch.int32)   # int32 pairs ride as int64
     with _lib.on_device(dev):
         # (no status word: this plan was made a few lines up from the classes it names; the kernel still checks it)
         rc = _lib.load().hqekv_cache_migrate(1 if is_k else 0, src, _SRC_NEW + 1, dst, n_dst, plan.data_ptr(), B * H, D,
@@ -560,15 +567,23 @@ def _compress_gather(pkv: tuple, new_K, new_V, res_K, res_V, history: int, compr
         if kept != hist_blocks:
             return None
         old[name] = blocks
-    # the two block rankings come down in one transfer when both carry theirs
-    k_ord = getattr(K_sorted_idx, "_hq_block_order", None)
-    v_ord = getattr(V_sorted_idx, "_hq_block_order", None)
+    # the two block rankings come down in one transfer when both carry theirs (and out of one sort call when neither
+    # has been sorted yet)
     k_order_h = v_order_h = None
+    if isinstance(K_sorted_idx, RankedBlocks) and isinstance(V_sorted_idx, RankedBlocks) \
+            and K_sorted_idx.scores.numel() == total_blocks == V_sorted_idx.scores.numel() \
+            and K_sorted_idx.scores.device == V_sorted_idx.scores.device:
+        both = RankedBlocks.sort_together(K_sorted_idx, V_sorted_idx).to("cpu", torch.int64).numpy()
+        k_order_h, v_order_h = both[0], both[1]
+    k_ord = getattr(K_sorted_idx, "_hq_block_order", None) if k_order_h is None else None
+    v_ord = getattr(V_sorted_idx, "_hq_block_order", None) if v_order_h is None else None
 
     def fresh(idx, ord_):   # the ranking that rides on a token list counts only while nobody has written into the list
         return (ord_ is not None and ord_[0].numel() == total_blocks
                 and getattr(idx, "_hq_block_order_version", None) == idx._version)
-    if fresh(K_sorted_idx, k_ord) and fresh(V_sorted_idx, v_ord) and k_ord[0].device == v_ord[0].device:
+    if k_order_h is not None:
+        pass
+    elif fresh(K_sorted_idx, k_ord) and fresh(V_sorted_idx, v_ord) and k_ord[0].device == v_ord[0].device:
         both = torch.stack((k_ord[0], v_ord[0])).to("cpu", torch.int64).numpy()
         k_order_h, v_order_h = both[0], both[1]
     elif fresh(V_sorted_idx, v_ord):
@@ -584,15 +599,23 @@ def _compress_gather(pkv: tuple, new_K, new_V, res_K, res_V, history: int, compr
     if k_plan is None or v_plan is None:
         return None
     dev = new_V.device
+    # one transfer for everything the device needs: both plans (int32 pairs riding as int64) and the positions of
+    # the tokens that survive on the V side
+    k_words, v_words, alive = k_plan[1], v_plan[1], v_plan[2]
+    parts = [np.ascontiguousarray(k_words).view(np.int64), np.ascontiguousarray(v_words).view(np.int64)]
+    if alive is not None:
+        parts.append((alive[:, None] * BLOCK + np.arange(BLOCK, dtype=np.int64)).reshape(-1))
+    sent = _to_dev(np.concatenate(parts), dev)
+    n_kw, n_vw = parts[0].size, parts[1].size
+    plan_dev = {"k": sent[:n_kw].view(torch.int32), "v": sent[n_kw:n_kw + n_vw].view(torch.int32)}
     sides = {}
-    for name, is_k, side, new, (counts, words, alive) in (("k", True, k_side, new_K, k_plan), ("v", False, v_side, new_V, v_plan)):
-        sides[name] = _gather_side(is_k, side, new, counts, words, strategy)
-        if name == "v" and alive is not None:   # evicted tokens leave the token ranges and the ring as well
-            keep_tok = (alive[:, None] * BLOCK + np.arange(BLOCK, dtype=np.int64)).reshape(-1)
-            keep_t = _to_dev(keep_tok, dev)
-            V_norm = V_norm[keep_t]
-            if last_weights is not None:
-                last_weights.eviction(keep_t)
+    for name, is_k, side, new, (counts, words, _) in (("k", True, k_side, new_K, k_plan), ("v", False, v_side, new_V, v_plan)):
+        sides[name] = _gather_side(is_k, side, new, counts, words, strategy, plan_dev[name])
+    if alive is not None:   # evicted tokens leave the token ranges and the ring as well
+        keep_t = sent[n_kw + n_vw:]
+        V_norm = V_norm[keep_t]
+        if last_weights is not None:
+            last_weights.eviction(keep_t)
     t = list(pkv)
     _write_side(t, sides["k"], K_SLOT, dev)
     _write_side(t, sides["v"], V_SLOT, dev)
@@ -620,15 +643,16 @@ def compress(past_key_value: tuple, compress_length: int, history_length, K_sort
         raise ValueError("compress_length and history_length must be multiples of 32")
     if K_bit_num.numel() != n_targets or V_bit_num.numel() != n_targets:
         raise ValueError(f"K_bit_num / V_bit_num must hold {n_targets} entries")
-    res_K = _none_if_empty(new_K[:, :, compress_length:, :].clone())
-    res_V = _none_if_empty(new_V[:, :, compress_length:, :].clone())
+    whole = new_K.shape[2] == compress_length and new_V.shape[2] == compress_length   # nothing stays behind
+    res_K = None if whole else _none_if_empty(new_K[:, :, compress_length:, :].clone())
+    res_V = None if whole else _none_if_empty(new_V[:, :, compress_length:, :].clone())
     new_K, new_V = new_K[:, :, :compress_length, :], new_V[:, :, :compress_length, :]
     total = history + compress_length
     block_num = total // BLOCK
 
     V_norm = V_token_range if V_token_range is not None else calculate_token_range(new_V, pkv[38])
     V_score = token_importance * V_norm if times_range else token_importance.clone()
-    V_sorted_idx = get_block_token_idx(BLOCK, block_num, V_score)
+    V_sorted_idx = rank_blocks(BLOCK, block_num, V_score)   # the token list is spelt out only if the step engine runs
 
     dev = new_V.device
     engine = engine or os.environ.get("HQEKV_POLICY_ENGINE", "auto")

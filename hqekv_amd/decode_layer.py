@@ -19,12 +19,13 @@ from __future__ import annotations
 
 from typing import Optional, Tuple
 
+import numpy as np
 import torch
 
 from .attention import SegmentMemo, value_length
 from .hqe_2 import KV_cache_hqe_2
 from .hqe_matmul import qkv_matmul_hqe_2
-from .public_func import get_block_token_idx, last_attn_weights, make_sum_equal
+from .public_func import last_attn_weights, rank_blocks
 
 LAST_TOKEN_NUM = 20
 BLOCK = 32
@@ -57,29 +58,47 @@ def gqa_prompt_attention(q, k, v, attention_mask, scaling):
                                                             attn_mask=attention_mask, is_causal=causal, scale=scaling)
 
 
+_F32 = np.float32
+
+
 def class_token_counts(total_length: int, ratio_q: torch.Tensor, ratio_e: torch.Tensor):
     """Tokens per target -- fp16, 8, 4, 2, 1 bit, evicted -- for a history of ``total_length`` tokens
     (model/llama_hqe.py:216-224).  64 tokens' worth of blocks stay fp16 and nothing goes to 8 bit; the rest is
     split by ``ratio_q`` (4, 2, 1 bit) and ``ratio_e`` (evicted), in float32 like the reference, rounded to
-    whole blocks and repaired to add up.  -> (shares (6,) float32, token counts (6,) int32)."""
+    whole blocks and repaired to add up (model/public_func.py:259-268).  -> (shares (6,) float32, token counts (6,)
+    int32).  The arithmetic runs on numpy float32 scalars and 6-element arrays -- the same IEEE operations in the
+    same order as the reference's CPU tensor ops, at a fraction of their dispatch cost."""
     blocks = total_length // BLOCK
-    shares = torch.zeros(6, dtype=torch.float32)
+    shares = np.zeros(6, dtype=np.float32)
     shares[0] = 64 / total_length
-    shares[2:5] = ratio_q
-    shares[5:] = ratio_e
-    shares[2:] = (1 - shares[0]) * shares[2:]
-    counts = make_sum_equal(torch.round(blocks * shares).to(torch.int), blocks)
-    counts *= BLOCK
-    return shares, counts
+    rest = _F32(1) - shares[0]
+    shares[2:5] = rest * ratio_q.numpy()
+    shares[5] = rest * ratio_e.numpy()[0]
+    counts = [int(c) for c in np.rint(_F32(blocks) * shares)]   # half to even, like torch.round
+    excess = sum(counts) - blocks
+    if excess < 0:
+        counts[4] -= excess
+    else:   # taken from the 1-bit entry, then from the entries below it, each down to zero at most
+        i = 4
+        while excess > 0 and i >= 0:
+            take = min(excess, counts[i])
+            counts[i] -= take
+            excess -= take
+            i -= 1
+    return torch.from_numpy(shares), torch.tensor([c * BLOCK for c in counts], dtype=torch.int32)
 
 
 def ratios_for_next_increment(history: int, ratio_e_0: torch.Tensor, ratio_q: torch.Tensor):
     """The eviction share applies to the tokens the next compression adds, not to the history it re-ranks:
     scale it by added / (history + added) and give the quantised classes the rest, in their old proportions
-    (model/llama_hqe.py:235-239).  -> (ratio_e, ratio_q)."""
+    (model/llama_hqe.py:235-239).  -> (ratio_e, ratio_q), float32 as in the reference (numpy scalars, see above)."""
     added = (history + BLOCK) // BLOCK * BLOCK - history
-    ratio_e = (added * ratio_e_0) / (history + added)
-    return ratio_e, (1 - ratio_e) * ratio_q / ratio_q.sum()
+    ratio_e = (_F32(added) * ratio_e_0.numpy()) / _F32(history + added)
+    rq = ratio_q.numpy()
+    total = rq[0]
+    for x in rq[1:]:
+        total = total + x
+    return torch.from_numpy(ratio_e), torch.from_numpy((_F32(1) - ratio_e) * rq / total)
 
 
 class HqeAttentionLayer:
@@ -241,7 +260,7 @@ class HqeAttentionLayer:
         importance = self.last_weights.calculate_token_importance()[:total_length].clone()
         # ranks the blocks AND divides `importance` by the block length in place, as the reference's helper
         # does; the policy below is handed the divided values [226-231]
-        K_token_idx = get_block_token_idx(BLOCK, total_length // BLOCK, importance)
+        K_token_idx = rank_blocks(BLOCK, total_length // BLOCK, importance)   # (spelt out as tokens only on demand)
         past_key_value = KV_cache_hqe_2(past_key_value, compress_length, self.history_reserve_length,
                                         K_token_idx, K_bit_num, V_bit_num, importance,
                                         self.quant_strategy, self.last_weights, BLOCK, BLOCK, self.times_range)

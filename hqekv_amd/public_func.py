@@ -22,7 +22,8 @@ def calculate_new_token_range(new_cache: Optional[torch.Tensor]):
     """Per-token (max_d - min_d) summed over batch and heads."""
     if new_cache is None:
         return None
-    return (torch.max(new_cache, dim=-1)[0] - torch.min(new_cache, dim=-1)[0]).sum(0).sum(0)
+    lo, hi = torch.aminmax(new_cache, dim=-1)
+    return (hi - lo).sum(0).sum(0)
 
 
 def calculate_token_range(new_cache: Optional[torch.Tensor], token_range: Optional[torch.Tensor]):
@@ -43,19 +44,67 @@ def get_block_importance(block_size: int, block_num: int, importance: torch.Tens
     return torch.sum(b, dim=-1)
 
 
+class RankedBlocks:
+    """A block ranking that has not been spelt out yet: ``scores`` holds the mean importance of every block,
+    ``order`` (made on first use) the block numbers, most important first -- a stable descending sort, so the
+    order is a function of the scores alone and whoever holds two rankings may sort them in one call.  The cache
+    policy plans from the block order; ``tokens()`` builds the token list the reference's helper returns (and
+    remembers it).  Reads like a tensor where the policy looks: ``numel()``, and the block order riding along under
+    the names it rides along with on a token list."""
+    __slots__ = ("scores", "block_size", "_order", "_tokens")
+    _version = 0                    # nobody can have written into positions that do not exist yet
+    _hq_block_order_version = 0
+
+    def __init__(self, scores: torch.Tensor, block_size: int):
+        self.scores, self.block_size, self._order, self._tokens = scores, block_size, None, None
+
+    @property
+    def order(self) -> torch.Tensor:
+        if self._order is None:
+            self._order = torch.sort(self.scores, descending=True, stable=True)[1]
+        return self._order
+
+    @staticmethod
+    def sort_together(a: "RankedBlocks", b: "RankedBlocks") -> torch.Tensor:
+        """Both orders from one sort call, as a (2, blocks) tensor; rows are what each would get alone."""
+        if a._order is None and b._order is None and a.scores.shape == b.scores.shape \
+                and a.scores.device == b.scores.device and a.scores.dtype == b.scores.dtype:
+            both = torch.sort(torch.stack((a.scores, b.scores)), dim=1, descending=True, stable=True)[1]
+            a._order, b._order = both[0], both[1]
+            return both
+        return torch.stack((a.order, b.order))
+
+    @property
+    def _hq_block_order(self):
+        return self.order, self.block_size
+
+    def numel(self) -> int:
+        return self.scores.numel() * self.block_size
+
+    def tokens(self) -> torch.Tensor:
+        if self._tokens is None:
+            order, bs = self.order, self.block_size
+            ar = torch.arange(bs, dtype=order.dtype, device=order.device)
+            idx = (order.reshape(-1, 1) * bs + ar.reshape(1, -1)).flatten()
+            # the block order rides along: the cache policy needs the ranking on the host and fetches these
+            # block_num entries instead of block_num * block_size
+            idx._hq_block_order = (order, bs)
+            idx._hq_block_order_version = idx._version   # ignored once somebody writes into idx
+            self._tokens = idx
+        return self._tokens
+
+
+def rank_blocks(block_size: int, block_num: int, importance: torch.Tensor) -> RankedBlocks:
+    """The ranking of ``get_block_token_idx`` without the token list (same in-place divide of ``importance``)."""
+    return RankedBlocks(get_block_importance(block_size, block_num, importance), block_size)
+
+
 def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tensor) -> torch.Tensor:
     """Token indices of the blocks ordered by descending mean importance, tokens inside a block in order
     (model/public_func.py:92-106, including the in-place divide of ``importance``).  The sort is stable --
     equal block scores keep their original order -- where the reference leaves the order of ties to the
     device sort."""
-    _, order = torch.sort(get_block_importance(block_size, block_num, importance), descending=True, stable=True)
-    ar = torch.arange(block_size, dtype=order.dtype, device=order.device)
-    idx = (order.reshape(-1, 1) * block_size + ar.reshape(1, -1)).flatten()
-    # the block order rides along: the cache policy needs the ranking on the host and fetches these
-    # block_num entries instead of block_num * block_size
-    idx._hq_block_order = (order, block_size)
-    idx._hq_block_order_version = idx._version   # ignored once somebody writes into idx
-    return idx
+    return rank_blocks(block_size, block_num, importance).tokens()
 
 
 def make_sum_equal(array: torch.Tensor, array_sum: int, start_idx: int = 4) -> torch.Tensor:
@@ -91,6 +140,7 @@ class last_attn_weights:
         self.kv_seq_len = 0
         self.next_line = 0
         self.weights = None
+        self._seen = None
 
     def set_max_length(self, max_length: int) -> None:
         self.max_length = max_length
@@ -101,9 +151,14 @@ class last_attn_weights:
 
     def calculate_token_importance(self) -> torch.Tensor:
         n, w = self.kv_seq_len, self.weights
-        # column j has been seen by min(last_length, n - j) rows: the newest tokens by fewer than all of them
-        seen = torch.clamp(n - torch.arange(n, device=w.device), max=self.last_length).to(w.dtype)
-        return w[:, :n].sum(0) / seen
+        # column j has been seen by min(last_length, n - j) rows: the newest tokens by fewer than all of them.
+        # One vector made once serves every n: r[i] = min(last_length, len(r) - i), and the counts for n columns are
+        # its last n entries.
+        r = self._seen
+        if r is None or r.shape[0] < n or r.device != w.device or r.dtype != w.dtype:
+            m = max(n, w.shape[1])
+            r = self._seen = torch.clamp(m - torch.arange(m, device=w.device), max=self.last_length).to(w.dtype)
+        return w[:, :n].sum(0) / r[r.shape[0] - n:]
 
     def eviction(self, reserve_idx: torch.Tensor) -> None:
         """Keep the columns ``reserve_idx`` (ascending positions of the survivors), packed to the left."""

@@ -185,3 +185,29 @@ def test_cover_once_verdict_is_not_reused_for_other_tensors():
     b[5] = 69
     assert idx_cover_once([a, b], 128)
     assert not idx_cover_once([a, b], 129) and not idx_cover_once([a], 128)
+
+
+def test_class_sizes_and_ratio_update_equal_the_tensor_arithmetic():
+    """The layer's class sizes and ratio update run on numpy float32 scalars; the reference does the same float32
+    operations on CPU tensors (model/llama_hqe.py:216-224,235-239), restated in the oracle: same shares, same counts,
+    same ratios, bit for bit, over random ratios, histories and lengths."""
+    import random
+    from hqekv_amd.decode_layer import class_token_counts, ratios_for_next_increment
+    rnd = random.Random(7)
+    for _ in range(3000):
+        total = rnd.choice([32, 64, 96, 128, 320, 1024, 26208, 32768, 131072, rnd.randrange(1, 5000) * 32])
+        b0 = rnd.random() * 0.5
+        a, c, d = rnd.random(), rnd.random(), rnd.random() * rnd.choice([0, 1])
+        e0 = torch.tensor([b0], dtype=torch.float32)
+        rq = torch.tensor([a, c, d], dtype=torch.float32) * ((1 - b0) / (a + c + d))
+        hist = rnd.randrange(0, 4000) * 32
+        add = (hist + 32) // 32 * 32 - hist
+        re_t = (add * e0) / (hist + add)                       # the reference's lines, on tensors
+        rq_t = (1 - re_t) * rq / rq.sum()
+        re_n, rq_n = ratios_for_next_increment(hist, e0, rq)
+        assert torch.equal(re_t, re_n) and torch.equal(rq_t, rq_n), (hist, b0, a, c, d)
+        shares_o, counts_o = O.split_history(total, rq_t, re_t)
+        shares_n, counts_n = class_token_counts(total, rq_n, re_n)
+        assert torch.equal(shares_o, shares_n) and torch.equal(counts_o, counts_n), (total, b0, a, c, d)
+        assert counts_n.dtype == counts_o.dtype and shares_n.dtype == torch.float32
+        assert int(counts_n.sum()) == total // 32 * 32 and bool((counts_n % 32 == 0).all())
