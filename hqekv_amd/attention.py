@@ -275,6 +275,7 @@ class SegmentMemo:
         self.dims = (None, None)
         self.partition = False                 # the classes' position arrays cover [0, kept) once per side
         self._step = None                      # what step_call keeps between steps
+        self._spare = None                     # (attn_weights, attn_output) allocated ahead for the next step
 
     def lookup(self, pkv: tuple, dev, low_uniform: bool) -> bool:
         held = self.held
@@ -341,14 +342,16 @@ class SegmentMemo:
         return self.ws
 
     def step_call(self, q: torch.Tensor, pkv: tuple, Tall: int, k: torch.Tensor, v: torch.Tensor, res, n: int,
-                  ring_store: Optional[torch.Tensor], ring_row: int, low_uniform: bool):
+                  ring_store: Optional[torch.Tensor], ring_row: int, low_uniform: bool, known: bool = False):
         """One decode step of a layer as one C call (``hqekv_decode_step``) with as little host work as the call
         allows: the class entries of the tables are the memo's, the residual is the first ``n`` token rows of the
         capacity buffers ``res`` = (K, V), this step's ``k`` / ``v`` (B,Hkv,L,D, dense) are read as a segment of
         their own and copied to row ``n`` of the buffers, and -- when ``ring_store`` (rows x max_length, fp16) is
-        given -- row ``ring_row`` of it receives the ring row.  -> (attn_weights, attn_output)."""
+        given -- row ``ring_row`` of it receives the ring row.  ``known``: the caller vouches that ``pkv`` carries the
+        class tensors the tables were built from (it is the tuple the previous step returned).
+        -> (attn_weights, attn_output)."""
         dev = q.device
-        if not self.lookup(pkv, dev, low_uniform):
+        if not (known and self.held is not None) and not self.lookup(pkv, dev, low_uniform):
             self.build(pkv, dev, low_uniform)
         B, Hq, _, D = q.shape
         Hkv, L = k.shape[1], k.shape[2]
@@ -381,8 +384,13 @@ class SegmentMemo:
         n_k += 1
         n_v += 1
         # (positions nobody writes must read as zero when the classes do not cover every position)
-        weights = (torch.empty if self.partition else torch.zeros)(B, Hq, 1, Tall, dtype=torch.float16, device=dev)
-        out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev)
+        spare, self._spare = self._spare, None
+        if spare is not None and self.partition and spare[0].shape == (B, Hq, 1, Tall) and spare[1].shape == (B, Hq, 1, D) \
+                and spare[0].device == dev:
+            weights, out = spare   # allocated while the previous step's kernels were running
+        else:
+            weights = (torch.empty if self.partition else torch.zeros)(B, Hq, 1, Tall, dtype=torch.float16, device=dev)
+            out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev)
         if ring_store is not None:
             x.ring_line = ring_store.data_ptr() + 2 * ring_row * ring_store.shape[1]
             x.ring_order = 2 if (Tall % 4 == 0 and Tall >= 256 and weights.data_ptr() % 8 == 0) else 1
@@ -407,6 +415,9 @@ class SegmentMemo:
                 if rc != -3:   # HQEKV_E_WORKSPACE: the cache has outgrown the workspace kept from earlier steps
                     break
         _lib.check(rc, "decode_step")
+        if self.partition:   # the next step's outputs, one position longer: off that step's path to its first launch
+            self._spare = (torch.empty(B, Hq, 1, Tall + L, dtype=torch.float16, device=dev),
+                           torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev))
         return weights, out
 
 

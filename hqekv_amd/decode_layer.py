@@ -125,6 +125,7 @@ class HqeAttentionLayer:
         self._res = None             # (K buffer, V buffer): the fp16 residual in capacity-sized storage
         self.fused_step = True       # ring row and residual appends inside the attention call (False: separate launches)
         self._own_tuple = False      # the tuple handed in carries the class tensors this layer built its tables from
+        self._returned = None        # (the tuple the last plain decode step returned, tokens in its residual)
 
     def reset(self) -> None:
         """What the reference's ``generate`` does per layer before a new prompt [555-557]."""
@@ -135,6 +136,7 @@ class HqeAttentionLayer:
         self.last_weights.reset()
         self._memo = SegmentMemo()
         self._res = None
+        self._returned = None
 
     def set_max_length(self, max_length: int) -> None:
         """Prompt length + new tokens: the width of the importance ring [691-695]."""
@@ -199,8 +201,15 @@ class HqeAttentionLayer:
             # The attention reads this step's key and value where they are, as a segment behind the residual, and
             # is queued first; the copies that append them to the residual [131-133] follow it on the stream, off
             # the step's critical path.
-            past_key_value = self._residual_in_buffers(past_key_value, key_states)
-            n = past_key_value[-3].shape[2] if past_key_value[-3] is not None else 0
+            back = self._returned
+            known = (back is not None and back[0] is past_key_value and self._res is not None
+                     and back[1] + L <= self._res[0].shape[2])
+            if known:   # the very tuple the previous step handed out: its residual is the head of the buffers
+                n, self._own_tuple = back[1], True
+            else:
+                past_key_value = self._residual_in_buffers(past_key_value, key_states)
+                n = past_key_value[-3].shape[2] if past_key_value[-3] is not None else 0
+            self._returned = None
             # tokens the classes hold = the history this layer has kept; a tuple from elsewhere is counted
             Tall = (self.history_reserve_length if self._own_tuple else value_length(past_key_value) - n) + n + L
             lw = self.last_weights
@@ -225,7 +234,7 @@ class HqeAttentionLayer:
                     lw.decode_row(query_states, Tall)   # creates the store
                 attn_weights, attn_output = self._memo.step_call(
                     query_states, past_key_value, Tall, key_states, value_states, self._res, n,
-                    lw.weights if on_device else None, lw.next_line, self.quant_strategy == "uniform_group")
+                    lw.weights if on_device else None, lw.next_line, self.quant_strategy == "uniform_group", known)
             else:
                 attn_weights, attn_output = qkv_matmul_hqe_2(query_states, past_key_value, attention_mask,
                                                              self.head_dim, self.quant_strategy, memo=self._memo,
@@ -239,6 +248,8 @@ class HqeAttentionLayer:
                 self._res[1][:, :, n:n + L].copy_(value_states)
             new_K, new_V = self._res[0][:, :, :n + L], self._res[1][:, :, :n + L]
             past_key_value = past_key_value[:-3] + (new_K, new_V, kv_seq_len)
+            if plain_inputs:
+                self._returned = (past_key_value, n + L)
         else:
             attn_weights, attn_output = self._prefill(query_states, key_states, value_states, attention_mask)
             past_key_value = (None,) * 39 + (key_states, value_states, kv_seq_len)
@@ -248,6 +259,7 @@ class HqeAttentionLayer:
             self.token_num += 1
             return attn_output, attn_weights, past_key_value, None
 
+        self._returned = None   # what follows builds another tuple
         # whole blocks of the un-quantised tokens join the history; the rest stays the fp16 residual
         compress_length = self.current_length // BLOCK * BLOCK
         total_length = self.history_reserve_length + compress_length
