@@ -33,7 +33,7 @@ import numpy as np
 import torch
 
 from . import pack_unpack as PU
-from .public_func import RankedBlocks, calculate_token_range, get_block_token_idx, rank_blocks
+from .public_func import RankedBlocks, calculate_token_range, get_block_token_idx, rank_blocks_weighted
 
 BLOCK = 32
 CLASS_BITS = (16, 8, 4, 2, 1)
@@ -651,8 +651,8 @@ def compress(past_key_value: tuple, compress_length: int, history_length, K_sort
     block_num = total // BLOCK
 
     V_norm = V_token_range if V_token_range is not None else calculate_token_range(new_V, pkv[38])
-    V_score = token_importance * V_norm if times_range else token_importance.clone()
-    V_sorted_idx = rank_blocks(BLOCK, block_num, V_score)   # the token list is spelt out only if the step engine runs
+    # (the token list is spelt out only if the step engine runs)
+    V_sorted_idx = rank_blocks_weighted(block_num, token_importance, V_norm if times_range else None)
 
     dev = new_V.device
     engine = engine or os.environ.get("HQEKV_POLICY_ENGINE", "auto")

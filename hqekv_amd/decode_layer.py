@@ -25,7 +25,7 @@ import torch
 from .attention import SegmentMemo, value_length
 from .hqe_2 import KV_cache_hqe_2
 from .hqe_matmul import qkv_matmul_hqe_2
-from .public_func import last_attn_weights, rank_blocks
+from .public_func import last_attn_weights
 
 LAST_TOKEN_NUM = 20
 BLOCK = 32
@@ -269,10 +269,9 @@ class HqeAttentionLayer:
         else:
             shares, K_bit_num = class_token_counts(total_length, self.ratio_q, self.ratio_e)
             V_bit_num = K_bit_num.clone()
-        importance = self.last_weights.calculate_token_importance()[:total_length].clone()
-        # ranks the blocks AND divides `importance` by the block length in place, as the reference's helper
-        # does; the policy below is handed the divided values [226-231]
-        K_token_idx = rank_blocks(BLOCK, total_length // BLOCK, importance)   # (spelt out as tokens only on demand)
+        # the importance of every token and the ranking of the blocks; like the reference's ranking helper, which
+        # divides its argument by the block length in place, this leaves the policy the divided values [226-231]
+        importance, K_token_idx = self.last_weights.ranked_importance(total_length)
         past_key_value = KV_cache_hqe_2(past_key_value, compress_length, self.history_reserve_length,
                                         K_token_idx, K_bit_num, V_bit_num, importance,
                                         self.quant_strategy, self.last_weights, BLOCK, BLOCK, self.times_range)

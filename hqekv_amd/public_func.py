@@ -18,10 +18,33 @@ def calculate_token_norm(new_cache: Optional[torch.Tensor], token_norm: Optional
     return n if token_norm is None else torch.cat((token_norm, n), dim=-1)
 
 
+def _token_major_slabs(x: torch.Tensor):
+    """Tokens between two (b, h) slabs of a (B, H, T, D) tensor whose rows are dense and whose slabs are equally
+    spaced (a dense tensor, or the head of a capacity buffer), else None."""
+    B, H, T, D = x.shape
+    sb, sh, st, sd = x.stride()
+    if sd != 1 or st != D or sh % D or sh < T * D or (B > 1 and sb != H * sh):
+        return None
+    return sh // D
+
+
 def calculate_new_token_range(new_cache: Optional[torch.Tensor]):
-    """Per-token (max_d - min_d) summed over batch and heads."""
+    """Per-token (max_d - min_d) summed over batch and heads (model/public_func.py:58-66): on the device one launch of
+    ``hqekv_token_range``, which adds in torch's own order."""
     if new_cache is None:
         return None
+    if new_cache.is_cuda and new_cache.dtype == torch.float16 and new_cache.dim() == 4 and new_cache.numel() \
+            and new_cache.shape[0] * new_cache.shape[1] <= 1024:
+        slab = _token_major_slabs(new_cache)
+        if slab is not None:
+            from . import _lib
+            B, H, T, D = new_cache.shape
+            out = torch.empty(T, dtype=torch.float16, device=new_cache.device)
+            with _lib.on_device(new_cache.device):
+                rc = _lib.load().hqekv_token_range(new_cache.data_ptr(), B, H, T, D, slab, out.data_ptr(),
+                                                   _lib.stream_ptr(new_cache.device))
+            _lib.check(rc, "token_range")
+            return out
     lo, hi = torch.aminmax(new_cache, dim=-1)
     return (hi - lo).sum(0).sum(0)
 
@@ -99,6 +122,25 @@ def rank_blocks(block_size: int, block_num: int, importance: torch.Tensor) -> Ra
     return RankedBlocks(get_block_importance(block_size, block_num, importance), block_size)
 
 
+def rank_blocks_weighted(block_num: int, importance: torch.Tensor, weights: Optional[torch.Tensor]) -> RankedBlocks:
+    """The ranking of ``importance * weights`` (``importance`` alone without weights) in blocks of 32, the V side's
+    (quant/hqe_2.py:510-518); neither argument is modified.  On the device one launch of
+    ``hqekv_weighted_block_scores`` in place of the product, the divide and the block sums."""
+    total = block_num * 32
+    if importance.is_cuda and importance.dtype == torch.float16 and importance.is_contiguous() \
+            and importance.numel() == total and total > 0 \
+            and (weights is None or (weights.is_cuda and weights.dtype == torch.float16 and weights.is_contiguous()
+                                     and weights.numel() == total)):
+        from . import _lib
+        scores = torch.empty(block_num, dtype=torch.float16, device=importance.device)
+        with _lib.on_device(importance.device):
+            rc = _lib.load().hqekv_weighted_block_scores(importance.data_ptr(), None if weights is None else weights.data_ptr(),
+                                                         total, scores.data_ptr(), _lib.stream_ptr(importance.device))
+        _lib.check(rc, "weighted_block_scores")
+        return RankedBlocks(scores, 32)
+    return rank_blocks(32, block_num, importance * weights if weights is not None else importance.clone())
+
+
 def get_block_token_idx(block_size: int, block_num: int, importance: torch.Tensor) -> torch.Tensor:
     """Token indices of the blocks ordered by descending mean importance, tokens inside a block in order
     (model/public_func.py:92-106, including the in-place divide of ``importance``).  The sort is stable --
@@ -159,6 +201,25 @@ class last_attn_weights:
             m = max(n, w.shape[1])
             r = self._seen = torch.clamp(m - torch.arange(m, device=w.device), max=self.last_length).to(w.dtype)
         return w[:, :n].sum(0) / r[r.shape[0] - n:]
+
+    def ranked_importance(self, total: int):
+        """What a compression needs from the ring for the first ``total`` tokens (a multiple of 32):
+        ``calculate_token_importance()[:total]`` divided by 32 -- the values ``get_block_token_idx`` leaves behind in
+        its argument, which the policy is handed (model/llama_hqe.py:226-231) -- and the ranking of the blocks by their
+        mean importance.  On the device one launch (``hqekv_importance_scores``) in place of the sum over the rows,
+        the divide by the counts, the copy, the in-place divide and the block sums.  -> (importance / 32, RankedBlocks)."""
+        n, w = self.kv_seq_len, self.weights
+        if w.is_cuda and w.dtype == torch.float16 and w.is_contiguous() and 0 < total <= n and total % 32 == 0:
+            from . import _lib
+            imp = torch.empty(total, dtype=torch.float16, device=w.device)
+            scores = torch.empty(total // 32, dtype=torch.float16, device=w.device)
+            with _lib.on_device(w.device):
+                rc = _lib.load().hqekv_importance_scores(w.data_ptr(), w.shape[0], w.shape[1], n, total, imp.data_ptr(),
+                                                         scores.data_ptr(), _lib.stream_ptr(w.device))
+            _lib.check(rc, "importance_scores")
+            return imp, RankedBlocks(scores, 32)
+        imp = self.calculate_token_importance()[:total].clone()
+        return imp, rank_blocks(32, total // 32, imp)
 
     def eviction(self, reserve_idx: torch.Tensor) -> None:
         """Keep the columns ``reserve_idx`` (ascending positions of the survivors), packed to the left."""

@@ -312,6 +312,25 @@ int hqekv_decode_step(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs,
 int hqekv_ring_row(const void *attn_weights, int64_t B, int64_t Hq, int64_t Tall, void *line, int order,
                    void *stream);
 
+/* What the cache policy ranks blocks by (model/public_func.py:217-221 calculate_token_importance, :85-106
+ * get_block_importance / get_block_token_idx with its in-place divide, quant/hqe_2.py:510-518 the V ranking's
+ * importance * range, model/public_func.py:58-73 calculate_token_range), one launch each instead of a chain of torch
+ * reductions.  All tensors fp16; every rounding and every order of additions is the one torch's GPU kernels use for
+ * these shapes (rows of a matrix: one walker per column, four interleaved fp32 accumulators; 32 contiguous values: a
+ * balanced tree over adjacent pairs), pinned against torch on the device.
+ *   hqekv_importance_scores   ring (rows x max_len, row stride max_len): importance_out[c] = (sum of column c /
+ *                             min(rows, n - c)) / 32 for c < total -- the values the ranking helper leaves behind in
+ *                             its argument -- and scores_out[b] = sum of block b's 32 values (total = 32 * blocks <= n)
+ *   hqekv_weighted_block_scores  scores_out[b] = sum over block b of (x[c] * weights[c]) / 32; weights NULL: x[c] / 32
+ *   hqekv_token_range         v (B, H, T, D) fp16 token-major, slabs slab_tokens * D elements apart:
+ *                             out[t] = sum_h sum_b (max_d v - min_d v), each sum rounded to fp16
+ */
+int hqekv_importance_scores(const void *ring, int32_t rows, int64_t max_len, int64_t n, int64_t total,
+                            void *importance_out, void *scores_out, void *stream);
+int hqekv_weighted_block_scores(const void *x, const void *weights, int64_t total, void *scores_out, void *stream);
+int hqekv_token_range(const void *v, int64_t B, int64_t H, int64_t T, int64_t D, int64_t slab_tokens, void *out,
+                      void *stream);
+
 /* ------------------------------------------------------------------ cache maintenance (one launch per side)
  * Replaces the per-(source, target) gathers, dequantise / re-quantise calls and torch.cat re-copies of one
  * compression -- V_high_2_eviction / K_high_2_eviction (quant/hqe_2.py:44-86), quant_new_K (:16-42), K_high_2_low

@@ -141,3 +141,94 @@ def test_layer_step_in_one_call_equals_the_separate_launches(dev, B, T0):
             else:
                 assert a == b, (where, i)
     assert compressions >= 2
+
+
+# ------------------------------------------------------------------ what the policy ranks blocks by
+def _ring_with_cancelling_columns(n, max_len, g, dev):
+    """A 20-row ring store whose column sums are small everywhere except for pairs of columns inside every block of 32
+    that hold +big and -big: the block sums then depend on the order the 32 values are added in, the column sums (big
+    values that cancel between rows, as in ``_order_sensitive``) on the order of the rows."""
+    X = _order_sensitive(1, 20, n, g)[0, :, 0].float()          # (20, n)
+    for b0 in range(0, n - 31, 32):
+        i, j = (torch.randperm(32, generator=g)[:2] + b0).tolist()
+        big = float(torch.randint(1024, 2048, (1,), generator=g)) / 8.0
+        X[:, i] = 0
+        X[:, j] = 0
+        X[3, i], X[3, j] = big, -big
+    store = torch.zeros(20, max_len, dtype=torch.float16, device=dev)
+    store[:, :n] = X.half().to(dev)
+    return store
+
+
+@pytest.mark.parametrize("max_len,n", [(600, 33), (600, 64), (4099, 320), (4099, 4064 + 5), (32968, 26240),
+                                       (32968, 26208 + 19), (131500, 104864)])
+def test_importance_and_block_scores_equal_torch_chain_on_device(dev, max_len, n):
+    """``ranked_importance`` / ``rank_blocks_weighted`` (one launch each) against the chain of torch operations they
+    stand for -- sum over the ring's rows, divide by the counts, copy, divide by 32 in place, sum the blocks; multiply
+    with the V ranges, divide, sum -- executed by torch on the device: importance, scores and order bit for bit."""
+    from hqekv_amd.public_func import get_block_importance, last_attn_weights, rank_blocks_weighted
+    g = torch.Generator().manual_seed(n)
+    total, nb = n // 32 * 32, n // 32
+    ring = last_attn_weights()
+    ring.set_max_length(max_len)
+    ring.weights = _ring_with_cancelling_columns(n, max_len, g, dev)
+    ring.kv_seq_len = n
+    imp_t = ring.calculate_token_importance()[:total].clone()
+    sc_t = get_block_importance(32, nb, imp_t)                    # divides imp_t in place, like the reference's helper
+    imp_k, ranked = ring.ranked_importance(total)
+    torch.cuda.synchronize()
+    assert torch.equal(imp_k.view(torch.int16), imp_t.view(torch.int16))
+    assert torch.equal(ranked.scores.view(torch.int16), sc_t.view(torch.int16))
+    assert torch.equal(ranked.order, torch.sort(sc_t, descending=True, stable=True)[1])
+    # the V side: importance (already divided) times the token ranges, divided again, summed per block
+    vn = (torch.rand(total, generator=g) * 40 + 0.01).half().to(dev)
+    for w in (vn, None):
+        v_t = imp_t * w if w is not None else imp_t.clone()
+        sv_t = get_block_importance(32, nb, v_t)
+        kept = imp_k.clone()
+        rw = rank_blocks_weighted(nb, imp_k, w)
+        torch.cuda.synchronize()
+        assert torch.equal(rw.scores.view(torch.int16), sv_t.view(torch.int16))
+        assert torch.equal(imp_k, kept) and (w is None or torch.equal(w, vn))      # arguments untouched
+
+
+@pytest.mark.parametrize("B,H,T,cap", [(1, 8, 32, 0), (2, 8, 32, 96), (3, 4, 64, 0), (4, 8, 300, 0), (8, 8, 33, 64),
+                                       (1, 2, 32, 0), (5, 3, 1, 0), (2, 8, 4099, 0)])
+def test_token_range_equals_torch_chain_on_device(dev, B, H, T, cap):
+    """``hqekv_token_range`` against (max - min over channels).sum(0).sum(0) executed by torch on the device, bit for
+    bit: random tokens, and tokens whose ranges span 25 binades so that fp32 sums lose low bits in an order-dependent
+    way; dense tensors and heads of capacity buffers."""
+    from hqekv_amd.public_func import calculate_new_token_range
+    g = torch.Generator().manual_seed(B * 100 + H * 10 + T)
+    D = 128
+    for kind in ("random", "wide"):
+        x = torch.randn(B, H, T, D, generator=g)
+        if kind == "wide":
+            x = torch.zeros(B, H, T, D)
+            x[..., 5] = torch.exp2(torch.randint(-10, 16, (B, H, T), generator=g).float()) * \
+                (torch.randint(1024, 2048, (B, H, T), generator=g).float() / 1024.0)
+        x = x.half()
+        if cap:
+            buf = torch.zeros(B, H, cap + T, D, dtype=torch.float16, device=dev)
+            buf[:, :, :T] = x.to(dev)
+            xd = buf[:, :, :T]
+        else:
+            xd = x.to(dev)
+        expect = (torch.max(xd, dim=-1)[0] - torch.min(xd, dim=-1)[0]).sum(0).sum(0)
+        got = calculate_new_token_range(xd)
+        torch.cuda.synchronize()
+        assert got.shape == expect.shape and got.dtype == expect.dtype
+        assert torch.equal(got.view(torch.int16), expect.view(torch.int16)), (kind, B, H, T)
+
+
+def test_policy_score_entries_reject_bad_arguments(dev):
+    from hqekv_amd import _lib
+    lib = _lib.load()
+    a = torch.zeros(20, 64, dtype=torch.float16, device=dev)
+    o = torch.zeros(64, dtype=torch.float16, device=dev)
+    assert lib.hqekv_importance_scores(a.data_ptr(), 20, 64, 64, 48, o.data_ptr(), o.data_ptr(), None) == -1   # not whole blocks
+    assert lib.hqekv_importance_scores(a.data_ptr(), 20, 64, 32, 64, o.data_ptr(), o.data_ptr(), None) == -1   # total > n
+    assert lib.hqekv_importance_scores(None, 20, 64, 64, 64, o.data_ptr(), o.data_ptr(), None) == -1
+    assert lib.hqekv_weighted_block_scores(o.data_ptr(), None, 33, o.data_ptr(), None) == -1
+    assert lib.hqekv_token_range(a.data_ptr(), 1, 1, 8, 128, 4, o.data_ptr(), None) == -1                      # slab < T
+    assert lib.hqekv_token_range(a.data_ptr(), 40, 40, 8, 128, 8, o.data_ptr(), None) == -4                    # B * H > 1024
