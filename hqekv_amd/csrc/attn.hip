@@ -48,7 +48,7 @@ struct SegDev {
   int32_t layout;      // HQEKV_LAYOUT_*: 1 = fp16 K stored token-major, 2 = 1-bit normal-quantile coding
   int32_t unit_begin;  // first chunk of this segment in the p.V partial buffer
   int32_t n_units;     // tiles (q.K^T) or chunks (p.V) of this segment
-  int64_t slab_tokens; // token rows between two (b, kv head) slabs of a token-major fp16 segment (>= n_tokens)
+  int64_t slab_tokens; // token rows between two (b, kv head) slabs of a token-major segment (>= n_tokens)
 };
 
 struct SegTable {
@@ -1547,8 +1547,8 @@ __device__ __forceinline__ void pv_fetch(const SegDev &sg, int64_t t0, int nt, i
     pr.pb = sg.idx[tb2];
   }
   if (QUANT) {  // a V class may hold any number of tokens: the last pair of an odd count reads row a twice
-    const uint2 *sc = reinterpret_cast<const uint2 *>(sg.scale + ((int64_t)bh * sg.n_tokens + ta) * NG);
-    const uint2 *zr = reinterpret_cast<const uint2 *>(sg.zero + ((int64_t)bh * sg.n_tokens + ta) * NG);
+    const uint2 *sc = reinterpret_cast<const uint2 *>(sg.scale + ((int64_t)bh * sg.slab_tokens + ta) * NG);
+    const uint2 *zr = reinterpret_cast<const uint2 *>(sg.zero + ((int64_t)bh * sg.slab_tokens + ta) * NG);
     const int second = (int)(tb2 - ta);
     pr.sa = sc[0];
     pr.sb = sc[second];
@@ -1635,7 +1635,7 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
   const int g = cl >> 2;
   const int sh2 = (BITS == 2) ? (cl & 1) * 16 : (BITS == 1) ? (cl & 3) * 8 : 0;
   const uint32_t wofs = (BITS == 1 ? (cl >> 2) : BITS == 2 ? (cl >> 1) : cl * WPL) * 4u;  // byte offset inside a token row
-  const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * (BITS == 16 ? sg.slab_tokens : sg.n_tokens) * ROWB,
+  const rsrc_t rc = make_rsrc((const char *)sg.data + (int64_t)bh * sg.slab_tokens * ROWB,
                               (uint32_t)(sg.n_tokens * ROWB));
   const uint32_t lane_off = (uint32_t)(2 * tl) * ROWB + wofs;   // this lane's first token of a step + word
 
@@ -2205,9 +2205,10 @@ static int build_table(const hqekv_seg *segs, int nseg, bool is_k, int64_t D, in
       return fail(HQEKV_E_ALIGN, "%s: segment %d fp16 data must be 16-byte aligned", who, k);
     if (s.n_tokens * D >= (1LL << 31))
       return fail(HQEKV_E_UNSUPPORTED, "%s: segment %d: n_tokens * D must stay below 2^31 per (b, head) slab", who, k);
-    const bool token_major_f16 = s.bits == 16 && (is_k ? s.layout == HQEKV_LAYOUT_TOKEN_MAJOR : true);
-    if (s.slab_tokens != 0 && (s.slab_tokens < s.n_tokens || !token_major_f16))
-      return fail(HQEKV_E_ARG, "%s: segment %d: slab_tokens applies to token-major fp16 segments and must be >= n_tokens", who, k);
+    // (every V class is token-major; on the K side only the fp16 residual is)
+    const bool token_major = is_k ? (s.bits == 16 && s.layout == HQEKV_LAYOUT_TOKEN_MAJOR) : true;
+    if (s.slab_tokens != 0 && (s.slab_tokens < s.n_tokens || !token_major))
+      return fail(HQEKV_E_ARG, "%s: segment %d: slab_tokens applies to token-major segments and must be >= n_tokens", who, k);
     SegDev &d = tb->seg[m++];
     d.data = s.data;
     d.scale = (const half_t *)s.scale;

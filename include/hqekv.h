@@ -183,9 +183,9 @@ typedef struct hqekv_seg {
   const void *scale;     /* NULL when bits == 16                                       */
   const void *zero;
   const int64_t *idx;    /* (n_tokens) or NULL                                         */
-  int64_t slab_tokens;   /* token-major fp16 segments only (the residual, the fp16 V class): token rows between two
-                            (b, kv head) slabs in memory when the segment is the head of a longer, capacity-sized
-                            buffer; 0 = n_tokens (dense)                                */
+  int64_t slab_tokens;   /* token-major segments only (the fp16 residual of either side, every V class -- codes, scale
+                            and zero alike): token rows between two (b, kv head) slabs in memory when the segment is a
+                            window of a longer, capacity-sized buffer; 0 = n_tokens (dense)        */
 } hqekv_seg;
 
 /* Replaces gemv_forward_cuda_qk_group_hq (quant/csrc/gemv_cuda.h:78-109; kernel

@@ -76,6 +76,36 @@ def test_kivi_layer_in_lockstep_with_oracle(dev, B, Hq, Hkv, T0, steps, k_bits, 
     assert n_vq + pkv_g[5].shape[2] == T0 + steps and pkv_g[5].shape[2] <= R
 
 
+def test_kivi_in_place_steps_grow_slide_and_mix_with_the_plain_sequence(dev, monkeypatch):
+    """The in-place decode step with tiny buffers -- the V class outgrows its capacity several times, the V tail window
+    wraps -- and with steps of upstream's plain sequence in between (an all-zero additive mask sends a step there; the
+    next step takes the tuple over into fresh buffers): the tuples stay bit-identical to the oracle's, and a second
+    layer that only ever runs the plain sequence sees the same tuples and outputs."""
+    from hqekv_amd.kivi_layer import KiviAttentionLayer
+    monkeypatch.setattr(KiviAttentionLayer, "MIN_V_ROWS", 8)
+    B, Hq, Hkv, T0, steps, R = 2, 8, 2, 45, 150, 32
+    fast, plain = KiviAttentionLayer(D, 2, 2, 32, R), KiviAttentionLayer(D, 2, 2, 32, R)
+    plain.in_place = False
+    orc = O.KiviLayerOracle(D, 2, 2, 32, R)
+    pf = pp = po = None
+    for step in range(steps + 1):
+        L = T0 if step == 0 else 1
+        q, k, v = _qkv(B, Hq, Hkv, L, 5200 + step)
+        mask = None
+        if step in (7, 8, 60, 111):
+            mask = torch.zeros(B, 1, 1, T0 + step, dtype=torch.float16, device=dev)
+        out_f, w_f, pf = fast(q.to(dev), k.to(dev), v.to(dev), mask, pf)
+        out_p, w_p, pp = plain(q.to(dev), k.to(dev), v.to(dev), mask, pp)
+        _, _, po = orc.step(q, k, v, None, po, observed=None if step == 0 else w_f.cpu())
+        where = f"step {step}"
+        _same_tuple(pf, po, where)
+        _same_tuple(pp, po, where)
+        if step and mask is None:
+            assert torch.allclose(w_f.float(), w_p.float(), rtol=RTOL, atol=ATOL), where
+            assert torch.allclose(out_f.float(), out_p.float(), rtol=RTOL, atol=ATOL), where
+    assert fast._st is not None and fast._st.vcode.shape[2] >= pf[4].shape[2] > 8 * 8   # grown more than once
+
+
 def test_kivi_decode_with_mask(dev):
     """An additive mask on a decode step takes the general path (scale, mask, clamp, softmax as its own launch)."""
     from hqekv_amd.kivi_layer import KiviAttentionLayer
