@@ -341,6 +341,8 @@ class SegmentMemo:
             self.ws = torch.empty(max(need + need // 8, 256) // 4, dtype=torch.float32, device=dev)
         return self.ws
 
+    SPARE_MAX_BYTES = 4 << 20   # largest attn_weights tensor that is allocated one step ahead
+
     def step_call(self, q: torch.Tensor, pkv: tuple, Tall: int, k: torch.Tensor, v: torch.Tensor, res, n: int,
                   ring_store: Optional[torch.Tensor], ring_row: int, low_uniform: bool, known: bool = False):
         """One decode step of a layer as one C call (``hqekv_decode_step``) with as little host work as the call
@@ -415,7 +417,9 @@ class SegmentMemo:
                 if rc != -3:   # HQEKV_E_WORKSPACE: the cache has outgrown the workspace kept from earlier steps
                     break
         _lib.check(rc, "decode_step")
-        if self.partition:   # the next step's outputs, one position longer: off that step's path to its first launch
+        # The next step's outputs, one position longer, allocated now: off that step's path to its first launch.  Only
+        # while they are small (every layer of a model holds its own): a long step does not notice the allocation.
+        if self.partition and B * Hq * (Tall + L) * 2 <= self.SPARE_MAX_BYTES:
             self._spare = (torch.empty(B, Hq, 1, Tall + L, dtype=torch.float16, device=dev),
                            torch.empty(B, Hq, 1, D, dtype=torch.float16, device=dev))
         return weights, out

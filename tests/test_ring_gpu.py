@@ -232,3 +232,41 @@ def test_policy_score_entries_reject_bad_arguments(dev):
     assert lib.hqekv_weighted_block_scores(o.data_ptr(), None, 33, o.data_ptr(), None) == -1
     assert lib.hqekv_token_range(a.data_ptr(), 1, 1, 8, 128, 4, o.data_ptr(), None) == -1                      # slab < T
     assert lib.hqekv_token_range(a.data_ptr(), 40, 40, 8, 128, 8, o.data_ptr(), None) == -4                    # B * H > 1024
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T", [(1, 32, 8, 2048 + 9), (4, 32, 8, 1024 + 3)])
+def test_step_extras_with_either_combine_route_and_dot_form(dev, B, Hq, Hkv, T):
+    """``hqekv_decode_step``'s ring row and appends ride in the combine launch -- or, when the combine is folded into
+    the p.V launch, in a launch of their own: both routes (forced by flag), with the dot products on the matrix cores
+    and on the vector ALU, give the ring row torch computes from the probabilities and the appended rows, and the
+    attention itself is the same bits as without the extras."""
+    from hqekv_amd import _lib, synth
+    from hqekv_amd.attention import decode_attention, value_length
+    from oracle import hqe_oracle as O
+    q, K, V = synth.make_qkv(B, Hq, Hkv, T, 128, 77 + B)
+    res = T % 32
+    classes = synth.split_blocks(T - res, (0.05, 0.15, 0.30, 0.30, 0.20), 5 + B)
+    cache = synth.cache_to(synth.build_cache(K, V, classes, res, O.uniform_group_quantize_pack_last_dim), dev)
+    Tall = value_length(cache) + 1                      # the step's own token rides as a tail segment
+    g = torch.Generator().manual_seed(3)
+    k_new = torch.randn(B, Hkv, 1, 128, generator=g).half().to(dev)
+    v_new = torch.randn(B, Hkv, 1, 128, generator=g).half().to(dev)
+    qd = q.to(dev)
+    for route in (_lib.SEPARATE_COMBINE, _lib.FOLD_COMBINE):
+        for dot in (_lib.DOT_MFMA, _lib.DOT_VALU):
+            flags = _lib.FUSE_SOFTMAX | route | dot
+            w0, o0 = decode_attention(qd, cache, None, Tall, zero_init=False, flags=flags, tail=(k_new, v_new))
+            kbuf = torch.zeros(B, Hkv, 64, 128, dtype=torch.float16, device=dev)
+            vbuf = torch.zeros_like(kbuf)
+            line = torch.full((Tall + 5,), -3.0, dtype=torch.float16, device=dev)
+            w1, o1 = decode_attention(qd, cache, None, Tall, zero_init=False, flags=flags, tail=(k_new, v_new),
+                                      step=dict(ring_line=line[1:Tall + 1], append=(kbuf, vbuf, 7)))
+            torch.cuda.synchronize()
+            where = (route, dot)
+            assert torch.equal(w0, w1) and torch.equal(o0, o1), where
+            assert torch.equal(line[1:Tall + 1].view(torch.int16), w1.sum(0).sum(0).reshape(Tall).view(torch.int16)), where
+            assert float(line[0]) == -3.0 and bool((line[Tall + 1:] == -3.0).all()), where
+            assert torch.equal(kbuf[:, :, 7], k_new[:, :, 0]) and torch.equal(vbuf[:, :, 7], v_new[:, :, 0]), where
+            kbuf[:, :, 7] = 0
+            vbuf[:, :, 7] = 0
+            assert not bool(kbuf.any()) and not bool(vbuf.any()), where   # nothing else written
