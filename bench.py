@@ -435,6 +435,7 @@ def measure_decode(workload: str, n_layers: int, K: int, W: int, args, dev):
     layers = build_layers(workload, n_layers, dev)
     plan_flags = default_flags() | _lib.qk_tiling(_lib.QK_TILINGS.get(args.qk_tiling, 0))
     plan_flags |= {"auto": 0, "mfma": _lib.DOT_MFMA, "valu": _lib.DOT_VALU}[args.dot]
+    plan_flags |= {"auto": 0, "fold": _lib.FOLD_COMBINE, "separate": _lib.SEPARATE_COMBINE}[args.combine]
     plans = [DecodePlan(q, cache, flags=plan_flags) for q, cache in layers]
     qs = [q.contiguous() for q, _ in layers]
     cfg = synth.CONFIGS[workload]
@@ -555,7 +556,7 @@ def measure_decode(workload: str, n_layers: int, K: int, W: int, args, dev):
                 "layers_cycled": n_layers, "launch": "hip-graph replay" if use_graph else "eager",
                 "timing": "median of 5 regions of `steps` steps, HIP events around the steps; 512 MiB rewritten "
                           "on the stream right before each region",
-                "qk_tiling": args.qk_tiling, "dot": args.dot,
+                "qk_tiling": args.qk_tiling, "dot": args.dot, "combine": args.combine,
                 "softmax": "fused into the two GEMV launches" if fused else "separate launch",
                 "algorithmic_bytes_per_step": alg_bytes},
         kernels_us={"qk_hybrid_kernel": round(qk_us, 3), "scale_softmax_kernel": round(sm_us, 3),
@@ -578,6 +579,8 @@ def main():
                     help="force one q.K^T tiling instead of the choice by launch size")
     ap.add_argument("--dot", default="auto", choices=["auto", "mfma", "valu"],
                     help="form of the inner products: matrix cores, vector ALU, or the library's default")
+    ap.add_argument("--combine", default="auto", choices=["auto", "fold", "separate"],
+                    help="who sums the split-K partials: the last p.V workgroup of each (b, kv head) or a launch of its own (auto: by launch size)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true",
