@@ -1525,41 +1525,55 @@ struct PvStage {
 // requests of the next block (and of the first block, at kernel start) overlap with other work.
 template <int NREP, int NG>
 struct PvPair {
-  int64_t pa, pb;
+  int64_t pa, pb;        // positions of the pair's tokens
+  int64_t ta;            // token a inside the class; token b is `second` rows on (0: there is none, a is read twice)
+  int32_t second;
   half_t va[NREP], vb[NREP];
   uint2 sa, sb, za, zb;  // 4 fp16 scales / zeros of token a and of token b (NG == 4)
   bool valid, has_b;
 };
 
-template <int NREP, int NG, bool QUANT>
-__device__ __forceinline__ void pv_fetch(const SegDev &sg, int64_t t0, int nt, int bh, half_t *const (&prow)[NREP],
-                                         PvPair<NREP, NG> &pr) {
-  static_assert(NG == 4, "a token's scale row is read as one 8-byte load");
+// The fetch has two dependent halves -- the positions, then what sits at the positions -- so that a caller with
+// something else to wait for can put it between them.
+template <int NREP, int NG>
+__device__ __forceinline__ void pv_fetch_positions(const SegDev &sg, int64_t t0, int nt, PvPair<NREP, NG> &pr) {
   const int tp = threadIdx.x;
   pr.valid = 2 * tp < nt;
   pr.has_b = 2 * tp + 1 < nt;
-  const int64_t ta = t0 + (pr.valid ? 2 * tp : 0);
-  const int64_t tb2 = pr.has_b ? ta + 1 : ta;
-  pr.pa = sg.pos_base + ta;
-  pr.pb = sg.pos_base + tb2;
+  pr.ta = t0 + (pr.valid ? 2 * tp : 0);
+  pr.second = pr.has_b ? 1 : 0;
+  pr.pa = sg.pos_base + pr.ta;
+  pr.pb = pr.pa + pr.second;
   if (sg.idx) {
-    pr.pa = sg.idx[ta];
-    pr.pb = sg.idx[tb2];
+    pr.pa = sg.idx[pr.ta];
+    pr.pb = sg.idx[pr.ta + pr.second];
   }
+}
+
+template <int NREP, int NG, bool QUANT>
+__device__ __forceinline__ void pv_fetch_values(const SegDev &sg, int bh, half_t *const (&prow)[NREP],
+                                                PvPair<NREP, NG> &pr) {
+  static_assert(NG == 4, "a token's scale row is read as one 8-byte load");
   if (QUANT) {  // a V class may hold any number of tokens: the last pair of an odd count reads row a twice
-    const uint2 *sc = reinterpret_cast<const uint2 *>(sg.scale + ((int64_t)bh * sg.slab_tokens + ta) * NG);
-    const uint2 *zr = reinterpret_cast<const uint2 *>(sg.zero + ((int64_t)bh * sg.slab_tokens + ta) * NG);
-    const int second = (int)(tb2 - ta);
+    const uint2 *sc = reinterpret_cast<const uint2 *>(sg.scale + ((int64_t)bh * sg.slab_tokens + pr.ta) * NG);
+    const uint2 *zr = reinterpret_cast<const uint2 *>(sg.zero + ((int64_t)bh * sg.slab_tokens + pr.ta) * NG);
     pr.sa = sc[0];
-    pr.sb = sc[second];
+    pr.sb = sc[pr.second];
     pr.za = zr[0];
-    pr.zb = zr[second];
+    pr.zb = zr[pr.second];
   }
 #pragma unroll
   for (int h = 0; h < NREP; ++h) {
     pr.va[h] = prow[h][pr.pa];
     pr.vb[h] = prow[h][pr.pb];
   }
+}
+
+template <int NREP, int NG, bool QUANT>
+__device__ __forceinline__ void pv_fetch(const SegDev &sg, int64_t t0, int nt, int bh, half_t *const (&prow)[NREP],
+                                         PvPair<NREP, NG> &pr) {
+  pv_fetch_positions<NREP, NG>(sg, t0, nt, pr);
+  pv_fetch_values<NREP, NG, QUANT>(sg, bh, prow, pr);
 }
 
 template <int NREP, int NG, bool QUANT, bool ZERO_FILL = false>
@@ -1620,7 +1634,8 @@ __device__ __forceinline__ void pv_commit(const PvPair<NREP, NG> &pr, half_t *co
 template <int BITS, int NREP, int D, bool NORMAL = false, bool MF = false>
 __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c1, int bh, int wave, int lane,
                                          half_t *const (&prow)[NREP], PvStage<NREP, D / 32> &st,
-                                         float (&acc)[NREP][PV_CPL], bool fused, const float *sm_ml) {
+                                         float (&acc)[NREP][PV_CPL], bool fused, const float *sm_ml,
+                                         const PvPair<NREP, D / 32> &first) {
   static_assert(D == 128, "16 lanes x 8 channels cover one token row");
   static_assert(!MF || NREP == 4, "the matrix-core form is a 4-head product");
   constexpr int NG = D / 32;
@@ -1660,11 +1675,11 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
   f4_t av[PV_CPL];  // matrix-core form: (4 heads) per channel of this lane
 #pragma unroll
   for (int i = 0; i < PV_CPL; ++i) av[i] = (f4_t){0.f, 0.f, 0.f, 0.f};
-  PvPair<NREP, NG> pr;
+  PvPair<NREP, NG> pr = first;   // the first block's positions were requested at the top of the kernel
   Words cur;
   {
     const int nt0 = (int)min((int64_t)PV_BLOCK, c1 - c0);
-    pv_fetch<NREP, NG, QUANT>(sg, c0, nt0, bh, prow, pr);
+    pv_fetch_values<NREP, NG, QUANT>(sg, bh, prow, pr);
     load_steps(c0, nt0, 0, cur);
   }
   for (int64_t t0 = c0; t0 < c1; t0 += PV_BLOCK) {
@@ -1809,15 +1824,23 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   half_t *prow[NREP];
 #pragma unroll
   for (int h = 0; h < NREP; ++h) prow[h] = p + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+  // The positions of the first block are asked for before anything else: what is read AT them (the logits) is the
+  // longest chain of dependent loads at the start of a workgroup's life, and the statistics below wait in its shadow.
+  PvPair<NREP, D / 32> first;
+  pv_fetch_positions<NREP, D / 32>(sg, c0, (int)min((int64_t)PV_BLOCK, c1 - c0), first);
   if (fused) {
-    // merge the per-tile (m, l) pairs of each head: wave w serves heads w, w+4, ...
+    // merge the per-tile (m, l) pairs of each head: wave w serves heads w, w+4, ...; up to 128 tiles are read once
+    // and kept in registers between the maximum and the sum
     for (int h = wave; h < NREP; h += PV_WAVES) {
       const float2 *sp = fz.stats + ((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat;
-      float m = -INFINITY;
-      for (int e = lane; e < fz.n_stat; e += 64) m = fmaxf(m, sp[e].x);
+      const float2 none = make_float2(-INFINITY, 0.f);
+      const float2 v0 = lane < fz.n_stat ? sp[lane] : none;
+      const float2 v1 = lane + 64 < fz.n_stat ? sp[lane + 64] : none;
+      float m = fmaxf(v0.x, v1.x);
+      for (int e = lane + 128; e < fz.n_stat; e += 64) m = fmaxf(m, sp[e].x);
       m = wave_max(m);
-      float l = 0.f;
-      for (int e = lane; e < fz.n_stat; e += 64) {
+      float l = (lane < fz.n_stat ? v0.y * __expf(v0.x - m) : 0.f) + (lane + 64 < fz.n_stat ? v1.y * __expf(v1.x - m) : 0.f);
+      for (int e = lane + 128; e < fz.n_stat; e += 64) {
         const float2 v = sp[e];
         l += v.y * __expf(v.x - m);
       }
@@ -1835,13 +1858,13 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
     for (int i = 0; i < PV_CPL; ++i) acc[h][i] = 0.f;
   switch (sg.bits) {  // (the first barrier inside pv_chunk also publishes sm_ml)
     case 1:
-      if (sg.layout == HQEKV_LAYOUT_NORMAL1) pv_chunk<1, NREP, D, true, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
-      else pv_chunk<1, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
+      if (sg.layout == HQEKV_LAYOUT_NORMAL1) pv_chunk<1, NREP, D, true, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml, first);
+      else pv_chunk<1, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml, first);
       break;
-    case 2: pv_chunk<2, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
-    case 4: pv_chunk<4, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
-    case 8: pv_chunk<8, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml); break;
-    default: pv_chunk<16, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml);
+    case 2: pv_chunk<2, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml, first); break;
+    case 4: pv_chunk<4, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml, first); break;
+    case 8: pv_chunk<8, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml, first); break;
+    default: pv_chunk<16, NREP, D, false, MF>(sg, c0, c1, bh, wave, lane, prow, st, acc, fused, sm_ml, first);
   }
   // Lanes 16, 32 and 48 apart hold the same channels of other tokens.  Their sum is needed in lanes 0-15
   // only: two lane-row swaps on the vector ALU per value (a swap exchanges rows of 16 lanes between two
