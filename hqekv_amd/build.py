@@ -16,7 +16,7 @@ PKG = Path(__file__).resolve().parent
 ROOT = PKG.parent
 CSRC = PKG / "csrc"
 LIB = PKG / "libhqekv.so"
-SOURCES = ["capi.hip", "quant_pack.hip", "attn.hip", "decode_static.hip", "migrate.hip", "planner.hip", "importance.hip"]
+SOURCES = ["capi.hip", "quant_pack.hip", "attn.hip", "decode_static.hip", "migrate.hip", "planner.hip", "importance.hip", "prompt_attn.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",

@@ -1,0 +1,341 @@
+// The prompt side of the attention layer (model/llama_hqe.py:141-188): causal attention over the whole prompt, and the
+// probabilities of its last rows, which seed the importance ring.  The reference calls flash-attention for the first
+// and a dense matmul + softmax over the last 20 query rows for the second; here both are matrix-core kernels for
+// head_dim 128 in fp16 with fp32 accumulation, reading K and V once per query head through the caches (the query
+// heads of one KV head are neighbours in the grid), without `repeat_kv` copies.
+//
+// Both kernels compute S^T = K . Q^T -- keys along M, queries along N of v_mfma_f32_32x32x16_f16 -- so that a lane
+// owns ONE query (column lane % 32): the running maximum, the sum and the rescaling of the output are per-lane
+// scalars, and the exponentials a lane holds (keys 8 g + 4 (lane / 32) + j of a 32-key tile, g = 0..3, j = 0..3) are
+// already laid out as the B operand of the second product, O^T = V^T . P^T.  That product needs, per lane, four
+// consecutive KEYS of one channel: the V tile is turned by 4 x 4 register transposes on its way into LDS
+// ([key quad][channel][4 keys]).
+#include "common.h"
+
+namespace hq {
+
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef float f16_t __attribute__((ext_vector_type(16)));
+
+constexpr int PA_D = 128;
+constexpr int PA_WAVES = 4;
+constexpr int PA_THREADS = 64 * PA_WAVES;
+constexpr int PA_BR = 32 * PA_WAVES;   // query rows per workgroup
+constexpr int PA_BC = 64;              // keys per tile
+constexpr int PA_KS = PA_D + 8;        // halfs per K row in LDS (the pad spreads the rows over the banks)
+constexpr int PA_VS = PA_D * 4 + 8;    // halfs per key quad of the turned V tile
+
+struct PromptArgs {
+  const half_t *q, *k, *v;
+  half_t *out;
+  int64_t q_b, q_h, q_t;   // strides in elements; the channel stride is 1
+  int64_t k_b, k_h, k_t;
+  int64_t v_b, v_h, v_t;
+  int64_t o_b, o_h, o_t;
+  int32_t Hq, Hkv, T;
+  float scale;
+};
+
+__device__ __forceinline__ uint32_t lo_pair(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
+__device__ __forceinline__ uint32_t hi_pair(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
+
+// one tile of keys on its way from memory to LDS: 16 bytes x 4 of K and of V per thread
+struct PaTileRegs {
+  uint4 kr[4], vr[4];
+};
+__device__ __forceinline__ void pa_tile_fetch(const half_t *kp, int64_t k_t, const half_t *vp, int64_t v_t, int k0, int T,
+                                              PaTileRegs &r) {
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = tid + PA_THREADS * i, row = idx >> 4, c = idx & 15;
+    const int key = min(k0 + row, T - 1);   // rows past the end repeat the last key; the scores mask them
+    r.kr[i] = *reinterpret_cast<const uint4 *>(kp + (int64_t)key * k_t + c * 8);
+  }
+  const int quad = tid >> 4, oct = tid & 15;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int key = min(k0 + 4 * quad + j, T - 1);
+    r.vr[j] = *reinterpret_cast<const uint4 *>(vp + (int64_t)key * v_t + oct * 8);
+  }
+}
+__device__ __forceinline__ void pa_tile_store(const PaTileRegs &r, half_t *ks, half_t *vs) {
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = tid + PA_THREADS * i, row = idx >> 4, c = idx & 15;
+    *reinterpret_cast<uint4 *>(ks + row * PA_KS + c * 8) = r.kr[i];
+  }
+  // 4 keys x 8 channels -> 8 channels x 4 keys
+  const int quad = tid >> 4, oct = tid & 15;
+  const uint32_t a[4] = {r.vr[0].x, r.vr[0].y, r.vr[0].z, r.vr[0].w}, b[4] = {r.vr[1].x, r.vr[1].y, r.vr[1].z, r.vr[1].w};
+  const uint32_t c[4] = {r.vr[2].x, r.vr[2].y, r.vr[2].z, r.vr[2].w}, e[4] = {r.vr[3].x, r.vr[3].y, r.vr[3].z, r.vr[3].w};
+  uint4 *dst = reinterpret_cast<uint4 *>(vs + quad * PA_VS + oct * 32);
+#pragma unroll
+  for (int p = 0; p < 4; ++p)   // channels 2p and 2p + 1 of this thread's eight
+    dst[p] = make_uint4(lo_pair(a[p], b[p]), lo_pair(c[p], e[p]), hi_pair(a[p], b[p]), hi_pair(c[p], e[p]));
+}
+
+// S^T of one 64-key tile for the wave's 32 queries: two 32-key tiles, 16 fp32 values per lane each
+__device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8], int n, int h, f16_t &s0, f16_t &s1) {
+  s0 = s1 = (f16_t)(0.f);
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const h8_t ka = *reinterpret_cast<const h8_t *>(ks + n * PA_KS + 16 * s + 8 * h);
+    const h8_t kb = *reinterpret_cast<const h8_t *>(ks + (32 + n) * PA_KS + 16 * s + 8 * h);
+    s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[s], s0, 0, 0, 0);
+    s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb, qreg[s], s1, 0, 0, 0);
+  }
+}
+// key (inside a 64-key tile) of element r of 32-key tile mt in this lane
+__device__ __forceinline__ int pa_key_of(int mt, int r, int h) { return 32 * mt + 8 * (r >> 2) + 4 * h + (r & 3); }
+
+template <bool CAUSAL>
+__global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a) {
+  __shared__ __align__(16) half_t ks[PA_BC * PA_KS];
+  __shared__ __align__(16) half_t vs[(PA_BC / 4) * PA_VS];
+  const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;   // the longest rows first
+  const int q0 = qb * PA_BR;
+  const int b = (int)blockIdx.y / a.Hq, hq = (int)blockIdx.y % a.Hq, hkv = hq / (a.Hq / a.Hkv);
+  const int T = a.T;
+  const half_t *qp = a.q + b * a.q_b + hq * a.q_h;
+  const half_t *kp = a.k + b * a.k_b + hkv * a.k_h;
+  const half_t *vp = a.v + b * a.v_b + hkv * a.v_h;
+  const int my_q = q0 + 32 * w + n;
+  h8_t qreg[8];
+  {
+    const half_t *qr = qp + (int64_t)min(my_q, T - 1) * a.q_t + 8 * h;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const h8_t *>(qr + 16 * s);
+  }
+  f16_t o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) o[dt] = (f16_t)(0.f);
+  float m = -INFINITY, lsum = 0.f;
+  const float sl2 = a.scale * 1.4426950408889634f;
+  const int kend = CAUSAL ? min(T, q0 + PA_BR) : T;
+  const int n_tiles = (kend + PA_BC - 1) / PA_BC;
+  const int wave_last_q = q0 + 32 * w + 31;
+  PaTileRegs tr;
+  pa_tile_fetch(kp, a.k_t, vp, a.v_t, 0, T, tr);
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    const int k0 = tile * PA_BC;
+    __syncthreads();   // the previous tile has been read by every wave
+    pa_tile_store(tr, ks, vs);
+    __syncthreads();
+    if (tile + 1 < n_tiles) pa_tile_fetch(kp, a.k_t, vp, a.v_t, k0 + PA_BC, T, tr);   // in flight across the products
+    if (CAUSAL && k0 > wave_last_q) continue;   // (uniform per wave) every key of the tile lies after every query of the wave
+    f16_t s[2];
+    pa_scores(ks, qreg, n, h, s[0], s[1]);
+    const bool edge = (k0 + PA_BC > T) || (CAUSAL && k0 + PA_BC - 1 > q0 + 32 * w);   // some element of the tile is masked
+    float mx = m;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float v = s[mt][r] * sl2;
+        if (edge) {
+          const int key = k0 + pa_key_of(mt, r, h);
+          if (key >= T || (CAUSAL && key > my_q)) v = -INFINITY;
+        }
+        s[mt][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float alpha = exp2f(m - mx);   // (the first tile always holds key 0, which no query masks: mx is finite)
+    m = mx;
+    float part = 0.f;
+    h8_t p[4];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = exp2f(s[mt][r] - mx);
+        part += e;
+        p[2 * mt + (r >> 3)][r & 7] = (half_t)e;
+      }
+    lsum = lsum * alpha + part;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) o[dt] *= alpha;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        const half_t *va = vs + (4 * t + h) * PA_VS + (32 * dt + n) * 4;
+        const h4_t lo = *reinterpret_cast<const h4_t *>(va), hi = *reinterpret_cast<const h4_t *>(va + 2 * PA_VS);
+        const h8_t av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, p[t], o[dt], 0, 0, 0);
+      }
+  }
+  lsum += __shfl_xor(lsum, 32, 64);
+  if (my_q < T) {
+    const float inv = 1.0f / lsum;
+    half_t *orow = a.out + b * a.o_b + hq * a.o_h + (int64_t)my_q * a.o_t;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        h4_t y;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) y[j] = (half_t)(o[dt][4 * g + j] * inv);
+        *reinterpret_cast<h4_t *>(orow + 32 * dt + 8 * g + 4 * h) = y;
+      }
+  }
+}
+
+// ---- probabilities of the last R <= 32 query rows, with the reference's roundings (model/llama_hqe.py:156-168):
+// the product rounded to fp16, times the scale rounded to fp16, plus the mask rounded to fp16, floored at the most
+// negative fp16, softmax in fp32, rounded to fp16.  One workgroup per (b, query head); its four waves deal the
+// 32-key tiles round-robin and walk them twice: maximum and sum, then the probabilities.
+struct LastRowsArgs {
+  const half_t *q, *k;
+  const half_t *mask;   // additive, (B, 1, R, T) with strides, or nullptr: causal
+  half_t *probs;        // (B, Hq, R, T) contiguous
+  int64_t q_b, q_h, q_t;
+  int64_t k_b, k_h, k_t;
+  int64_t m_b, m_r;
+  int32_t Hq, Hkv, T, R;
+  float scale;
+};
+
+__global__ __launch_bounds__(PA_THREADS, 2) void prompt_last_rows_kernel(LastRowsArgs a) {
+  __shared__ float sh_m[PA_WAVES][32], sh_l[PA_WAVES][32];
+  const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int b = (int)blockIdx.x / a.Hq, hq = (int)blockIdx.x % a.Hq, hkv = hq / (a.Hq / a.Hkv);
+  const int T = a.T, R = a.R;
+  const half_t *kp = a.k + b * a.k_b + hkv * a.k_h;
+  const int row = min(n, R - 1);         // lanes past the last row repeat it and store nothing
+  const int my_q = T - R + row;
+  h8_t qreg[8];
+  {
+    const half_t *qr = a.q + b * a.q_b + hq * a.q_h + (int64_t)my_q * a.q_t + 8 * h;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const h8_t *>(qr + 16 * s);
+  }
+  const half_t *mrow = a.mask ? a.mask + b * a.m_b + (int64_t)row * a.m_r : nullptr;
+  const int n_tiles = (T + 31) / 32;
+  // the 16 scores of this lane for 32-key tile `tile`, as the reference's fp16 chain leaves them (in fp32)
+  auto tile_scores = [&](int tile, float (&x)[16]) {
+    const int key_row = min(32 * tile + n, T - 1);
+    const half_t *kr = kp + (int64_t)key_row * a.k_t + 8 * h;
+    f16_t s = (f16_t)(0.f);
+#pragma unroll
+    for (int st = 0; st < 8; ++st)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const h8_t *>(kr + 16 * st), qreg[st], s, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = 32 * tile + 8 * (r >> 2) + 4 * h + (r & 3);
+      half_t v = (half_t)((float)(half_t)s[r] * a.scale);
+      if (mrow) {
+        v = (half_t)((float)v + (float)mrow[min(key, T - 1)]);
+        v = (half_t)fmaxf((float)v, -65504.f);
+        x[r] = key < T ? (float)v : -INFINITY;
+      } else {
+        x[r] = (key < T && key <= my_q) ? (float)v : -INFINITY;
+      }
+    }
+  };
+  float m = -INFINITY, l = 0.f;
+  for (int tile = w; tile < n_tiles; tile += PA_WAVES) {
+    float x[16];
+    tile_scores(tile, x);
+    float mx = m;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, x[r]);
+    if (mx == -INFINITY) continue;   // nothing but masked keys so far
+    float part = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part += __expf(x[r] - mx);
+    l = l * __expf(m - mx) + part;
+    m = mx;
+  }
+  {  // the two halves of the wave, then the four waves
+    const float mo = __shfl_xor(m, 32, 64), lo = __shfl_xor(l, 32, 64);
+    const float mx = fmaxf(m, mo);
+    l = (m == -INFINITY ? 0.f : l * __expf(m - mx)) + (mo == -INFINITY ? 0.f : lo * __expf(mo - mx));
+    m = mx;
+    if (h == 0) {
+      sh_m[w][n] = m;
+      sh_l[w][n] = l;
+    }
+    __syncthreads();
+    float mx2 = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < PA_WAVES; ++k) mx2 = fmaxf(mx2, sh_m[k][n]);
+    float tot = 0.f;
+#pragma unroll
+    for (int k = 0; k < PA_WAVES; ++k) tot += sh_m[k][n] == -INFINITY ? 0.f : sh_l[k][n] * __expf(sh_m[k][n] - mx2);
+    m = mx2;
+    l = tot;
+  }
+  const float inv = 1.0f / l;
+  half_t *prow = a.probs + (((int64_t)b * a.Hq + hq) * R + row) * (int64_t)T;
+  for (int tile = w; tile < n_tiles; tile += PA_WAVES) {
+    float x[16];
+    tile_scores(tile, x);
+    if (n >= R) continue;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int key = 32 * tile + 8 * g + 4 * h;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (key + j < T) prow[key + j] = (half_t)(__expf(x[4 * g + j] - m) * inv);
+    }
+  }
+}
+
+}  // namespace hq
+
+using namespace hq;
+
+static bool rows_16_byte_aligned(const void *p, int64_t s0, int64_t s1, int64_t s2) {
+  return ((uintptr_t)p & 15) == 0 && s0 % 8 == 0 && s1 % 8 == 0 && s2 % 8 == 0;
+}
+
+extern "C" int hqekv_prompt_attn(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides,
+                                 const void *v, const int64_t *v_strides, void *out, const int64_t *out_strides, int64_t B,
+                                 int64_t Hq, int64_t Hkv, int64_t T, int64_t D, float scale, int causal, void *stream) {
+  if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !out_strides)
+    return fail(HQEKV_E_ARG, "prompt_attn: null pointer");
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv) return fail(HQEKV_E_ARG, "prompt_attn: need B, T > 0 and Hq %% Hkv == 0");
+  if (D != PA_D) return fail(HQEKV_E_UNSUPPORTED, "prompt_attn: head_dim %lld (supported: 128)", (long long)D);
+  if (T > 0x7fffff00LL || B * Hq > 65535) return fail(HQEKV_E_UNSUPPORTED, "prompt_attn: T or B * Hq too large");
+  if (!rows_16_byte_aligned(q, q_strides[0], q_strides[1], q_strides[2]) || !rows_16_byte_aligned(k, k_strides[0], k_strides[1], k_strides[2]) ||
+      !rows_16_byte_aligned(v, v_strides[0], v_strides[1], v_strides[2]) || ((uintptr_t)out & 7) || out_strides[0] % 4 || out_strides[1] % 4 || out_strides[2] % 4)
+    return fail(HQEKV_E_ALIGN, "prompt_attn: rows of q, k, v must be 16-byte aligned (of out: 8-byte)");
+  PromptArgs a;
+  a.q = (const half_t *)q; a.k = (const half_t *)k; a.v = (const half_t *)v; a.out = (half_t *)out;
+  a.q_b = q_strides[0]; a.q_h = q_strides[1]; a.q_t = q_strides[2];
+  a.k_b = k_strides[0]; a.k_h = k_strides[1]; a.k_t = k_strides[2];
+  a.v_b = v_strides[0]; a.v_h = v_strides[1]; a.v_t = v_strides[2];
+  a.o_b = out_strides[0]; a.o_h = out_strides[1]; a.o_t = out_strides[2];
+  a.Hq = (int32_t)Hq; a.Hkv = (int32_t)Hkv; a.T = (int32_t)T; a.scale = scale;
+  const dim3 grid((unsigned)((T + PA_BR - 1) / PA_BR), (unsigned)(B * Hq));
+  if (causal) hipLaunchKernelGGL(prompt_attn_kernel<true>, grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(prompt_attn_kernel<false>, grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+  return check_launch("prompt_attn");
+}
+
+extern "C" int hqekv_prompt_last_rows(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides,
+                                      const void *mask, const int64_t *mask_strides, void *probs, int64_t B, int64_t Hq,
+                                      int64_t Hkv, int64_t T, int64_t D, int64_t R, float scale, void *stream) {
+  if (!q || !k || !probs || !q_strides || !k_strides || (mask && !mask_strides)) return fail(HQEKV_E_ARG, "prompt_last_rows: null pointer");
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv || R <= 0 || R > 32 || R > T)
+    return fail(HQEKV_E_ARG, "prompt_last_rows: need B > 0, Hq %% Hkv == 0 and 0 < R <= min(32, T)");
+  if (D != PA_D) return fail(HQEKV_E_UNSUPPORTED, "prompt_last_rows: head_dim %lld (supported: 128)", (long long)D);
+  if (T > 0x7fffff00LL || B * Hq > 0x7fffffffLL) return fail(HQEKV_E_UNSUPPORTED, "prompt_last_rows: T or B * Hq too large");
+  if (!rows_16_byte_aligned(q, q_strides[0], q_strides[1], q_strides[2]) || !rows_16_byte_aligned(k, k_strides[0], k_strides[1], k_strides[2]))
+    return fail(HQEKV_E_ALIGN, "prompt_last_rows: rows of q and k must be 16-byte aligned");
+  LastRowsArgs a;
+  a.q = (const half_t *)q; a.k = (const half_t *)k; a.mask = (const half_t *)mask; a.probs = (half_t *)probs;
+  a.q_b = q_strides[0]; a.q_h = q_strides[1]; a.q_t = q_strides[2];
+  a.k_b = k_strides[0]; a.k_h = k_strides[1]; a.k_t = k_strides[2];
+  a.m_b = mask ? mask_strides[0] : 0; a.m_r = mask ? mask_strides[1] : 0;
+  a.Hq = (int32_t)Hq; a.Hkv = (int32_t)Hkv; a.T = (int32_t)T; a.R = (int32_t)R; a.scale = scale;
+  hipLaunchKernelGGL(prompt_last_rows_kernel, dim3((unsigned)(B * Hq)), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+  return check_launch("prompt_last_rows");
+}

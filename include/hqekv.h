@@ -331,6 +331,26 @@ int hqekv_weighted_block_scores(const void *x, const void *weights, int64_t tota
 int hqekv_token_range(const void *v, int64_t B, int64_t H, int64_t T, int64_t D, int64_t slab_tokens, void *out,
                       void *stream);
 
+/* ------------------------------------------------------------------ the prompt side of the attention layer
+ * Replaces, for head_dim 128 in fp16, what model/llama_hqe.py:141-188 does over a prompt: flash_attention_forward
+ * (:147-155) and, for the importance ring, the dense matmul + mask + softmax over the last 20 query rows with
+ * repeat_kv copies of K (:157-168).  Tensors are (B, H, T, 128) fp16 given by their strides in ELEMENTS for the
+ * batch, head and token axes (channel stride 1, rows 16-byte aligned), so slices of a fused QKV projection are read
+ * where they lie; K and V have Hkv heads, query head h reads KV head h / (Hq / Hkv).
+ *   hqekv_prompt_attn       out (B, Hq, T, 128, strides as given) = softmax(q k^T * scale [causal]) v, fp32
+ *                           accumulation and running softmax, probabilities rounded to fp16 before the second product
+ *   hqekv_prompt_last_rows  probs (B, Hq, R, T) contiguous: the probabilities of the last R <= 32 query rows with the
+ *                           reference's roundings -- product to fp16, times scale to fp16, plus mask to fp16, floored
+ *                           at -65504, softmax in fp32, to fp16.  mask: additive fp16 (B, 1, R, T) given by its batch
+ *                           and row strides (key stride 1), or NULL for the causal rule (row r sees keys <= T - R + r).
+ */
+int hqekv_prompt_attn(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides, const void *v,
+                      const int64_t *v_strides, void *out, const int64_t *out_strides, int64_t B, int64_t Hq, int64_t Hkv,
+                      int64_t T, int64_t D, float scale, int causal, void *stream);
+int hqekv_prompt_last_rows(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides,
+                           const void *mask, const int64_t *mask_strides, void *probs, int64_t B, int64_t Hq, int64_t Hkv,
+                           int64_t T, int64_t D, int64_t R, float scale, void *stream);
+
 /* ------------------------------------------------------------------ cache maintenance (one launch per side)
  * Replaces the per-(source, target) gathers, dequantise / re-quantise calls and torch.cat re-copies of one
  * compression -- V_high_2_eviction / K_high_2_eviction (quant/hqe_2.py:44-86), quant_new_K (:16-42), K_high_2_low
