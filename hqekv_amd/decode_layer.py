@@ -10,10 +10,11 @@ Per call (model/llama_hqe.py, line numbers in brackets):
             [211-214]), block ranking [228], ``KV_cache_hqe_2`` [230-231], bookkeeping and the ratio
             update for the next 32-token increment [233-239].
 
-Decode attention, quantisation, demotion and eviction run on the HIP kernels of this package.  The prompt
-attention (outside the quantised path) uses torch: ``scaled_dot_product_attention`` with grouped query heads for
-the output and one batched matmul for the last 20 rows of probabilities, the only rows the ring keeps [146-170];
-neither materialises ``repeat_kv`` copies of K or V.
+Decode attention, quantisation, demotion and eviction run on the HIP kernels of this package, and so does the
+prompt for fp16 tensors of head_dim 128: one matrix-core kernel for the causal attention over the whole prompt
+(flash-attention in the reference [146-154]) and one for the probabilities of the last 20 rows, the only rows the
+ring keeps [156-170].  A prompt with an explicit additive mask, another head size or element type goes through
+torch's fused attention for the output.  Neither path materialises ``repeat_kv`` copies of K or V.
 """
 from __future__ import annotations
 
@@ -22,6 +23,7 @@ from typing import Optional, Tuple
 import numpy as np
 import torch
 
+from . import prompt_attention
 from .attention import SegmentMemo, value_length
 from .hqe_2 import KV_cache_hqe_2
 from .hqe_matmul import qkv_matmul_hqe_2
@@ -42,10 +44,13 @@ _GQA_SDPA = [True]   # torch's fused attention takes grouped query heads directl
 
 
 def gqa_prompt_attention(q, k, v, attention_mask, scaling):
-    """softmax(q k^T * scaling + mask) v over a whole prompt with grouped query heads, through torch's fused attention
-    (the prompt is outside the quantised path; the reference calls flash-attention here, model/llama_hqe.py:146-154).
-    K and V are handed over as they are, (B,Hkv,T,D); only when the fused kernel refuses grouped heads are they
-    expanded."""
+    """softmax(q k^T * scaling + mask) v over a whole prompt with grouped query heads (the reference calls
+    flash-attention here, model/llama_hqe.py:146-154).  Without a mask -- the causal rule -- fp16 tensors of head_dim
+    128 go to the library's matrix-core kernel (``prompt_attention``); a prompt with an explicit additive mask, another
+    head size or element type goes through torch's fused attention.  K and V are handed over as they are, (B,Hkv,T,D);
+    only when torch's kernel refuses grouped heads are they expanded."""
+    if attention_mask is None and prompt_attention.supported(q, k, v):
+        return prompt_attention.prompt_attention(q, k, v, scaling, causal=True)
     n_rep = q.shape[1] // k.shape[1]
     causal = attention_mask is None and k.shape[-2] > 1
     if n_rep > 1 and _GQA_SDPA[0]:
@@ -56,6 +61,26 @@ def gqa_prompt_attention(q, k, v, attention_mask, scaling):
             _GQA_SDPA[0] = False
     return torch.nn.functional.scaled_dot_product_attention(q, _repeat_kv(k, n_rep), _repeat_kv(v, n_rep),
                                                             attn_mask=attention_mask, is_causal=causal, scale=scaling)
+
+
+def last_rows_probabilities(q, k, attention_mask, scaling, rows):
+    """Probabilities of the last ``rows`` query rows of a prompt over all keys, (B,Hq,rows,T), as the reference
+    computes them for the importance ring (model/llama_hqe.py:156-168): the library's kernel for fp16 tensors of
+    head_dim 128 (same roundings; without a mask the causal rule), torch otherwise.  The query heads that share a KV
+    head are folded into the row dimension of one batched product instead of materialising ``repeat_kv`` copies."""
+    if rows <= prompt_attention.MAX_LAST_ROWS and prompt_attention.supported(q, k):
+        return prompt_attention.prompt_last_rows(q, k, scaling, rows, attention_mask)
+    B, Hq, T, D = q.shape
+    Hkv = k.shape[1]
+    q_last = q[:, :, T - rows:, :].reshape(B, Hkv, (Hq // Hkv) * rows, D)          # (b, kv head, [rep, row], d)
+    w = (torch.matmul(q_last, k.transpose(2, 3)) * scaling).view(B, Hq, rows, T)
+    if attention_mask is not None:
+        w = w + attention_mask[:, :, -rows:, :]
+        w = torch.max(w, torch.tensor(torch.finfo(w.dtype).min, dtype=w.dtype, device=w.device))
+    elif rows > 1 or T > 1:
+        keep = torch.arange(T, device=q.device)[None, :] <= (T - rows + torch.arange(rows, device=q.device))[:, None]
+        w = w.masked_fill(~keep, torch.finfo(w.dtype).min)
+    return torch.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
 
 
 _F32 = np.float32
@@ -145,18 +170,9 @@ class HqeAttentionLayer:
     # ------------------------------------------------------------------ prompt
     def _prefill(self, q, k, v, attention_mask):
         """Prompt attention [141-188]: the output over all rows, and the probabilities of the last 20 rows only (what
-        the ring keeps).  K and V are read once per KV head: the query heads that share a KV head are folded into the
-        row dimension of one batched product instead of materialising ``repeat_kv`` copies of K and V."""
-        B, Hq, T, D = q.shape
-        Hkv = k.shape[1]
-        n_rep = Hq // Hkv
-        rows = min(T, LAST_TOKEN_NUM)
-        q_last = q[:, :, T - rows:, :].reshape(B, Hkv, n_rep * rows, D)          # (b, kv head, [rep, row], d)
-        w = (torch.matmul(q_last, k.transpose(2, 3)) * self.scaling).view(B, Hq, rows, T)
-        if attention_mask is not None:
-            w = w + attention_mask[:, :, -rows:, :]
-            w = torch.max(w, torch.tensor(torch.finfo(w.dtype).min, dtype=w.dtype, device=w.device))
-        attn_weights = torch.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
+        the ring keeps).  K and V are read once per KV head, without ``repeat_kv`` copies."""
+        rows = min(q.shape[2], LAST_TOKEN_NUM)
+        attn_weights = last_rows_probabilities(q, k, attention_mask, self.scaling, rows)
         attn_output = gqa_prompt_attention(q, k, v, attention_mask, self.scaling)
         return attn_weights, attn_output
 

@@ -122,3 +122,23 @@ def test_prompt_entries_refuse_bad_arguments():
         prompt_last_rows(q, k, 0.1, 0)
     with pytest.raises(Exception):
         prompt_attention(q, k[:, :1].expand(1, 3, 40, 128), v, 0.1)   # 4 query heads over 3 KV heads
+
+
+def test_layer_prompt_without_a_mask_equals_the_causal_mask():
+    """The attention layer's prompt call: no mask (the library's kernels, causal rule) against an explicit causal mask
+    (torch's fused attention for the output), same probabilities for the ring and the same cache tuple."""
+    from hqekv_amd.decode_layer import HqeAttentionLayer
+    B, Hq, Hkv, T = 2, 8, 2, 157
+    q, k, v = _qkv(B, Hq, Hkv, T, 404)
+    outs = []
+    for mask in (None, _causal_mask(T, q.device)):
+        layer = HqeAttentionLayer(128, bit_0=0.2, bit_4=0.4, bit_2=0.4, bit_1=0.0)
+        layer.set_max_length(T + 8)
+        outs.append(layer(q, k, v, mask, None, None))
+    (o_a, w_a, pkv_a, _), (o_b, w_b, pkv_b, _) = outs
+    torch.testing.assert_close(o_a.float(), o_b.float(), rtol=2e-3, atol=2e-3)
+    assert w_a.shape == w_b.shape == (B, Hq, 20, T)
+    torch.testing.assert_close(w_a.float(), w_b.float(), rtol=2e-3, atol=2e-6)
+    assert len(pkv_a) == len(pkv_b) == 42
+    for fa, fb in zip(pkv_a, pkv_b):
+        assert (fa is None) == (fb is None)
