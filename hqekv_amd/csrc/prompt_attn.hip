@@ -131,35 +131,39 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     f16_t s[2];
     pa_scores(ks, qreg, n, h, s[0], s[1]);
     const bool edge = (k0 + PA_BC > T) || (CAUSAL && k0 + PA_BC - 1 > q0 + 32 * w);   // some element of the tile is masked
-    float mx = m;
+    // the running maximum is kept in units of the scaled logit (base-2 exponent); a raw score enters as s * sl2
+    float raw = -INFINITY;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        float v = s[mt][r] * sl2;
         if (edge) {
           const int key = k0 + pa_key_of(mt, r, h);
-          if (key >= T || (CAUSAL && key > my_q)) v = -INFINITY;
+          if (key >= T || (CAUSAL && key > my_q)) s[mt][r] = -INFINITY;
         }
-        s[mt][r] = v;
-        mx = fmaxf(mx, v);
+        raw = fmaxf(raw, s[mt][r]);
       }
+    float mx = fmaxf(m, raw * sl2);   // (sl2 > 0)
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float alpha = exp2f(m - mx);   // (the first tile always holds key 0, which no query masks: mx is finite)
-    m = mx;
+    // (the first tile always holds key 0, which no query masks: mx is finite from then on)
+    if (__builtin_amdgcn_ballot_w64(mx != m) != 0) {   // somebody's maximum moved: rescale what has been added up so far
+      const float alpha = __builtin_amdgcn_exp2f(m - mx);   // (the bare instruction: results below 2^-126 may flush to zero)
+      lsum *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) o[dt] *= alpha;
+      m = mx;
+    }
     float part = 0.f;
     h8_t p[4];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float e = exp2f(s[mt][r] - mx);
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r], sl2, -mx));
         part += e;
         p[2 * mt + (r >> 3)][r & 7] = (half_t)e;
       }
-    lsum = lsum * alpha + part;
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt) o[dt] *= alpha;
+    lsum += part;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -302,6 +306,7 @@ extern "C" int hqekv_prompt_attn(const void *q, const int64_t *q_strides, const 
   if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !out_strides)
     return fail(HQEKV_E_ARG, "prompt_attn: null pointer");
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv) return fail(HQEKV_E_ARG, "prompt_attn: need B, T > 0 and Hq %% Hkv == 0");
+  if (!(scale > 0.f)) return fail(HQEKV_E_ARG, "prompt_attn: the scale must be positive");
   if (D != PA_D) return fail(HQEKV_E_UNSUPPORTED, "prompt_attn: head_dim %lld (supported: 128)", (long long)D);
   if (T > 0x7fffff00LL || B * Hq > 65535) return fail(HQEKV_E_UNSUPPORTED, "prompt_attn: T or B * Hq too large");
   if (!rows_16_byte_aligned(q, q_strides[0], q_strides[1], q_strides[2]) || !rows_16_byte_aligned(k, k_strides[0], k_strides[1], k_strides[2]) ||
