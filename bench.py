@@ -34,6 +34,7 @@ WORKLOADS = {
     "c4": "Qwen3-8B shape, B=8, ctx 65536 hybrid: fp16 10% / 4-bit 20% / 2-bit 50% / evicted 20%",
     "c5": "decode-attention share of config 5: Llama-3.1-8B shape, B=4, ctx 131072 hybrid: fp16 2% / 8-bit 3% / 4-bit 25% / 2-bit 50% / evicted 20% (2.56 bit average), 32 layers resident",
     "c3": "quantize-and-pack: 8 KV heads x 128 x 8192 new fp16 tokens appended at token 24576 of a 32768-token cache",
+    "prompt": "prompt side: causal attention over a 32768-token prompt (B=1, Hq=32, Hkv=8, D=128, fp16) + the last 20 rows' probabilities",
 }
 
 
@@ -279,6 +280,54 @@ def bench_quantize(args):
         out["cpu_baseline"] = cpu
     print(json.dumps(out))
 
+
+
+# ------------------------------------------------------------------------------------------------ prompt side
+def bench_prompt(args):
+    """The prompt's attention (what the reference takes from flash-attention) and the probabilities of its last 20
+    rows, on the library's matrix-core kernels; torch's fused attention on the same tensors beside it."""
+    import math
+    from hqekv_amd.prompt_attention import prompt_attention, prompt_last_rows
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, T, D, R = 1, 32, 8, args.prompt_len if args.prompt_len != 131072 else 32768, 128, 20
+    g = torch.Generator(device=dev).manual_seed(1241)
+    q = torch.randn(B, Hq, T, D, generator=g, device=dev, dtype=torch.float16)
+    k = torch.randn(B, Hkv, T, D, generator=g, device=dev, dtype=torch.float16)
+    v = torch.randn(B, Hkv, T, D, generator=g, device=dev, dtype=torch.float16)
+    scale = 1.0 / math.sqrt(D)
+    steps, warm = max(1, min(args.steps, 20)), max(1, min(args.warmup, 3))
+
+    def timed(fn):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / steps
+    ms = timed(lambda: prompt_attention(q, k, v, scale))
+    ms_rows = timed(lambda: prompt_last_rows(q, k, scale, R))
+    ms_torch = timed(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale, enable_gqa=True))
+    flop = 4.0 * B * Hq * (T * (T + 1) / 2) * D   # two products, causal: T (T + 1) / 2 (query, key) pairs
+    out = prompt_attention(q, k, v, scale)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale, enable_gqa=True)
+    torch.cuda.synchronize()
+    tf = flop / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "TFLOP/s of the causal prompt attention (fp16, fp32 accumulation)", "value": round(tf, 1), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"prompt: {WORKLOADS['prompt']}", "T": T},
+        "last_rows_ms": round(ms_rows, 4),
+        "torch_fused_attention": {"ms": round(ms_torch, 4), "TFLOP/s": round(flop / (ms_torch * 1e-3) / 1e12, 1),
+                                  "note": "torch.nn.functional.scaled_dot_product_attention(is_causal, enable_gqa) on the same tensors, same process"},
+        "max_abs_difference_from_torch": float((out.float() - ref.float()).abs().max()),
+        "roofline": {"bound": "mfma", "kernel": "prompt_attn_kernel<true>", "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": round(tf / 2500.0, 4), "traffic": None},
+    }))
 
 
 # ------------------------------------------------------------------------------------------------ config 5
@@ -603,6 +652,9 @@ def main():
 
     if args.workload == "c3":
         bench_quantize(args)
+        return
+    if args.workload == "prompt":
+        bench_prompt(args)
         return
     if args.end_to_end:
         if args.workload != "c5":
