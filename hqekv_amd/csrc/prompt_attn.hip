@@ -8,10 +8,13 @@
 // owns ONE query (column lane % 32): the running maximum, the sum and the rescaling of the output are per-lane
 // scalars, and the exponentials a lane holds (keys 8 g + 4 (lane / 32) + j of a 32-key tile, g = 0..3, j = 0..3) are
 // already laid out as the B operand of the second product, O^T = V^T . P^T.  That product needs, per lane, four
-// consecutive KEYS of one channel: the V tile is turned by 4 x 4 register transposes on its way into LDS, and laid out
-// [16-key step][lane half][channel][8 keys] so that the eight keys a lane feeds to one product -- 4 h + j and
-// 8 + 4 h + j of the step, for lane half h -- are one 16-byte read.
+// consecutive KEYS of one channel: the V tile is turned by 4 x 4 register transposes on its way into LDS
+// ([key quad][channel][4 keys]).
 #include "common.h"
+
+#ifndef HQ_PA_QLDS
+#define HQ_PA_QLDS 2
+#endif
 
 namespace hq {
 
@@ -24,8 +27,9 @@ constexpr int PA_WAVES = 4;
 constexpr int PA_THREADS = 64 * PA_WAVES;
 constexpr int PA_BR = 32 * PA_WAVES;   // query rows per workgroup
 constexpr int PA_BC = 64;              // keys per tile
+constexpr int PA_QLDS = HQ_PA_QLDS;     // of the eight 16-channel steps of a lane's query row, how many wait in LDS instead of registers
 constexpr int PA_KS = PA_D + 8;        // halfs per K row in LDS (the pad spreads the rows over the banks)
-constexpr int PA_VG = PA_D * 8;        // halfs per (16-key step, lane half) group of the turned V tile: 128 channels x 8 keys
+constexpr int PA_VS = PA_D * 4 + 8;    // halfs per key quad of the turned V tile
 
 struct PromptArgs {
   const half_t *q, *k, *v;
@@ -45,21 +49,23 @@ __device__ __forceinline__ uint32_t hi_pair(uint32_t a, uint32_t b) { return __b
 struct PaTileRegs {
   uint4 kr[4], vr[4];
 };
-__device__ __forceinline__ void pa_tile_fetch(const half_t *kp, int64_t k_t, const half_t *vp, int64_t v_t, int k0, int T,
-                                              PaTileRegs &r) {
-  const int tid = threadIdx.x;
+// (buffer loads: one per-thread offset for each of K and V, the tile's rows through the scalar offset; rows past the
+// end of the prompt read as zeros, and the scores mask them)
+struct PaSource {
+  rsrc_t k, v;
+  uint32_t k_lane, v_lane;   // this thread's byte offsets inside a tile
+  uint32_t k_row, v_row;     // bytes between two keys
+};
+__device__ __forceinline__ uint4 buf_load16(rsrc_t r, uint32_t voff, uint32_t soff) {
+  typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+  const v4u x = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+  return make_uint4(x.x, x.y, x.z, x.w);
+}
+__device__ __forceinline__ void pa_tile_fetch(const PaSource &src, int k0, PaTileRegs &r) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int idx = tid + PA_THREADS * i, row = idx >> 4, c = idx & 15;
-    const int key = min(k0 + row, T - 1);   // rows past the end repeat the last key; the scores mask them
-    r.kr[i] = *reinterpret_cast<const uint4 *>(kp + (int64_t)key * k_t + c * 8);
-  }
-  const int quad = tid >> 4, oct = tid & 15;
+  for (int i = 0; i < 4; ++i) r.kr[i] = buf_load16(src.k, src.k_lane, (uint32_t)(k0 + 16 * i) * src.k_row);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int key = min(k0 + 4 * quad + j, T - 1);
-    r.vr[j] = *reinterpret_cast<const uint4 *>(vp + (int64_t)key * v_t + oct * 8);
-  }
+  for (int j = 0; j < 4; ++j) r.vr[j] = buf_load16(src.v, src.v_lane, (uint32_t)(k0 + j) * src.v_row);
 }
 __device__ __forceinline__ void pa_tile_store(const PaTileRegs &r, half_t *ks, half_t *vs) {
   const int tid = threadIdx.x;
@@ -68,27 +74,27 @@ __device__ __forceinline__ void pa_tile_store(const PaTileRegs &r, half_t *ks, h
     const int idx = tid + PA_THREADS * i, row = idx >> 4, c = idx & 15;
     *reinterpret_cast<uint4 *>(ks + row * PA_KS + c * 8) = r.kr[i];
   }
-  // 4 keys x 8 channels -> 8 channels x 4 keys; key quad = 4 t + 2 e + h: step t, first or second four of a lane's eight, lane half h
+  // 4 keys x 8 channels -> 8 channels x 4 keys
   const int quad = tid >> 4, oct = tid & 15;
   const uint32_t a[4] = {r.vr[0].x, r.vr[0].y, r.vr[0].z, r.vr[0].w}, b[4] = {r.vr[1].x, r.vr[1].y, r.vr[1].z, r.vr[1].w};
   const uint32_t c[4] = {r.vr[2].x, r.vr[2].y, r.vr[2].z, r.vr[2].w}, e[4] = {r.vr[3].x, r.vr[3].y, r.vr[3].z, r.vr[3].w};
-  uint2 *dst = reinterpret_cast<uint2 *>(vs + (2 * (quad >> 2) + (quad & 1)) * PA_VG + oct * 64 + ((quad >> 1) & 1) * 4);
+  uint4 *dst = reinterpret_cast<uint4 *>(vs + quad * PA_VS + oct * 32);
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {   // channels 2p and 2p + 1 of this thread's eight, 16 bytes apart
-    dst[4 * p] = make_uint2(lo_pair(a[p], b[p]), lo_pair(c[p], e[p]));
-    dst[4 * p + 2] = make_uint2(hi_pair(a[p], b[p]), hi_pair(c[p], e[p]));
-  }
+  for (int p = 0; p < 4; ++p)   // channels 2p and 2p + 1 of this thread's eight
+    dst[p] = make_uint4(lo_pair(a[p], b[p]), lo_pair(c[p], e[p]), hi_pair(a[p], b[p]), hi_pair(c[p], e[p]));
 }
 
 // S^T of one 64-key tile for the wave's 32 queries: two 32-key tiles, 16 fp32 values per lane each
-__device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8], int n, int h, f16_t &s0, f16_t &s1) {
+__device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8 - PA_QLDS], const h8_t *q_lds, int n, int h, f16_t &s0,
+                                          f16_t &s1) {
   s0 = s1 = (f16_t)(0.f);
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
     const h8_t ka = *reinterpret_cast<const h8_t *>(ks + n * PA_KS + 16 * s + 8 * h);
     const h8_t kb = *reinterpret_cast<const h8_t *>(ks + (32 + n) * PA_KS + 16 * s + 8 * h);
-    s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[s], s0, 0, 0, 0);
-    s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb, qreg[s], s1, 0, 0, 0);
+    const h8_t qq = s < PA_QLDS ? q_lds[s] : qreg[s < PA_QLDS ? 0 : s - PA_QLDS];
+    s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qq, s0, 0, 0, 0);
+    s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb, qq, s1, 0, 0, 0);
   }
 }
 // key (inside a 64-key tile) of element r of 32-key tile mt in this lane
@@ -97,7 +103,7 @@ __device__ __forceinline__ int pa_key_of(int mt, int r, int h) { return 32 * mt 
 template <bool CAUSAL>
 __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a) {
   __shared__ __align__(16) half_t ks[PA_BC * PA_KS];
-  __shared__ __align__(16) half_t vs[(PA_BC / 8) * PA_VG];
+  __shared__ __align__(16) half_t vs[(PA_BC / 4) * PA_VS];
   const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;   // the longest rows first
@@ -108,11 +114,20 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   const half_t *kp = a.k + b * a.k_b + hkv * a.k_h;
   const half_t *vp = a.v + b * a.v_b + hkv * a.v_h;
   const int my_q = q0 + 32 * w + n;
-  h8_t qreg[8];
+  // the lane's query row: 8 steps of 16 channels, of which it supplies 8 (by lane half); the first steps wait in a
+  // slot of LDS that only this lane touches (the registers are all spoken for: one spilled value costs a wait for
+  // every load in flight, every tile)
+  __shared__ __align__(16) h8_t q_slots[PA_QLDS > 0 ? PA_THREADS * PA_QLDS : 1];
+  h8_t *q_lds = q_slots + threadIdx.x * PA_QLDS;
+  h8_t qreg[8 - PA_QLDS];
   {
     const half_t *qr = qp + (int64_t)min(my_q, T - 1) * a.q_t + 8 * h;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const h8_t *>(qr + 16 * s);
+    for (int s = 0; s < 8; ++s) {
+      const h8_t x = *reinterpret_cast<const h8_t *>(qr + 16 * s);
+      if (s < PA_QLDS) q_lds[s] = x;
+      else qreg[s < PA_QLDS ? 0 : s - PA_QLDS] = x;
+    }
   }
   f16_t o[4];
 #pragma unroll
@@ -122,42 +137,47 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   const int kend = CAUSAL ? min(T, q0 + PA_BR) : T;
   const int n_tiles = (kend + PA_BC - 1) / PA_BC;
   const int wave_last_q = q0 + 32 * w + 31;
+  PaSource src;
+  src.k = make_rsrc(kp, (uint32_t)min((int64_t)T * a.k_t * 2, (int64_t)0xfffffff0));
+  src.v = make_rsrc(vp, (uint32_t)min((int64_t)T * a.v_t * 2, (int64_t)0xfffffff0));
+  src.k_row = (uint32_t)a.k_t * 2u;
+  src.v_row = (uint32_t)a.v_t * 2u;
+  src.k_lane = (uint32_t)(threadIdx.x >> 4) * src.k_row + (threadIdx.x & 15) * 16u;        // rows tid / 16 + 16 i
+  src.v_lane = (uint32_t)(threadIdx.x >> 4) * 4u * src.v_row + (threadIdx.x & 15) * 16u;   // rows 4 (tid / 16) + j
   PaTileRegs tr;
-  pa_tile_fetch(kp, a.k_t, vp, a.v_t, 0, T, tr);
+  pa_tile_fetch(src, 0, tr);
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int k0 = tile * PA_BC;
     __syncthreads();   // the previous tile has been read by every wave
     pa_tile_store(tr, ks, vs);
     __syncthreads();
-    if (tile + 1 < n_tiles) pa_tile_fetch(kp, a.k_t, vp, a.v_t, k0 + PA_BC, T, tr);   // in flight across the products
+    if (tile + 1 < n_tiles) pa_tile_fetch(src, k0 + PA_BC, tr);   // in flight across the products
     if (CAUSAL && k0 > wave_last_q) continue;   // (uniform per wave) every key of the tile lies after every query of the wave
     f16_t s[2];
-    pa_scores(ks, qreg, n, h, s[0], s[1]);
+    pa_scores(ks, qreg, q_lds, n, h, s[0], s[1]);
     const bool edge = (k0 + PA_BC > T) || (CAUSAL && k0 + PA_BC - 1 > q0 + 32 * w);   // some element of the tile is masked
     // the running maximum is kept in units of the scaled logit (base-2 exponent); a raw score enters as s * sl2
+    if (edge) {   // (uniform per wave; one branch around all 32 selects)
+      const int last_key = (CAUSAL ? min(my_q, T - 1) : T - 1) - k0 - 4 * h;   // the last visible key, relative to element r's base
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (32 * mt + 8 * (r >> 2) + (r & 3) > last_key) s[mt][r] = -INFINITY;
+    }
     float raw = -INFINITY;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        if (edge) {
-          const int key = k0 + pa_key_of(mt, r, h);
-          if (key >= T || (CAUSAL && key > my_q)) s[mt][r] = -INFINITY;
-        }
-        raw = fmaxf(raw, s[mt][r]);
-      }
+      for (int r = 0; r < 16; ++r) raw = fmaxf(raw, s[mt][r]);
     float mx = fmaxf(m, raw * sl2);   // (sl2 > 0)
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     // (the first tile always holds key 0, which no query masks: mx is finite from then on)
     if (__builtin_amdgcn_ballot_w64(mx != m) != 0) {   // somebody's maximum moved: rescale what has been added up so far
       const float alpha = __builtin_amdgcn_exp2f(m - mx);   // (the bare instruction: results below 2^-126 may flush to zero)
       lsum *= alpha;
-      // (in place by construction: left to the compiler, the products land in fresh registers and the path that skips
-      // the rescale copies all 64 accumulators to meet them)
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) asm volatile("v_mul_f32 %0, %1, %0" : "+v"(o[dt][r]) : "v"(alpha));
+      for (int dt = 0; dt < 4; ++dt) o[dt] *= alpha;
       m = mx;
     }
     float part = 0.f;
@@ -175,7 +195,9 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
-        const h8_t av = *reinterpret_cast<const h8_t *>(vs + (2 * t + h) * PA_VG + (32 * dt + n) * 8);
+        const half_t *va = vs + (4 * t + h) * PA_VS + (32 * dt + n) * 4;
+        const h4_t lo = *reinterpret_cast<const h4_t *>(va), hi = *reinterpret_cast<const h4_t *>(va + 2 * PA_VS);
+        const h8_t av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, p[t], o[dt], 0, 0, 0);
       }
   }
