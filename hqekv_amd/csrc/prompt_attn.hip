@@ -8,8 +8,10 @@
 // owns ONE query (column lane % 32): the running maximum, the sum and the rescaling of the output are per-lane
 // scalars, and the exponentials a lane holds (keys 8 g + 4 (lane / 32) + j of a 32-key tile, g = 0..3, j = 0..3) are
 // already laid out as the B operand of the second product, O^T = V^T . P^T.  That product needs, per lane, four
-// consecutive KEYS of one channel: the V tile is turned by 4 x 4 register transposes on its way into LDS
-// ([key quad][channel][4 keys]).
+// consecutive KEYS of one channel: the V tile is turned by 4 x 4 register transposes on its way into LDS, and laid out
+// [16-key step][lane half][channel slot][8 keys] so that the eight keys a lane feeds to one product -- 4 h + j and
+// 8 + 4 h + j of the step, for lane half h -- are one 16-byte read.  Channel d sits in slot d ^ ((d >> 4) & 7): the
+// sixteen writers of a row (channels 8 apart) and the 32 readers (adjacent channels) both spread over all banks.
 #include "common.h"
 
 #ifndef HQ_PA_QLDS
@@ -29,7 +31,7 @@ constexpr int PA_BR = 32 * PA_WAVES;   // query rows per workgroup
 constexpr int PA_BC = 64;              // keys per tile
 constexpr int PA_QLDS = HQ_PA_QLDS;     // of the eight 16-channel steps of a lane's query row, how many wait in LDS instead of registers
 constexpr int PA_KS = PA_D + 8;        // halfs per K row in LDS (the pad spreads the rows over the banks)
-constexpr int PA_VS = PA_D * 4 + 8;    // halfs per key quad of the turned V tile
+constexpr int PA_VG = PA_D * 8;        // halfs per (16-key step, lane half) group of the turned V tile: 128 channels x 8 keys
 
 struct PromptArgs {
   const half_t *q, *k, *v;
@@ -74,14 +76,17 @@ __device__ __forceinline__ void pa_tile_store(const PaTileRegs &r, half_t *ks, h
     const int idx = tid + PA_THREADS * i, row = idx >> 4, c = idx & 15;
     *reinterpret_cast<uint4 *>(ks + row * PA_KS + c * 8) = r.kr[i];
   }
-  // 4 keys x 8 channels -> 8 channels x 4 keys
+  // 4 keys x 8 channels -> 8 channels x 4 keys; key quad = 4 t + 2 e + h: step t, first or second four of a lane's eight, lane half h
   const int quad = tid >> 4, oct = tid & 15;
   const uint32_t a[4] = {r.vr[0].x, r.vr[0].y, r.vr[0].z, r.vr[0].w}, b[4] = {r.vr[1].x, r.vr[1].y, r.vr[1].z, r.vr[1].w};
   const uint32_t c[4] = {r.vr[2].x, r.vr[2].y, r.vr[2].z, r.vr[2].w}, e[4] = {r.vr[3].x, r.vr[3].y, r.vr[3].z, r.vr[3].w};
-  uint4 *dst = reinterpret_cast<uint4 *>(vs + quad * PA_VS + oct * 32);
+  half_t *grp = vs + (2 * (quad >> 2) + (quad & 1)) * PA_VG + ((quad >> 1) & 1) * 4;
+  const int sw = (oct >> 1) & 7;   // ((d >> 4) & 7) for this thread's channels d = 8 oct + ch
 #pragma unroll
-  for (int p = 0; p < 4; ++p)   // channels 2p and 2p + 1 of this thread's eight
-    dst[p] = make_uint4(lo_pair(a[p], b[p]), lo_pair(c[p], e[p]), hi_pair(a[p], b[p]), hi_pair(c[p], e[p]));
+  for (int p = 0; p < 4; ++p) {   // channels 2p and 2p + 1 of this thread's eight
+    *reinterpret_cast<uint2 *>(grp + (8 * oct + ((2 * p) ^ sw)) * 8) = make_uint2(lo_pair(a[p], b[p]), lo_pair(c[p], e[p]));
+    *reinterpret_cast<uint2 *>(grp + (8 * oct + ((2 * p + 1) ^ sw)) * 8) = make_uint2(hi_pair(a[p], b[p]), hi_pair(c[p], e[p]));
+  }
 }
 
 // S^T of one 64-key tile for the wave's 32 queries: two 32-key tiles, 16 fp32 values per lane each
@@ -103,7 +108,7 @@ __device__ __forceinline__ int pa_key_of(int mt, int r, int h) { return 32 * mt 
 template <bool CAUSAL>
 __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a) {
   __shared__ __align__(16) half_t ks[PA_BC * PA_KS];
-  __shared__ __align__(16) half_t vs[(PA_BC / 4) * PA_VS];
+  __shared__ __align__(16) half_t vs[(PA_BC / 8) * PA_VG];
   const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;   // the longest rows first
@@ -136,7 +141,6 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   const float sl2 = a.scale * 1.4426950408889634f;
   const int kend = CAUSAL ? min(T, q0 + PA_BR) : T;
   const int n_tiles = (kend + PA_BC - 1) / PA_BC;
-  const int wave_last_q = q0 + 32 * w + 31;
   PaSource src;
   src.k = make_rsrc(kp, (uint32_t)min((int64_t)T * a.k_t * 2, (int64_t)0xfffffff0));
   src.v = make_rsrc(vp, (uint32_t)min((int64_t)T * a.v_t * 2, (int64_t)0xfffffff0));
@@ -152,7 +156,8 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     pa_tile_store(tr, ks, vs);
     __syncthreads();
     if (tile + 1 < n_tiles) pa_tile_fetch(src, k0 + PA_BC, tr);   // in flight across the products
-    if (CAUSAL && k0 > wave_last_q) continue;   // (uniform per wave) every key of the tile lies after every query of the wave
+    // (a tile that lies after every query of this wave is worked through like any other: all its elements are masked,
+    // the maximum stays and the exponentials are zeros; skipping it would cost a copy of the accumulators per tile)
     f16_t s[2];
     pa_scores(ks, qreg, q_lds, n, h, s[0], s[1]);
     const bool edge = (k0 + PA_BC > T) || (CAUSAL && k0 + PA_BC - 1 > q0 + 32 * w);   // some element of the tile is masked
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     float mx = fmaxf(m, raw * sl2);   // (sl2 > 0)
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     // (the first tile always holds key 0, which no query masks: mx is finite from then on)
-    if (__builtin_amdgcn_ballot_w64(mx != m) != 0) {   // somebody's maximum moved: rescale what has been added up so far
+    {
       const float alpha = __builtin_amdgcn_exp2f(m - mx);   // (the bare instruction: results below 2^-126 may flush to zero)
       lsum *= alpha;
 #pragma unroll
@@ -195,9 +200,8 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
-        const half_t *va = vs + (4 * t + h) * PA_VS + (32 * dt + n) * 4;
-        const h4_t lo = *reinterpret_cast<const h4_t *>(va), hi = *reinterpret_cast<const h4_t *>(va + 2 * PA_VS);
-        const h8_t av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const int d = 32 * dt + n;
+        const h8_t av = *reinterpret_cast<const h8_t *>(vs + (2 * t + h) * PA_VG + (d ^ ((d >> 4) & 7)) * 8);
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, p[t], o[dt], 0, 0, 0);
       }
   }
