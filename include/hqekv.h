@@ -339,6 +339,7 @@ int hqekv_token_range(const void *v, int64_t B, int64_t H, int64_t T, int64_t D,
  * where they lie; K and V have Hkv heads, query head h reads KV head h / (Hq / Hkv).
  *   hqekv_prompt_attn       out (B, Hq, T, 128, strides as given) = softmax(q k^T * scale [causal]) v, fp32
  *                           accumulation and running softmax, probabilities rounded to fp16 before the second product
+ *                           (scale > 0; B * Hq <= 65535)
  *   hqekv_prompt_last_rows  probs (B, Hq, R, T) contiguous: the probabilities of the last R <= 32 query rows with the
  *                           reference's roundings -- product to fp16, times scale to fp16, plus mask to fp16, floored
  *                           at -65504, softmax in fp32, to fp16.  mask: additive fp16 (B, 1, R, T) given by its batch

@@ -122,6 +122,8 @@ def test_prompt_entries_refuse_bad_arguments():
         prompt_last_rows(q, k, 0.1, 0)
     with pytest.raises(Exception):
         prompt_attention(q, k[:, :1].expand(1, 3, 40, 128), v, 0.1)   # 4 query heads over 3 KV heads
+    with pytest.raises(Exception):
+        prompt_attention(q, k, v, -0.1)                               # the running maximum assumes a positive scale
 
 
 def test_layer_prompt_without_a_mask_equals_the_causal_mask():
