@@ -144,3 +144,25 @@ def test_layer_prompt_without_a_mask_equals_the_causal_mask():
     assert len(pkv_a) == len(pkv_b) == 42
     for fa, fb in zip(pkv_a, pkv_b):
         assert (fa is None) == (fb is None)
+
+
+def test_prompt_attention_at_full_size_against_torch_fused_attention():
+    """The benchmark's shape (B=1, 32 query heads over 8 KV heads, 32768 tokens): against torch's own fused attention
+    on the device -- two fp16-probability implementations, so the tolerance is twice the one against fp32 --, and the
+    rows of the last block against the fp32 definition."""
+    from hqekv_amd.prompt_attention import prompt_attention
+    B, Hq, Hkv, T = 1, 32, 8, 32768
+    g = torch.Generator(device=_dev()).manual_seed(99)
+    q = torch.randn(B, Hq, T, 128, generator=g, device=_dev(), dtype=torch.float16)
+    k = torch.randn(B, Hkv, T, 128, generator=g, device=_dev(), dtype=torch.float16)
+    v = torch.randn(B, Hkv, T, 128, generator=g, device=_dev(), dtype=torch.float16)
+    scale = 1.0 / math.sqrt(128)
+    out = prompt_attention(q, k, v, scale)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale, enable_gqa=True)
+    torch.testing.assert_close(out.float(), ref.float(), rtol=4e-3, atol=4e-3)
+    # the last 64 rows of two heads, dense in fp32
+    for h in (0, 31):
+        s = (q[0, h, -64:].float() @ k[0, h // 4].float().T) * scale
+        keep = torch.arange(T, device=_dev())[None, :] <= torch.arange(T - 64, T, device=_dev())[:, None]
+        want = torch.softmax(s.masked_fill(~keep, float("-inf")), dim=-1) @ v[0, h // 4].float()
+        torch.testing.assert_close(out[0, h, -64:].float(), want, rtol=2e-3, atol=2e-3)
