@@ -39,13 +39,13 @@ WORKLOADS = {
 
 
 def kernel_source_sha16() -> str:
-    """Hash of the HIP sources the library is built from: recorded next to counter-derived figures so that a
-    figure measured on other kernels is recognised as stale."""
+    """Hash of the HIP sources the decode-attention kernels are built from (attn.hip and the headers): recorded next
+    to counter-derived figures so that a figure measured on other kernels is recognised as stale."""
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "hqekv_amd", "csrc")
     for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".h")):
+        if name == "attn.hip" or name.endswith(".h"):
             h.update(name.encode())
             h.update(open(os.path.join(csrc, name), "rb").read())
     return h.hexdigest()[:16]

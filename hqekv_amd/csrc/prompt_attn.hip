@@ -178,7 +178,11 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     float mx = fmaxf(m, raw * sl2);   // (sl2 > 0)
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     // (the first tile always holds key 0, which no query masks: mx is finite from then on)
-    {
+    // Per lane on purpose: a divergent branch keeps the accumulators where they are (inactive lanes must keep their
+    // values, so the products are in place under the execution mask, skipped when no lane needs them); a wave-uniform
+    // branch made the compiler copy all 64 accumulators per tile, and without a branch the 64 products are a quarter
+    // of the tile's vector instructions.
+    if (mx != m) {   // this query's maximum moved: rescale what it has added up so far
       const float alpha = __builtin_amdgcn_exp2f(m - mx);   // (the bare instruction: results below 2^-126 may flush to zero)
       lsum *= alpha;
 #pragma unroll
