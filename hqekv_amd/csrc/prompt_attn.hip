@@ -142,8 +142,8 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   const int kend = CAUSAL ? min(T, q0 + PA_BR) : T;
   const int n_tiles = (kend + PA_BC - 1) / PA_BC;
   PaSource src;
-  src.k = make_rsrc(kp, (uint32_t)min((int64_t)T * a.k_t * 2, (int64_t)0xfffffff0));
-  src.v = make_rsrc(vp, (uint32_t)min((int64_t)T * a.v_t * 2, (int64_t)0xfffffff0));
+  src.k = make_rsrc(kp, (uint32_t)((int64_t)T * a.k_t * 2));   // (below 4 GiB: checked by the host)
+  src.v = make_rsrc(vp, (uint32_t)((int64_t)T * a.v_t * 2));
   src.k_row = (uint32_t)a.k_t * 2u;
   src.v_row = (uint32_t)a.v_t * 2u;
   src.k_lane = (uint32_t)(threadIdx.x >> 4) * src.k_row + (threadIdx.x & 15) * 16u;        // rows tid / 16 + 16 i
@@ -347,6 +347,9 @@ extern "C" int hqekv_prompt_attn(const void *q, const int64_t *q_strides, const 
   if (!rows_16_byte_aligned(q, q_strides[0], q_strides[1], q_strides[2]) || !rows_16_byte_aligned(k, k_strides[0], k_strides[1], k_strides[2]) ||
       !rows_16_byte_aligned(v, v_strides[0], v_strides[1], v_strides[2]) || ((uintptr_t)out & 7) || out_strides[0] % 4 || out_strides[1] % 4 || out_strides[2] % 4)
     return fail(HQEKV_E_ALIGN, "prompt_attn: rows of q, k, v must be 16-byte aligned (of out: 8-byte)");
+  // (the tiles of K and V are fetched through 32-bit buffer offsets from each head's first row)
+  if (T * k_strides[2] * 2 >= (1LL << 32) || T * v_strides[2] * 2 >= (1LL << 32) || k_strides[2] <= 0 || v_strides[2] <= 0)
+    return fail(HQEKV_E_UNSUPPORTED, "prompt_attn: a head's K or V rows must span less than 4 GiB (T * token stride * 2 bytes)");
   PromptArgs a;
   a.q = (const half_t *)q; a.k = (const half_t *)k; a.v = (const half_t *)v; a.out = (half_t *)out;
   a.q_b = q_strides[0]; a.q_h = q_strides[1]; a.q_t = q_strides[2];
