@@ -47,7 +47,7 @@ EXPORTS = (
     "hqekv_qk_hybrid", "hqekv_scale_softmax", "hqekv_pv_workspace_bytes", "hqekv_pv_hybrid",
     "hqekv_decode_workspace_bytes", "hqekv_decode_attn", "hqekv_decode_attn_static", "hqekv_decode_step", "hqekv_ring_row",
     "hqekv_importance_scores", "hqekv_weighted_block_scores", "hqekv_token_range",
-    "hqekv_prompt_attn", "hqekv_prompt_last_rows",
+    "hqekv_prompt_attn", "hqekv_prompt_last_rows", "hqekv_prompt_last_rows_workspace_bytes",
     "hqekv_cache_migrate", "hqekv_plan_side",
 )
 
@@ -130,7 +130,8 @@ _PROTOS = {
     "hqekv_weighted_block_scores": (C.c_int, [_vp, _vp, _i64, _vp, _vp]),
     "hqekv_token_range": (C.c_int, [_vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
     "hqekv_prompt_attn": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _int, _vp]),
-    "hqekv_prompt_last_rows": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp]),
+    "hqekv_prompt_last_rows": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp, _i64, _vp]),
+    "hqekv_prompt_last_rows_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "hqekv_decode_attn_static": (C.c_int, [_SEGP, _int, _SEGP, _int, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]),
     "hqekv_plan_side": (C.c_int, [C.POINTER(_vp), _vp, C.c_int32, C.c_int32, _vp, _vp, C.c_int32, _vp, _vp, _vp, _vp]),
     "hqekv_cache_migrate": (C.c_int, [_int, _CCP, _int, _CCP, _int, _vp, _i64, _i64, _vp, _vp]),

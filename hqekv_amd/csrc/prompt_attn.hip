@@ -238,8 +238,14 @@ struct LastRowsArgs {
   int64_t m_b, m_r;
   int32_t Hq, Hkv, T, R;
   float scale;
+  float2 *partial;      // (B * Hq, slices, 32) (maximum, sum) of a slice of the keys, or nullptr: one workgroup per head does it all
+  int32_t slices;
 };
 
+// PHASE 0: one workgroup per (b, query head) walks all keys twice.  With the keys cut into slices (grid.y) for short
+// prompts and small batches: PHASE 1 leaves each slice's (maximum, sum) per row in `partial`, PHASE 2 merges them and
+// writes the slice's probabilities.
+template <int PHASE>
 __global__ __launch_bounds__(PA_THREADS, 2) void prompt_last_rows_kernel(LastRowsArgs a) {
   __shared__ float sh_m[PA_WAVES][32], sh_l[PA_WAVES][32];
   const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -256,7 +262,9 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_last_rows_kernel(LastRow
     for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const h8_t *>(qr + 16 * s);
   }
   const half_t *mrow = a.mask ? a.mask + b * a.m_b + (int64_t)row * a.m_r : nullptr;
-  const int n_tiles = (T + 31) / 32;
+  const int all_tiles = (T + 31) / 32;
+  const int per_slice = PHASE == 0 ? all_tiles : (all_tiles + a.slices - 1) / a.slices;
+  const int tile0 = PHASE == 0 ? 0 : (int)blockIdx.y * per_slice, n_tiles = min(all_tiles, tile0 + per_slice);
   // the 16 scores of this lane for 32-key tile `tile`, as the reference's fp16 chain leaves them (in fp32)
   auto tile_scores = [&](int tile, float (&x)[16]) {
     const int key_row = min(32 * tile + n, T - 1);
@@ -279,20 +287,21 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_last_rows_kernel(LastRow
     }
   };
   float m = -INFINITY, l = 0.f;
-  for (int tile = w; tile < n_tiles; tile += PA_WAVES) {
-    float x[16];
-    tile_scores(tile, x);
-    float mx = m;
+  if (PHASE != 2) {
+    for (int tile = tile0 + w; tile < n_tiles; tile += PA_WAVES) {
+      float x[16];
+      tile_scores(tile, x);
+      float mx = m;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, x[r]);
-    if (mx == -INFINITY) continue;   // nothing but masked keys so far
-    float part = 0.f;
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, x[r]);
+      if (mx == -INFINITY) continue;   // nothing but masked keys so far
+      float part = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) part += __expf(x[r] - mx);
-    l = l * __expf(m - mx) + part;
-    m = mx;
-  }
-  {  // the two halves of the wave, then the four waves
+      for (int r = 0; r < 16; ++r) part += __expf(x[r] - mx);
+      l = l * __expf(m - mx) + part;
+      m = mx;
+    }
+    // the two halves of the wave, then the four waves
     const float mo = __shfl_xor(m, 32, 64), lo = __shfl_xor(l, 32, 64);
     const float mx = fmaxf(m, mo);
     l = (m == -INFINITY ? 0.f : l * __expf(m - mx)) + (mo == -INFINITY ? 0.f : lo * __expf(mo - mx));
@@ -310,10 +319,21 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_last_rows_kernel(LastRow
     for (int k = 0; k < PA_WAVES; ++k) tot += sh_m[k][n] == -INFINITY ? 0.f : sh_l[k][n] * __expf(sh_m[k][n] - mx2);
     m = mx2;
     l = tot;
+    if (PHASE == 1) {
+      if (threadIdx.x < 32) a.partial[((int64_t)blockIdx.x * a.slices + blockIdx.y) * 32 + n] = make_float2(m, l);
+      return;
+    }
+  } else {   // merge the slices' statistics, in slice order
+    const float2 *ps = a.partial + (int64_t)blockIdx.x * a.slices * 32 + n;
+    for (int sl = 0; sl < a.slices; ++sl) m = fmaxf(m, ps[sl * 32].x);
+    for (int sl = 0; sl < a.slices; ++sl) {
+      const float2 v = ps[sl * 32];
+      l += v.x == -INFINITY ? 0.f : v.y * __expf(v.x - m);
+    }
   }
   const float inv = 1.0f / l;
   half_t *prow = a.probs + (((int64_t)b * a.Hq + hq) * R + row) * (int64_t)T;
-  for (int tile = w; tile < n_tiles; tile += PA_WAVES) {
+  for (int tile = tile0 + w; tile < n_tiles; tile += PA_WAVES) {
     float x[16];
     tile_scores(tile, x);
     if (n >= R) continue;
@@ -363,9 +383,25 @@ extern "C" int hqekv_prompt_attn(const void *q, const int64_t *q_strides, const 
   return check_launch("prompt_attn");
 }
 
+static int last_rows_slices(int64_t B, int64_t Hq, int64_t T) {
+  // enough workgroups for the chip when there are few heads; a slice keeps at least 2048 keys
+  int64_t s = (512 + B * Hq - 1) / (B * Hq);
+  const int64_t most = (T + 2047) / 2048;
+  if (s > most) s = most;
+  if (s > 64) s = 64;
+  return s < 1 ? 1 : (int)s;
+}
+
+extern "C" int64_t hqekv_prompt_last_rows_workspace_bytes(int64_t B, int64_t Hq, int64_t T) {
+  if (B <= 0 || Hq <= 0 || T <= 0) return -1;
+  const int sl = last_rows_slices(B, Hq, T);
+  return sl > 1 ? B * Hq * sl * 32 * (int64_t)sizeof(float2) : 0;
+}
+
 extern "C" int hqekv_prompt_last_rows(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides,
                                       const void *mask, const int64_t *mask_strides, void *probs, int64_t B, int64_t Hq,
-                                      int64_t Hkv, int64_t T, int64_t D, int64_t R, float scale, void *stream) {
+                                      int64_t Hkv, int64_t T, int64_t D, int64_t R, float scale, void *workspace,
+                                      int64_t workspace_bytes, void *stream) {
   if (!q || !k || !probs || !q_strides || !k_strides || (mask && !mask_strides)) return fail(HQEKV_E_ARG, "prompt_last_rows: null pointer");
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv || R <= 0 || R > 32 || R > T)
     return fail(HQEKV_E_ARG, "prompt_last_rows: need B > 0, Hq %% Hkv == 0 and 0 < R <= min(32, T)");
@@ -379,6 +415,20 @@ extern "C" int hqekv_prompt_last_rows(const void *q, const int64_t *q_strides, c
   a.k_b = k_strides[0]; a.k_h = k_strides[1]; a.k_t = k_strides[2];
   a.m_b = mask ? mask_strides[0] : 0; a.m_r = mask ? mask_strides[1] : 0;
   a.Hq = (int32_t)Hq; a.Hkv = (int32_t)Hkv; a.T = (int32_t)T; a.R = (int32_t)R; a.scale = scale;
-  hipLaunchKernelGGL(prompt_last_rows_kernel, dim3((unsigned)(B * Hq)), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+  // the keys in slices when the caller brought room for the slices' statistics; else one workgroup per head
+  const int sl = last_rows_slices(B, Hq, T);
+  const int64_t need = hqekv_prompt_last_rows_workspace_bytes(B, Hq, T);
+  if (sl > 1 && workspace && workspace_bytes >= need) {
+    if ((uintptr_t)workspace & 7) return fail(HQEKV_E_ALIGN, "prompt_last_rows: workspace not 8-byte aligned");
+    a.partial = (float2 *)workspace;
+    a.slices = sl;
+    const dim3 grid((unsigned)(B * Hq), (unsigned)sl);
+    hipLaunchKernelGGL(prompt_last_rows_kernel<1>, grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(prompt_last_rows_kernel<2>, grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+  } else {
+    a.partial = nullptr;
+    a.slices = 1;
+    hipLaunchKernelGGL(prompt_last_rows_kernel<0>, dim3((unsigned)(B * Hq)), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+  }
   return check_launch("prompt_last_rows");
 }

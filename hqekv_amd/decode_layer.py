@@ -68,7 +68,9 @@ def last_rows_probabilities(q, k, attention_mask, scaling, rows):
     computes them for the importance ring (model/llama_hqe.py:156-168): the library's kernel for fp16 tensors of
     head_dim 128 (same roundings; without a mask the causal rule), torch otherwise.  The query heads that share a KV
     head are folded into the row dimension of one batched product instead of materialising ``repeat_kv`` copies."""
-    if rows <= prompt_attention.MAX_LAST_ROWS and prompt_attention.supported(q, k):
+    mask_fits = attention_mask is None or (attention_mask.dim() == 4 and attention_mask.shape[1] == 1
+                                           and attention_mask.shape[0] in (1, q.shape[0]) and attention_mask.shape[3] == q.shape[2])
+    if rows <= prompt_attention.MAX_LAST_ROWS and mask_fits and prompt_attention.supported(q, k):
         return prompt_attention.prompt_last_rows(q, k, scaling, rows, attention_mask)
     B, Hq, T, D = q.shape
     Hkv = k.shape[1]

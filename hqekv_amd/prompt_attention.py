@@ -49,9 +49,10 @@ def prompt_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scaling:
 
 
 def prompt_last_rows(q: torch.Tensor, k: torch.Tensor, scaling: float, rows: int,
-                     attention_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     attention_mask: Optional[torch.Tensor] = None, sliced: bool = True) -> torch.Tensor:
     """Probabilities of the last ``rows`` query rows over all keys -> (B, Hq, rows, T) fp16, with the reference's
-    roundings.  ``attention_mask``: additive (B or 1, 1, >= rows, T), its last ``rows`` rows are used; None: causal."""
+    roundings.  ``attention_mask``: additive (B or 1, 1, >= rows, T), its last ``rows`` rows are used; None: causal.
+    ``sliced``: let the library cut the keys into slices over more workgroups (two launches) when there are few heads."""
     if not supported(q, k):
         raise NotImplementedError("prompt_last_rows: fp16 CUDA tensors of head_dim 128 only")
     B, Hq, T, D = q.shape
@@ -61,15 +62,21 @@ def prompt_last_rows(q: torch.Tensor, k: torch.Tensor, scaling: float, rows: int
     q, k = _rows(q), _rows(k)
     m_ptr, m_str = None, None
     if attention_mask is not None:
+        if attention_mask.dim() != 4 or attention_mask.shape[1] != 1 or attention_mask.shape[3] != T \
+                or attention_mask.shape[0] not in (1, B) or attention_mask.shape[2] < rows:
+            raise ValueError(f"prompt_last_rows: mask of shape {tuple(attention_mask.shape)} (expected (B or 1, 1, >= rows, T))")
         m = attention_mask[:, :, -rows:, :]
-        if m.dtype != q.dtype or m.stride(3) != 1 or m.shape[3] != T or m.shape[1] != 1:
-            m = m[:, :1].to(q.dtype).contiguous()
+        if m.dtype != q.dtype or m.stride(3) != 1:
+            m = m.to(q.dtype).contiguous()
         m_ptr = m.data_ptr()
         m_str = (C.c_int64 * 2)(m.stride(0) if m.shape[0] > 1 else 0, m.stride(2))
     probs = torch.empty((B, Hq, rows, T), dtype=q.dtype, device=q.device)
+    lib = _lib.load()
+    ws_bytes = lib.hqekv_prompt_last_rows_workspace_bytes(B, Hq, T) if sliced else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes > 0 else None
     with _lib.on_device(q.device):
-        rc = _lib.load().hqekv_prompt_last_rows(q.data_ptr(), _strides(q), k.data_ptr(), _strides(k), m_ptr, m_str,
-                                                probs.data_ptr(), B, Hq, Hkv, T, D, rows, float(scaling),
-                                                _lib.stream_ptr(q.device))
+        rc = lib.hqekv_prompt_last_rows(q.data_ptr(), _strides(q), k.data_ptr(), _strides(k), m_ptr, m_str,
+                                        probs.data_ptr(), B, Hq, Hkv, T, D, rows, float(scaling),
+                                        ws.data_ptr() if ws is not None else None, ws_bytes, _lib.stream_ptr(q.device))
     _lib.check(rc, "prompt_last_rows")
     return probs

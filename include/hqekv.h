@@ -344,13 +344,17 @@ int hqekv_token_range(const void *v, int64_t B, int64_t H, int64_t T, int64_t D,
  *                           reference's roundings -- product to fp16, times scale to fp16, plus mask to fp16, floored
  *                           at -65504, softmax in fp32, to fp16.  mask: additive fp16 (B, 1, R, T) given by its batch
  *                           and row strides (key stride 1), or NULL for the causal rule (row r sees keys <= T - R + r).
+ *                           workspace (hqekv_prompt_last_rows_workspace_bytes, may be 0): room for per-slice statistics,
+ *                           with which few heads are spread over the chip in two launches; NULL: one workgroup per head.
  */
 int hqekv_prompt_attn(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides, const void *v,
                       const int64_t *v_strides, void *out, const int64_t *out_strides, int64_t B, int64_t Hq, int64_t Hkv,
                       int64_t T, int64_t D, float scale, int causal, void *stream);
+int64_t hqekv_prompt_last_rows_workspace_bytes(int64_t B, int64_t Hq, int64_t T);
 int hqekv_prompt_last_rows(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides,
                            const void *mask, const int64_t *mask_strides, void *probs, int64_t B, int64_t Hq, int64_t Hkv,
-                           int64_t T, int64_t D, int64_t R, float scale, void *stream);
+                           int64_t T, int64_t D, int64_t R, float scale, void *workspace, int64_t workspace_bytes,
+                           void *stream);
 
 /* ------------------------------------------------------------------ cache maintenance (one launch per side)
  * Replaces the per-(source, target) gathers, dequantise / re-quantise calls and torch.cat re-copies of one

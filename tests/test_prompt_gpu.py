@@ -120,6 +120,8 @@ def test_prompt_entries_refuse_bad_arguments():
         prompt_last_rows(q, k, 0.1, 33)
     with pytest.raises(ValueError):
         prompt_last_rows(q, k, 0.1, 0)
+    with pytest.raises(ValueError):
+        prompt_last_rows(q, k, 0.1, 20, attention_mask=torch.zeros(1, 4, 40, 40, dtype=torch.float16, device=q.device))   # a mask per head
     with pytest.raises(Exception):
         prompt_attention(q, k[:, :1].expand(1, 3, 40, 128), v, 0.1)   # 4 query heads over 3 KV heads
     with pytest.raises(Exception):
@@ -166,3 +168,20 @@ def test_prompt_attention_at_full_size_against_torch_fused_attention():
         keep = torch.arange(T, device=_dev())[None, :] <= torch.arange(T - 64, T, device=_dev())[:, None]
         want = torch.softmax(s.masked_fill(~keep, float("-inf")), dim=-1) @ v[0, h // 4].float()
         torch.testing.assert_close(out[0, h, -64:].float(), want, rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T,rows", [(1, 4, 1, 9000, 20), (1, 32, 8, 32768, 20), (2, 8, 2, 4097, 32)])
+def test_last_rows_in_key_slices_equal_the_single_workgroup_form(B, Hq, Hkv, T, rows):
+    """Few heads: the keys are cut into slices over more workgroups (two launches and a workspace).  Same
+    probabilities as one workgroup per head, to the last fp16 step or two (the slices' sums are merged in another
+    order), and both within tolerance of the reference chain."""
+    from hqekv_amd import _lib
+    from hqekv_amd.prompt_attention import prompt_last_rows
+    assert _lib.load().hqekv_prompt_last_rows_workspace_bytes(B, Hq, T) > 0
+    q, k, _ = _qkv(B, Hq, Hkv, T, 3000 + T)
+    scale = 1.0 / math.sqrt(128)
+    a = prompt_last_rows(q, k, scale, rows, sliced=True)
+    b = prompt_last_rows(q, k, scale, rows, sliced=False)
+    torch.testing.assert_close(a.float(), b.float(), rtol=2e-3, atol=2e-6)
+    want = _reference_last_rows(q, k, scale, rows, _causal_mask(T, q.device))
+    torch.testing.assert_close(a.float(), want.float(), rtol=2e-3, atol=2e-6)
