@@ -283,19 +283,18 @@ def bench_quantize(args):
 
 
 # ------------------------------------------------------------------------------------------------ prompt side
-def bench_prompt(args):
-    """The prompt's attention (what the reference takes from flash-attention) and the probabilities of its last 20
-    rows, on the library's matrix-core kernels; torch's fused attention on the same tensors beside it."""
+def measure_prompt(T: int, steps: int, warm: int) -> dict:
+    """Causal prompt attention (B=1, Hq=32, Hkv=8, D=128, fp16) and the last 20 rows' probabilities on the library's
+    matrix-core kernels, torch's fused attention on the same tensors beside it."""
     import math
     from hqekv_amd.prompt_attention import prompt_attention, prompt_last_rows
     dev = torch.device("cuda:0")
-    B, Hq, Hkv, T, D, R = 1, 32, 8, args.prompt_len if args.prompt_len != 131072 else 32768, 128, 20
+    B, Hq, Hkv, D, R = 1, 32, 8, 128, 20
     g = torch.Generator(device=dev).manual_seed(1241)
     q = torch.randn(B, Hq, T, D, generator=g, device=dev, dtype=torch.float16)
     k = torch.randn(B, Hkv, T, D, generator=g, device=dev, dtype=torch.float16)
     v = torch.randn(B, Hkv, T, D, generator=g, device=dev, dtype=torch.float16)
     scale = 1.0 / math.sqrt(D)
-    steps, warm = max(1, min(args.steps, 20)), max(1, min(args.warmup, 3))
 
     def timed(fn):
         for _ in range(warm):
@@ -308,25 +307,34 @@ def bench_prompt(args):
         b.record()
         torch.cuda.synchronize()
         return a.elapsed_time(b) / steps
+
+    def fused(): return torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale, enable_gqa=True)
     ms = timed(lambda: prompt_attention(q, k, v, scale))
     ms_rows = timed(lambda: prompt_last_rows(q, k, scale, R))
-    ms_torch = timed(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale, enable_gqa=True))
+    ms_torch = timed(fused)
     flop = 4.0 * B * Hq * (T * (T + 1) / 2) * D   # two products, causal: T (T + 1) / 2 (query, key) pairs
-    out = prompt_attention(q, k, v, scale)
-    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale, enable_gqa=True)
+    diff = float((prompt_attention(q, k, v, scale).float() - fused().float()).abs().max())
     torch.cuda.synchronize()
     tf = flop / (ms * 1e-3) / 1e12
+    return {"T": T, "steps": steps, "warmup": warm, "ms": round(ms, 4), "TFLOP/s": round(tf, 1), "last_rows_ms": round(ms_rows, 4),
+            "torch_fused_attention": {"ms": round(ms_torch, 4), "TFLOP/s": round(flop / (ms_torch * 1e-3) / 1e12, 1),
+                                      "note": "torch.nn.functional.scaled_dot_product_attention(is_causal, enable_gqa) on the same tensors, same process"},
+            "max_abs_difference_from_torch": diff,
+            "roofline": {"bound": "mfma", "kernel": "prompt_attn_kernel<true>", "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                         "frac": round(tf / 2500.0, 4), "traffic": None}}
+
+
+def bench_prompt(args):
+    T = args.prompt_len if args.prompt_len != 131072 else 32768
+    steps, warm = max(1, min(args.steps, 20)), max(1, min(args.warmup, 3))
+    m = measure_prompt(T, steps, warm)
     print(json.dumps({
-        "metric": "TFLOP/s of the causal prompt attention (fp16, fp32 accumulation)", "value": round(tf, 1), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "metric": "TFLOP/s of the causal prompt attention (fp16, fp32 accumulation)", "value": m["TFLOP/s"], "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": m["ms"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"prompt: {WORKLOADS['prompt']}", "T": T},
-        "last_rows_ms": round(ms_rows, 4),
-        "torch_fused_attention": {"ms": round(ms_torch, 4), "TFLOP/s": round(flop / (ms_torch * 1e-3) / 1e12, 1),
-                                  "note": "torch.nn.functional.scaled_dot_product_attention(is_causal, enable_gqa) on the same tensors, same process"},
-        "max_abs_difference_from_torch": float((out.float() - ref.float()).abs().max()),
-        "roofline": {"bound": "mfma", "kernel": "prompt_attn_kernel<true>", "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s",
-                     "frac": round(tf / 2500.0, 4), "traffic": None},
+        "last_rows_ms": m["last_rows_ms"], "torch_fused_attention": m["torch_fused_attention"],
+        "max_abs_difference_from_torch": m["max_abs_difference_from_torch"], "roofline": m["roofline"],
     }))
 
 
@@ -713,6 +721,13 @@ def main():
             torch.cuda.empty_cache()
         except torch.OutOfMemoryError as e:   # a smaller GPU: the headline stands on its own
             out["extra"] = {"skipped": f"configuration 4 does not fit: {e}"}
+
+    if args.workload == "c2" and not args.no_extra:
+        # the prompt side beside the headline: a short run of the causal prompt attention (16384 tokens)
+        try:
+            out["extra_prompt"] = measure_prompt(16384, 5, 2)
+        except (torch.OutOfMemoryError, RuntimeError) as e:
+            out["extra_prompt"] = {"skipped": str(e)[:200]}
 
     if args.workload == "c5":
         # one generated token passes through every resident layer once
