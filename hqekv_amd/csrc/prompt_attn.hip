@@ -29,7 +29,7 @@ constexpr int PA_WAVES = 4;
 constexpr int PA_THREADS = 64 * PA_WAVES;
 constexpr int PA_BR = 32 * PA_WAVES;   // query rows per workgroup
 constexpr int PA_BC = 64;              // keys per tile
-constexpr int PA_QLDS = HQ_PA_QLDS;     // of the eight 16-channel steps of a lane's query row, how many wait in LDS instead of registers
+constexpr int PA_QLDS = HQ_PA_QLDS;    // of the eight 16-channel steps of a lane's query row, how many wait in LDS instead of registers
 constexpr int PA_KS = PA_D + 8;        // halfs per K row in LDS (the pad spreads the rows over the banks)
 constexpr int PA_VG = PA_D * 8;        // halfs per (16-key step, lane half) group of the turned V tile: 128 channels x 8 keys
 
@@ -97,14 +97,11 @@ __device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8
   for (int s = 0; s < 8; ++s) {
     const h8_t ka = *reinterpret_cast<const h8_t *>(ks + n * PA_KS + 16 * s + 8 * h);
     const h8_t kb = *reinterpret_cast<const h8_t *>(ks + (32 + n) * PA_KS + 16 * s + 8 * h);
-    const h8_t qq = s < PA_QLDS ? q_lds[s] : qreg[s < PA_QLDS ? 0 : s - PA_QLDS];
+    const h8_t qq = s < PA_QLDS ? q_lds[s * PA_THREADS] : qreg[s < PA_QLDS ? 0 : s - PA_QLDS];
     s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qq, s0, 0, 0, 0);
     s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb, qq, s1, 0, 0, 0);
   }
 }
-// key (inside a 64-key tile) of element r of 32-key tile mt in this lane
-__device__ __forceinline__ int pa_key_of(int mt, int r, int h) { return 32 * mt + 8 * (r >> 2) + 4 * h + (r & 3); }
-
 template <bool CAUSAL>
 __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a) {
   __shared__ __align__(16) half_t ks[PA_BC * PA_KS];
@@ -123,14 +120,14 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   // slot of LDS that only this lane touches (the registers are all spoken for: one spilled value costs a wait for
   // every load in flight, every tile)
   __shared__ __align__(16) h8_t q_slots[PA_QLDS > 0 ? PA_THREADS * PA_QLDS : 1];
-  h8_t *q_lds = q_slots + threadIdx.x * PA_QLDS;
+  h8_t *q_lds = q_slots + threadIdx.x;   // step s at q_lds[s * PA_THREADS]: adjacent lanes 16 bytes apart
   h8_t qreg[8 - PA_QLDS];
   {
     const half_t *qr = qp + (int64_t)min(my_q, T - 1) * a.q_t + 8 * h;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const h8_t x = *reinterpret_cast<const h8_t *>(qr + 16 * s);
-      if (s < PA_QLDS) q_lds[s] = x;
+      if (s < PA_QLDS) q_lds[s * PA_THREADS] = x;
       else qreg[s < PA_QLDS ? 0 : s - PA_QLDS] = x;
     }
   }
