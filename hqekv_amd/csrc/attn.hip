@@ -95,7 +95,15 @@ struct FuseArgs {
   uint32_t *arrive;
   half_t *out;         // (B*Hq, D) attention output, written by the last workgroup of each (b, kv head)
   int32_t two_step;    // never fold the bias removal of a code into its multiply (HQEKV_TWO_STEP_DEQUANT)
+  // A ratio of query heads to KV heads that no kernel is instantiated for (3, 5, 6, 7, 12, ...) is served in slices of
+  // 8, 4, 2 or 1 heads per KV head, one launch each: the launch's NREP heads are heads head_off .. head_off + NREP - 1
+  // of the head_group query heads of their KV head.  head_group 0: the launch covers all NREP heads (the usual case).
+  int32_t head_group, head_off;
 };
+// first query head (inside its batch row) that a workgroup of KV head `hkv` works on
+__device__ __forceinline__ int first_head(const FuseArgs &fz, int hkv, int nrep) {
+  return fz.head_group ? hkv * fz.head_group + fz.head_off : hkv * nrep;
+}
 
 // What the caller of a decode step does next to the attention (model/llama_hqe.py:131-133, 200), folded into the
 // step's last launch: the row of the importance ring -- the probabilities summed over the batch, rounded to fp16,
@@ -642,7 +650,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
           l_run[h] = l_run[h] * keep + wave_sum(e);
           m_run[h] = mn;
         }
-        if (valid && lg == 0) scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = rr;
+        if (valid && lg == 0) scores[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall + pos] = rr;
       }
     }
   } else {
@@ -668,7 +676,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
           l_run[h] = l_run[h] * __expf(m_run[h] - mn) + __expf(x - mn);
           m_run[h] = mn;
         }
-        if (lane == 0) scores[((int64_t)b * Hq + hkv * NREP + h) * Tall + pos] = r;
+        if (lane == 0) scores[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall + pos] = r;
       }
     }
   }
@@ -689,7 +697,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
         const float lw = red[(w * NREP + h) * 2 + 1];
         if (lw > 0.f) l += lw * __expf(red[(w * NREP + h) * 2] - m);
       }
-      fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+      fz.stats[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
     }
   }
 }
@@ -728,7 +736,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   const int tile_end = min(tile_begin + tpw, (int)sg.n_units);
   const bool tm = sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR;
   const uint32_t n = (uint32_t)sg.n_tokens;
-  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * D);
+  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + first_head(fz, hkv, NREP)) * D);
   // The query is staged by the first tile only; for every tile the call is the workgroup barrier between
   // "first loads requested" and "arithmetic starts", and between two tiles' uses of the reduction buffer.
   bool staged = false;
@@ -839,7 +847,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
           if (lane == 0) wave_ml[h][wave - hl * WPH] = make_float2(m, l);
         }
         if (tok < n) {
-          half_t *srow = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+          half_t *srow = scores + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall;
           // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
           // vector store; otherwise 2-byte scatters through idx
           if (contig && (((uintptr_t)(srow + pos[0])) & (VPT * 2 - 1)) == 0) {
@@ -861,7 +869,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
 #pragma unroll
           for (int w = 0; w < WPH; ++w)
             if (wave_ml[h][w].y > 0.f) l += wave_ml[h][w].y * __expf(wave_ml[h][w].x - m);
-          fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+          fz.stats[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
         }
       }
     }
@@ -1276,7 +1284,7 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
   const SegDev sg = tb.seg[si];
   const int tile = (int)blockIdx.y - begin_of_seg(tb, si);
 
-  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + hkv * NREP) * 128);
+  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + first_head(fz, hkv, NREP)) * 128);
   auto stage_q_pairs = [&]() {
 #pragma unroll
     for (int h = 0; h < NREP; ++h) q2s[lane * NREP + h] = as_h2(qsrc[h * 64 + lane]);
@@ -1369,10 +1377,10 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
       if (!valid) l_lane = 0.f;
       const float l = wave_sum(l_lane);
       if (lane == 0)
-        fz.stats[((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+        fz.stats[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
     }
     if (valid) {
-      half_t *srow = scores + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+      half_t *srow = scores + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall;
       // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one vector
       // store; otherwise 2-byte scatters through idx
       if (contig && (((uintptr_t)(srow + pos[0])) & (2 * TPL - 1)) == 0) {
@@ -1823,7 +1831,7 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   const bool fused = fz.stats != nullptr;
   half_t *prow[NREP];
 #pragma unroll
-  for (int h = 0; h < NREP; ++h) prow[h] = p + ((int64_t)b * Hq + hkv * NREP + h) * Tall;
+  for (int h = 0; h < NREP; ++h) prow[h] = p + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall;
   // The positions of the first block are asked for before anything else: what is read AT them (the logits) is the
   // longest chain of dependent loads at the start of a workgroup's life, and the statistics below wait in its shadow.
   PvPair<NREP, D / 32> first;
@@ -1832,7 +1840,7 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
     // merge the per-tile (m, l) pairs of each head: wave w serves heads w, w+4, ...; up to 128 tiles are read once
     // and kept in registers between the maximum and the sum
     for (int h = wave; h < NREP; h += PV_WAVES) {
-      const float2 *sp = fz.stats + ((int64_t)b * Hq + hkv * NREP + h) * fz.n_stat;
+      const float2 *sp = fz.stats + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat;
       const float2 none = make_float2(-INFINITY, 0.f);
       const float2 v0 = lane < fz.n_stat ? sp[lane] : none;
       const float2 v1 = lane + 64 < fz.n_stat ? sp[lane + 64] : none;
@@ -1904,7 +1912,7 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   for (int k = threadIdx.x; k < NREP * D; k += PV_THREADS) {
     const float v = red[k] + red[NREP * D + k] + red[2 * NREP * D + k] + red[3 * NREP * D + k];
     const int h = k / D, d = k % D;
-    float *dst = partial + ((int64_t)chunk_id * n_bhq + (int64_t)b * Hq + hkv * NREP + h) * D + d;
+    float *dst = partial + ((int64_t)chunk_id * n_bhq + (int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * D + d;
     if (fold) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // write-through
     else *dst = v;
   }
@@ -1936,7 +1944,7 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   static_assert(D % 2 == 0, "channel pairs");
   for (int o = threadIdx.x; o < NREP * (D / 2); o += PV_THREADS) {
     const int h = o / (D / 2), d = 2 * (o % (D / 2));
-    const int64_t row = (int64_t)b * Hq + hkv * NREP + h;
+    const int64_t row = (int64_t)b * Hq + first_head(fz, hkv, NREP) + h;
     const uint64_t *src = reinterpret_cast<const uint64_t *>(partial + row * D + d);
     const int64_t cstride = n_bhq * D / 2;  // in 8-byte units
     float t0 = 0.f, t1 = 0.f;
@@ -2267,8 +2275,7 @@ static int check_heads(const char *who, int64_t B, int64_t Hq, int64_t Hkv, int6
     return fail(HQEKV_E_ARG, "%s: need B>0 and Hq %% Hkv == 0 (B=%lld Hq=%lld Hkv=%lld)", who, (long long)B,
                 (long long)Hq, (long long)Hkv);
   const int64_t nrep = Hq / Hkv;
-  if (!(nrep == 1 || nrep == 2 || nrep == 4 || nrep == 8))
-    return fail(HQEKV_E_UNSUPPORTED, "%s: Hq/Hkv=%lld (supported: 1, 2, 4, 8)", who, (long long)nrep);
+  if (nrep > 64) return fail(HQEKV_E_UNSUPPORTED, "%s: Hq/Hkv=%lld (supported: up to 64)", who, (long long)nrep);
   if (B * Hkv > 0x7fffffffLL) return fail(HQEKV_E_ARG, "%s: B*Hkv too large", who);
   if (D <= 0 || D % 32 != 0) return fail(HQEKV_E_ARG, "%s: D=%lld must be a positive multiple of 32", who, (long long)D);
   return HQEKV_OK;
@@ -2309,17 +2316,53 @@ static int resolve_qk_tiling(int forced, const hqekv_seg *segs, int nseg, int64_
   return HQEKV_OK;
 }
 
-// Which form of the dot products a call uses: the matrix-core one exists for four query heads per KV head.
+static bool one_slice(int64_t nrep) { return nrep == 1 || nrep == 2 || nrep == 4 || nrep == 8; }
+
+// Which form of the dot products a call uses: the matrix-core one exists for four query heads per KV head, and
+// for the slices of four heads of a ratio that is served in slices.
 static bool dot_on_matrix_cores(int flags, int64_t nrep) {
-  if (nrep != 4 || (flags & HQEKV_DOT_VALU)) return false;
+  if ((nrep != 4 && one_slice(nrep)) || (flags & HQEKV_DOT_VALU)) return false;
   if (flags & HQEKV_DOT_MFMA) return true;
   return HQ_DEFAULT_DOT_MFMA;
 }
 
+// Query heads per KV head are served by kernels for 8, 4, 2 and 1 of them; any other ratio is cut into such slices
+// (5 = 4 + 1, 6 = 4 + 2, 7 = 4 + 2 + 1, 12 = 8 + 4, ...), one launch per slice, each reading the K or V side again.
+struct HeadSlices {
+  int n, off[16], size[16];
+};
+static HeadSlices head_slices(int64_t nrep) {
+  HeadSlices hs{};
+  int off = 0;
+  for (int c : {8, 4, 2, 1})
+    while (nrep - off >= c && hs.n < 16) {
+      hs.off[hs.n] = off;
+      hs.size[hs.n++] = c;
+      off += c;
+    }
+  return hs;
+}
+static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
+                           int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf, int nrep);
+
 static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
                      int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf) {
   if (tb.total_units == 0) return HQEKV_OK;
-  const int nrep = (int)(Hq / Hkv);
+  const int64_t nrep = Hq / Hkv;
+  if (one_slice(nrep)) return launch_qk_heads(tb, q, scores, B, Hq, Hkv, D, Tall, fz, st, tiling, mf, (int)nrep);
+  const HeadSlices hs = head_slices(nrep);
+  for (int k = 0; k < hs.n; ++k) {
+    FuseArgs f = fz;
+    f.head_group = (int32_t)nrep;
+    f.head_off = hs.off[k];
+    const int rc = launch_qk_heads(tb, q, scores, B, Hq, Hkv, D, Tall, f, st, tiling, mf, hs.size[k]);
+    if (rc) return rc;
+  }
+  return HQEKV_OK;
+}
+
+static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
+                           int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf, int nrep) {
   dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units);
   if (tiling >= 3) {
 #define LAUNCH(N_, TPL_, MF_)                                                                                        \
@@ -2390,27 +2433,36 @@ static int64_t seg_total_tokens(const hqekv_seg *segs, int nseg) {
 static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, float *partial, int64_t B,
                      int64_t Hq, int64_t Hkv, int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st,
                      bool mf, int stages = 3, const StepEpilogue *ep = nullptr) {
-  const int nrep = (int)(Hq / Hkv);
   const int64_t n_bhq = B * Hq;
   if (tb.total_units > 0 && (stages & 1)) {
     dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units), block(PV_THREADS);
+    const bool whole = one_slice(Hq / Hkv);
+    HeadSlices hs = head_slices(Hq / Hkv);
+    if (whole) hs = HeadSlices{1, {0}, {(int)(Hq / Hkv)}};
+    for (int k = 0; k < hs.n; ++k) {
+      FuseArgs f = fz;
+      if (!whole) {
+        f.head_group = (int32_t)(Hq / Hkv);
+        f.head_off = hs.off[k];
+      }
 #define LAUNCH(N_, D_, MF_)                                                                                   \
   hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_, MF_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
-                     (int)Hkv, Tall, chunk, n_bhq, fz)
+                     (int)Hkv, Tall, chunk, n_bhq, f)
 #define LAUNCH_D(N_) LAUNCH(N_, 128, false)
-    switch (nrep) {
-      case 1: LAUNCH_D(1); break;
-      case 2: LAUNCH_D(2); break;
-      case 4:
-        if (mf) LAUNCH(4, 128, true);
-        else LAUNCH_D(4);
-        break;
-      default: LAUNCH_D(8);
-    }
+      switch (hs.size[k]) {
+        case 1: LAUNCH_D(1); break;
+        case 2: LAUNCH_D(2); break;
+        case 4:
+          if (mf) LAUNCH(4, 128, true);
+          else LAUNCH_D(4);
+          break;
+        default: LAUNCH_D(8);
+      }
 #undef LAUNCH_D
 #undef LAUNCH
-    int rc = check_launch("pv_hybrid_kernel");
-    if (rc) return rc;
+      int rc = check_launch("pv_hybrid_kernel");
+      if (rc) return rc;
+    }
   }
   const bool combine = (stages & 2) && !fz.arrive;   // folded: the last p.V workgroups have written the output
   const bool epilogue = ep && (ep->ring_line || ep->app_rows > 0) && stages == 3;
@@ -2660,15 +2712,16 @@ static int decode_impl(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs
   fz.two_step = (flags & HQEKV_TWO_STEP_DEQUANT) ? 1 : 0;
   const bool fold_pays = seg_total_tokens(v_segs, n_v) * B * Hkv >= CB_FOLD_MIN_TOKEN_ROWS;
   const bool fold_forced = (flags & HQEKV_FOLD_COMBINE) != 0;
+  // (a ratio of heads served in slices runs several p.V launches against the one counter: it keeps the combine launch)
   if (kt.total_units > 0 && vt.total_units > 0 && vt.total_units <= CB_FOLD_MAX && !(flags & HQEKV_SEPARATE_COMBINE) &&
-      (fold_pays || fold_forced)) {
+      (fold_pays || fold_forced) && one_slice(Hq / Hkv)) {
     fz.arrive = (uint32_t *)(ws + L.arrive_off);
     fz.out = (half_t *)attn_out;
   }
   if ((flags & HQEKV_DOT_MFMA) && (flags & HQEKV_DOT_VALU))
     return fail(HQEKV_E_ARG, "decode_attn: HQEKV_DOT_MFMA and HQEKV_DOT_VALU exclude each other");
-  if ((flags & HQEKV_DOT_MFMA) && Hq / Hkv != 4)
-    return fail(HQEKV_E_UNSUPPORTED, "decode_attn: the matrix-core dot products need Hq/Hkv == 4 (got %lld)", (long long)(Hq / Hkv));
+  if ((flags & HQEKV_DOT_MFMA) && Hq / Hkv != 4 && one_slice(Hq / Hkv))
+    return fail(HQEKV_E_UNSUPPORTED, "decode_attn: the matrix-core dot products need Hq/Hkv == 4, or a ratio that is served in slices (got %lld)", (long long)(Hq / Hkv));
   const bool mf = dot_on_matrix_cores(flags, Hq / Hkv);
   if (flags & HQEKV_ONLY_RAW_QK) {   // the q.K^T launch alone, raw fp16 scores: no scaling, no statistics, no softmax
     FuseArgs raw{};

@@ -479,7 +479,7 @@ def test_random_configurations(dev):
         rnd = random.Random(1000 + case)
         B = rnd.choice([1, 1, 2, 3])
         Hkv = rnd.choice([1, 2, 4, 8])
-        Hq = Hkv * rnd.choice([1, 2, 4, 4, 8])
+        Hq = Hkv * rnd.choice([1, 2, 4, 4, 8])   # (other ratios: test_head_ratios_served_in_slices)
         nblocks = rnd.choice([1, 2, 3, 8, 17, 40, 64, 100])
         residual = rnd.choice([0, 0, 1, 5, 31, 32, 97, 200])
         nfr = 6 if rnd.random() < 0.5 else 5
@@ -536,6 +536,35 @@ def test_random_configurations(dev):
         assert torch.allclose(o.float(), o_stage, rtol=RTOL, atol=ATOL), what
         checked += 1
     assert checked >= 150
+
+
+@pytest.mark.parametrize("ratio", [3, 5, 6, 7, 12, 13])
+@pytest.mark.parametrize("fused", [1, 0], ids=["fused", "general"])
+@pytest.mark.parametrize("tiling", ["8waves", "wave512"])
+def test_head_ratios_served_in_slices(dev, ratio, fused, tiling):
+    """Query heads per KV head other than 1, 2, 4, 8 (repeat_kv takes any ratio: model/public_func.py:127-135) run
+    as slices of 8, 4, 2 and 1 heads, one launch pair each: every head row against the oracle, with the matrix-core
+    slices of four and without them, with and without an additive mask, and again over the same plan (the slices share
+    one workspace)."""
+    from hqekv_amd import _lib
+    from hqekv_amd.attention import DecodePlan, decode_attention
+    B, Hkv, T, residual = 2, 2, 1024 + 37, 37
+    q, cache = _case(B, ratio * Hkv, Hkv, T, 128, (0.1, 0.2, 0.3, 0.3, 0.1), residual, 300 + ratio)
+    c = synth.cache_to(cache, dev)
+    Tall = cache[41]
+    w_ref, o_ref = O.qkv_matmul(q, cache, None, 128, use_mask=False, round_per_class=False)
+    for dot in (0, _lib.DOT_VALU):
+        plan = DecodePlan(q.to(dev), c, flags=fused | dot | _lib.qk_tiling(_lib.QK_TILINGS[tiling]))
+        for rep in range(2):
+            w, o = plan.run(q.to(dev))
+            _close(w, w_ref, f"attn_weights dot={dot} rep={rep}")
+            _close(o, o_ref, f"attn_output dot={dot} rep={rep}")
+    mask = torch.zeros(B, 1, 1, Tall, dtype=torch.float16)
+    mask[..., : Tall // 3] = torch.finfo(torch.float16).min
+    wm_ref, om_ref = O.qkv_matmul(q, cache, mask, 128, use_mask=True, round_per_class=False)
+    wm, om = decode_attention(q.to(dev), c, mask.to(dev), Tall, zero_init=True, flags=fused)
+    _close(wm, wm_ref, "masked attn_weights")
+    _close(om, om_ref, "masked attn_output")
 
 
 @pytest.mark.parametrize("tiling", ["8waves", "4waves", "wave512", "wave256"])
