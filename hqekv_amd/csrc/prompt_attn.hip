@@ -104,8 +104,8 @@ __device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8
 }
 template <bool CAUSAL>
 __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a) {
-  __shared__ __align__(16) half_t ks[PA_BC * PA_KS];
-  __shared__ __align__(16) half_t vs[(PA_BC / 8) * PA_VG];
+  __shared__ __align__(16) half_t ks_all[2][PA_BC * PA_KS];
+  __shared__ __align__(16) half_t vs_all[2][(PA_BC / 8) * PA_VG];
   const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;   // the longest rows first
@@ -145,14 +145,18 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   src.v_row = (uint32_t)a.v_t * 2u;
   src.k_lane = (uint32_t)(threadIdx.x >> 4) * src.k_row + (threadIdx.x & 15) * 16u;        // rows tid / 16 + 16 i
   src.v_lane = (uint32_t)(threadIdx.x >> 4) * 4u * src.v_row + (threadIdx.x & 15) * 16u;   // rows 4 (tid / 16) + j
+  // Two tiles in LDS, one barrier per tile: iteration j parks tile j + 1 (requested during iteration j - 1) in the
+  // buffer that tile j - 1 was read from -- every wave has passed this iteration's barrier, so it has finished that
+  // tile -- requests tile j + 2 and works on tile j, which the barrier made visible.
   PaTileRegs tr;
   pa_tile_fetch(src, 0, tr);
-  for (int tile = 0; tile < n_tiles; ++tile) {
+  pa_tile_store(tr, ks_all[0], vs_all[0]);
+  pa_tile_fetch(src, PA_BC, tr);   // (rows past the end of the prompt read as zeros; a tile past the last one is parked and never used)
+  auto step = [&](int tile, const half_t *ks, const half_t *vs, half_t *ks_nxt, half_t *vs_nxt) {
     const int k0 = tile * PA_BC;
-    __syncthreads();   // the previous tile has been read by every wave
-    pa_tile_store(tr, ks, vs);
     __syncthreads();
-    if (tile + 1 < n_tiles) pa_tile_fetch(src, k0 + PA_BC, tr);   // in flight across the products
+    pa_tile_store(tr, ks_nxt, vs_nxt);
+    pa_tile_fetch(src, k0 + 2 * PA_BC, tr);   // in flight across the products
     // (a tile that lies after every query of this wave is worked through like any other: all its elements are masked,
     // the maximum stays and the exponentials are zeros; skipping it would cost a copy of the accumulators per tile)
     f16_t s[2];
@@ -205,6 +209,11 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
         const h8_t av = *reinterpret_cast<const h8_t *>(vs + (2 * t + h) * PA_VG + (d ^ ((d >> 4) & 7)) * 8);
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, p[t], o[dt], 0, 0, 0);
       }
+  };
+  // two tiles per round, so that each half works on fixed buffers; an odd count runs one tile more, all of it masked
+  for (int tile = 0; tile < n_tiles; tile += 2) {
+    step(tile, ks_all[0], vs_all[0], ks_all[1], vs_all[1]);
+    step(tile + 1, ks_all[1], vs_all[1], ks_all[0], vs_all[0]);
   }
   lsum += __shfl_xor(lsum, 32, 64);
   if (my_q < T) {
