@@ -465,21 +465,15 @@ def test_linearity_in_v_at_scale(dev):
     torch.testing.assert_close(o.float(), expect, rtol=2e-3, atol=2e-3)
 
 
-def test_random_configurations(dev):
-    """200 seeded random configurations: batch, GQA ratio 1..8, context 32..3500, class shares (with and
-    without the 1-bit class, either 1-bit coding), residual lengths, shuffled positions, masks, fused and
-    general path.  Probabilities against the oracle; the output against the oracle's p.V of the SAME
-    probabilities (a raw score on an fp16 rounding boundary may round the other way in another summation
-    order and move a peaked row by half a percent, which the first check tolerates and the second one
-    would otherwise inherit)."""
+def _random_configurations(dev, n_cases, seed0, ratios, kv_heads, least):
     import random
     from hqekv_amd.attention import decode_attention
     checked = 0
-    for case in range(200):
+    for case in range(seed0, seed0 + n_cases):
         rnd = random.Random(1000 + case)
         B = rnd.choice([1, 1, 2, 3])
-        Hkv = rnd.choice([1, 2, 4, 8])
-        Hq = Hkv * rnd.choice([1, 2, 4, 4, 8])   # (other ratios: test_head_ratios_served_in_slices)
+        Hkv = rnd.choice(kv_heads)
+        Hq = Hkv * rnd.choice(ratios)
         nblocks = rnd.choice([1, 2, 3, 8, 17, 40, 64, 100])
         residual = rnd.choice([0, 0, 1, 5, 31, 32, 97, 200])
         nfr = 6 if rnd.random() < 0.5 else 5
@@ -535,7 +529,22 @@ def test_random_configurations(dev):
         o_stage = torch.matmul(w.float(), O.repeat_kv(v_dense, Hq // Hkv).float())
         assert torch.allclose(o.float(), o_stage, rtol=RTOL, atol=ATOL), what
         checked += 1
-    assert checked >= 150
+    assert checked >= least
+
+
+def test_random_configurations(dev):
+    """200 seeded random configurations: batch, GQA ratio 1..8, context 32..3500, class shares (with and
+    without the 1-bit class, either 1-bit coding), residual lengths, shuffled positions, masks, fused and
+    general path.  Probabilities against the oracle; the output against the oracle's p.V of the SAME
+    probabilities (a raw score on an fp16 rounding boundary may round the other way in another summation
+    order and move a peaked row by half a percent, which the first check tolerates and the second one
+    would otherwise inherit)."""
+    _random_configurations(dev, 200, 0, [1, 2, 4, 4, 8], [1, 2, 4, 8], 150)
+
+
+def test_random_configurations_of_sliced_head_ratios(dev):
+    """The same draw for head ratios that run as slices of 8, 4, 2 and 1 heads (3, 5, 6, 7, 9, 12)."""
+    _random_configurations(dev, 60, 5000, [3, 5, 6, 7, 9, 12], [1, 2, 4], 40)
 
 
 @pytest.mark.parametrize("ratio", [3, 5, 6, 7, 12, 13])
