@@ -23,7 +23,7 @@ TWO_STEP_DEQUANT = 8
 ONLY_QK = 0x100
 ONLY_PV = 0x200
 ONLY_COMBINE = 0x400
-DOT_MFMA = 0x800    # inner products on the matrix cores (Hq/Hkv == 4, or the slices of four of a ratio served in slices)
+DOT_MFMA = 0x800    # inner products on the matrix cores (Hq/Hkv == 4, or a slice of four of a ratio above 8)
 DOT_VALU = 0x1000   # inner products on the vector ALU
 ONLY_RAW_QK = 0x2000   # the q.K^T launch alone, raw fp16 scores
 QK_TILINGS = {"8waves": 1, "4waves": 2, "wave512": 3, "wave256": 4}   # HQEKV_QK_TILING_*: tilings a call may force

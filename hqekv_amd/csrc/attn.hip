@@ -95,9 +95,9 @@ struct FuseArgs {
   uint32_t *arrive;
   half_t *out;         // (B*Hq, D) attention output, written by the last workgroup of each (b, kv head)
   int32_t two_step;    // never fold the bias removal of a code into its multiply (HQEKV_TWO_STEP_DEQUANT)
-  // A ratio of query heads to KV heads that no kernel is instantiated for (3, 5, 6, 7, 12, ...) is served in slices of
-  // 8, 4, 2 or 1 heads per KV head, one launch each: the launch's NREP heads are heads head_off .. head_off + NREP - 1
-  // of the head_group query heads of their KV head.  head_group 0: the launch covers all NREP heads (the usual case).
+  // More than eight query heads per KV head are served in slices of at most eight, one launch each: the launch's NREP
+  // heads are heads head_off .. head_off + NREP - 1 of the head_group query heads of their KV head.  head_group 0: the
+  // launch covers all NREP heads (the usual case).
   int32_t head_group, head_off;
 };
 // first query head (inside its batch row) that a workgroup of KV head `hkv` works on
@@ -702,10 +702,14 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
   }
 }
 
-// heads reduced per pass of the cross-wave reduction: 32 KB of LDS per pass either way
+// heads reduced per pass of the cross-wave reduction: the largest of 4 (four waves per tile only), 2, 1 that divides
+// the heads of the launch; at most 32 KB of LDS per pass
+__host__ __device__ constexpr int qk_reduce_heads(int nrep, int waves) {
+  return (waves == 4 && nrep % 4 == 0) ? 4 : (nrep % 2 == 0 ? 2 : 1);
+}
 template <int NREP, int QK_WAVES>
 struct QkReduce {
-  static constexpr int RH = QK_WAVES == 4 ? (NREP < 4 ? NREP : 4) : (NREP < 2 ? NREP : 2);
+  static constexpr int RH = qk_reduce_heads(NREP, QK_WAVES);
   static constexpr int VPT = RH * QK_TILE / (QK_WAVES * 64);  // values a thread sums and stores per pass
   static constexpr int WPH = QK_WAVES / RH;                    // waves that share a head in a pass
   static_assert(VPT >= 1 && VPT <= QK_TPL && WPH >= 1, "reduction shape");
@@ -2316,30 +2320,30 @@ static int resolve_qk_tiling(int forced, const hqekv_seg *segs, int nseg, int64_
   return HQEKV_OK;
 }
 
-static bool one_slice(int64_t nrep) { return nrep == 1 || nrep == 2 || nrep == 4 || nrep == 8; }
+static bool one_slice(int64_t nrep) { return nrep >= 1 && nrep <= 8; }
 
 // Which form of the dot products a call uses: the matrix-core one exists for four query heads per KV head, and
-// for the slices of four heads of a ratio that is served in slices.
+// for a slice of four heads of a ratio above eight (12 = 8 + 4).
 static bool dot_on_matrix_cores(int flags, int64_t nrep) {
   if ((nrep != 4 && one_slice(nrep)) || (flags & HQEKV_DOT_VALU)) return false;
   if (flags & HQEKV_DOT_MFMA) return true;
   return HQ_DEFAULT_DOT_MFMA;
 }
 
-// Query heads per KV head are served by kernels for 8, 4, 2 and 1 of them; any other ratio is cut into such slices
-// (5 = 4 + 1, 6 = 4 + 2, 7 = 4 + 2 + 1, 12 = 8 + 4, ...), one launch per slice, each reading the K or V side again.
+// The kernels exist for 1 to 8 query heads per KV head; a larger ratio is cut into slices of at most eight
+// (12 = 8 + 4, 13 = 8 + 5, ...), one launch per slice, each reading the K or V side again.
 struct HeadSlices {
   int n, off[16], size[16];
 };
 static HeadSlices head_slices(int64_t nrep) {
   HeadSlices hs{};
   int off = 0;
-  for (int c : {8, 4, 2, 1})
-    while (nrep - off >= c && hs.n < 16) {
-      hs.off[hs.n] = off;
-      hs.size[hs.n++] = c;
-      off += c;
-    }
+  while (off < nrep && hs.n < 16) {
+    const int c = nrep - off >= 8 ? 8 : (int)(nrep - off);
+    hs.off[hs.n] = off;
+    hs.size[hs.n++] = c;
+    off += c;
+  }
   return hs;
 }
 static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
@@ -2373,11 +2377,15 @@ static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int6
     switch (nrep) {
       case 1: LAUNCH_DS(1); break;
       case 2: LAUNCH_DS(2); break;
+      case 3: LAUNCH_DS(3); break;
       case 4:
         if (!mf) LAUNCH_DS(4);
         else if (tiling == 3) LAUNCH(4, 8, true);
         else LAUNCH(4, 4, true);
         break;
+      case 5: LAUNCH_DS(5); break;
+      case 6: LAUNCH_DS(6); break;
+      case 7: LAUNCH_DS(7); break;
       default: LAUNCH_DS(8);
     }
 #undef LAUNCH_DS
@@ -2387,7 +2395,7 @@ static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int6
   const int waves = tiling == 1 ? 8 : 4;
   const int tpw = 1;  // tiles per workgroup (2 and 4 measured no faster at B=8, 64k context)
   dim3 block((unsigned)waves * 64);
-  const int rh = waves == 4 ? (nrep < 4 ? nrep : 4) : (nrep < 2 ? nrep : 2);  // QkReduce::RH
+  const int rh = qk_reduce_heads(nrep, waves);  // QkReduce::RH
   const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
 #define LAUNCH(N_, W_, MF_)                                                                                        \
   hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_, MF_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
@@ -2397,11 +2405,15 @@ static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int6
   switch (nrep) {
     case 1: LAUNCH_W(1); break;
     case 2: LAUNCH_W(2); break;
+    case 3: LAUNCH_W(3); break;
     case 4:
       if (!mf) LAUNCH_W(4);
       else if (waves == 8) LAUNCH(4, 8, true);
       else LAUNCH(4, 4, true);
       break;
+    case 5: LAUNCH_W(5); break;
+    case 6: LAUNCH_W(6); break;
+    case 7: LAUNCH_W(7); break;
     default: LAUNCH_W(8);
   }
 #undef LAUNCH_W
@@ -2452,10 +2464,14 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
       switch (hs.size[k]) {
         case 1: LAUNCH_D(1); break;
         case 2: LAUNCH_D(2); break;
+        case 3: LAUNCH_D(3); break;
         case 4:
           if (mf) LAUNCH(4, 128, true);
           else LAUNCH_D(4);
           break;
+        case 5: LAUNCH_D(5); break;
+        case 6: LAUNCH_D(6); break;
+        case 7: LAUNCH_D(7); break;
         default: LAUNCH_D(8);
       }
 #undef LAUNCH_D
@@ -2712,7 +2728,7 @@ static int decode_impl(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs
   fz.two_step = (flags & HQEKV_TWO_STEP_DEQUANT) ? 1 : 0;
   const bool fold_pays = seg_total_tokens(v_segs, n_v) * B * Hkv >= CB_FOLD_MIN_TOKEN_ROWS;
   const bool fold_forced = (flags & HQEKV_FOLD_COMBINE) != 0;
-  // (a ratio of heads served in slices runs several p.V launches against the one counter: it keeps the combine launch)
+  // (more than eight heads per KV head run as several p.V launches against the one counter: they keep the combine launch)
   if (kt.total_units > 0 && vt.total_units > 0 && vt.total_units <= CB_FOLD_MAX && !(flags & HQEKV_SEPARATE_COMBINE) &&
       (fold_pays || fold_forced) && one_slice(Hq / Hkv)) {
     fz.arrive = (uint32_t *)(ws + L.arrive_off);
@@ -2721,7 +2737,7 @@ static int decode_impl(const hqekv_seg *k_segs, int n_k, const hqekv_seg *v_segs
   if ((flags & HQEKV_DOT_MFMA) && (flags & HQEKV_DOT_VALU))
     return fail(HQEKV_E_ARG, "decode_attn: HQEKV_DOT_MFMA and HQEKV_DOT_VALU exclude each other");
   if ((flags & HQEKV_DOT_MFMA) && Hq / Hkv != 4 && one_slice(Hq / Hkv))
-    return fail(HQEKV_E_UNSUPPORTED, "decode_attn: the matrix-core dot products need Hq/Hkv == 4, or a ratio that is served in slices (got %lld)", (long long)(Hq / Hkv));
+    return fail(HQEKV_E_UNSUPPORTED, "decode_attn: the matrix-core dot products need Hq/Hkv == 4, or a ratio above 8 (got %lld)", (long long)(Hq / Hkv));
   const bool mf = dot_on_matrix_cores(flags, Hq / Hkv);
   if (flags & HQEKV_ONLY_RAW_QK) {   // the q.K^T launch alone, raw fp16 scores: no scaling, no statistics, no softmax
     FuseArgs raw{};

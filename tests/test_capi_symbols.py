@@ -43,7 +43,7 @@ def test_argument_validation_without_a_gpu():
     rc = lib.hqekv_qk_hybrid(None, 0, None, None, 1, 6, 4, 128, 10, None)
     assert rc == -1  # Hq % Hkv
     rc = lib.hqekv_qk_hybrid(None, 0, None, None, 1, 12, 4, 128, 10, None)
-    assert rc == -1  # a group of 3 query heads per KV head is served (in slices): only the null pointers are wrong
+    assert rc == -1  # a group of 3 query heads per KV head is served: only the null pointers are wrong
     rc = lib.hqekv_qk_hybrid(None, 0, None, None, 1, 130, 2, 128, 10, None)
     assert rc == -4 and b"up to 64" in lib.hqekv_last_error()
     rc = lib.hqekv_normal1_quant_pack_rows(None, 0, 0, None, 0, 0, None, None, 0, 0, 1, 1, 48, None)

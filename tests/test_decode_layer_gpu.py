@@ -53,8 +53,8 @@ def _same_tuple(got, want, where, normal=False):
     (1, 8, 2, 300, 72, "high_uniform_group_low_normal_group", 0.25),   # the reference's shipped default
     (1, 4, 2, 20, 70, "uniform_group", 0.0),                            # prompt shorter than one block
     (2, 16, 4, 511, 40, "high_uniform_group_low_normal_group", 0.1),    # ragged prompt, GQA 4, two batch rows
-    (1, 6, 2, 200, 40, "uniform_group", 0.0),                           # three query heads per KV head (slices 2 + 1)
-    (2, 12, 2, 130, 40, "high_uniform_group_low_normal_group", 0.1),    # six per KV head (slices 4 + 2)
+    (1, 6, 2, 200, 40, "uniform_group", 0.0),                           # three query heads per KV head
+    (2, 12, 2, 130, 40, "high_uniform_group_low_normal_group", 0.1),    # six per KV head
 ])
 def test_layer_in_lockstep_with_oracle(dev, B, Hq, Hkv, T0, steps, strategy, bit_1):
     from hqekv_amd.decode_layer import HqeAttentionLayer

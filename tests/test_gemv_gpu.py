@@ -59,7 +59,7 @@ def test_pv_shape_any_token_count(dev, bit, T):
     _close(out, O.gemv_uniform_group(32, p, code, s, z, bit))
 
 
-@pytest.mark.parametrize("n_rep", [1, 2, 3, 4, 6, 7, 8, 11])   # (3, 6, 7, 11: served in slices of 8, 4, 2, 1 heads)
+@pytest.mark.parametrize("n_rep", [1, 2, 3, 4, 6, 7, 8, 11])   # (11: served as slices of 8 + 3 heads)
 def test_gqa_group_sizes(dev, n_rep):
     from hqekv_amd.matmul import cuda_bmm_fA_qB_uniform_group
     g = torch.Generator().manual_seed(300 + n_rep)

@@ -543,18 +543,18 @@ def test_random_configurations(dev):
 
 
 def test_random_configurations_of_sliced_head_ratios(dev):
-    """The same draw for head ratios that run as slices of 8, 4, 2 and 1 heads (3, 5, 6, 7, 9, 12)."""
+    """The same draw for the other head ratios up to 8 and for ratios that run as slices of at most eight heads (9, 12)."""
     _random_configurations(dev, 60, 5000, [3, 5, 6, 7, 9, 12], [1, 2, 4], 40)
 
 
 @pytest.mark.parametrize("ratio", [3, 5, 6, 7, 12, 13])
 @pytest.mark.parametrize("fused", [1, 0], ids=["fused", "general"])
 @pytest.mark.parametrize("tiling", ["8waves", "wave512"])
-def test_head_ratios_served_in_slices(dev, ratio, fused, tiling):
-    """Query heads per KV head other than 1, 2, 4, 8 (repeat_kv takes any ratio: model/public_func.py:127-135) run
-    as slices of 8, 4, 2 and 1 heads, one launch pair each: every head row against the oracle, with the matrix-core
-    slices of four and without them, with and without an additive mask, and again over the same plan (the slices share
-    one workspace)."""
+def test_other_head_ratios(dev, ratio, fused, tiling):
+    """Query heads per KV head other than 1, 2, 4, 8 (repeat_kv takes any ratio: model/public_func.py:127-135): 3, 5,
+    6, 7 have kernels of their own, 12 and 13 run as slices of at most eight heads, one launch pair each: every head
+    row against the oracle, with the matrix-core slice of four and without it, with and without an additive mask, and
+    again over the same plan (slices share one workspace)."""
     from hqekv_amd import _lib
     from hqekv_amd.attention import DecodePlan, decode_attention
     B, Hkv, T, residual = 2, 2, 1024 + 37, 37
