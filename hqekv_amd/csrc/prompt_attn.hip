@@ -7,31 +7,25 @@
 // Both kernels compute S^T = K . Q^T -- keys along M, queries along N of v_mfma_f32_32x32x16_f16 -- so that a lane
 // owns ONE query (column lane % 32): the running maximum, the sum and the rescaling of the output are per-lane
 // scalars, and the exponentials a lane holds (keys 8 g + 4 (lane / 32) + j of a 32-key tile, g = 0..3, j = 0..3) are
-// already laid out as the B operand of the second product, O^T = V^T . P^T.  That product needs, per lane, four
-// consecutive KEYS of one channel: the V tile is turned by 4 x 4 register transposes on its way into LDS, and laid out
-// [16-key step][lane half][channel slot][8 keys] so that the eight keys a lane feeds to one product -- 4 h + j and
-// 8 + 4 h + j of the step, for lane half h -- are one 16-byte read.  Channel d sits in slot d ^ ((d >> 4) & 7): the
-// sixteen writers of a row (channels 8 apart) and the 32 readers (adjacent channels) both spread over all banks.
+// already laid out as the B operand of the second product, O^T = V^T . P^T.  That product needs, per lane, eight
+// KEYS of one channel (4 h + j and 8 + 4 h + j of a 16-key step, for lane half h): V stays row-major in LDS and the
+// operand comes out of two transposing reads (ds_read_b64_tr_b16: a group of 16 lanes names four key rows x 32 bytes,
+// every lane receives four consecutive keys of one channel).
 #include "common.h"
-
-#ifndef HQ_PA_QLDS
-#define HQ_PA_QLDS 2
-#endif
 
 namespace hq {
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
 typedef float f16_t __attribute__((ext_vector_type(16)));
+typedef __fp16 h4raw_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+typedef __attribute__((address_space(3))) h4raw_t lds_h4_t;
 
 constexpr int PA_D = 128;
 constexpr int PA_WAVES = 4;
 constexpr int PA_THREADS = 64 * PA_WAVES;
 constexpr int PA_BR = 32 * PA_WAVES;   // query rows per workgroup
 constexpr int PA_BC = 64;              // keys per tile
-constexpr int PA_QLDS = HQ_PA_QLDS;    // of the eight 16-channel steps of a lane's query row, how many wait in LDS instead of registers
-constexpr int PA_KS = PA_D + 8;        // halfs per K row in LDS (the pad spreads the rows over the banks)
-constexpr int PA_VG = PA_D * 8;        // halfs per (16-key step, lane half) group of the turned V tile: 128 channels x 8 keys
 
 struct PromptArgs {
   const half_t *q, *k, *v;
@@ -44,68 +38,62 @@ struct PromptArgs {
   float scale;
 };
 
-__device__ __forceinline__ uint32_t lo_pair(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
-__device__ __forceinline__ uint32_t hi_pair(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 
-// one tile of keys on its way from memory to LDS: 16 bytes x 4 of K and of V per thread
-struct PaTileRegs {
-  uint4 kr[4], vr[4];
-};
-// (buffer loads: one per-thread offset for each of K and V, the tile's rows through the scalar offset; rows past the
-// end of the prompt read as zeros, and the scores mask them)
+// A tile of keys goes from memory to LDS without passing through registers (`buffer_load_dwordx4 ... lds`: lane l's
+// 16 bytes land at M0 + 16 l, so one wave instruction fills four 256-byte rows).  K and V are both row-major in LDS,
+// [key][128 channels], unpadded; banks are spread by a swizzle of the 16-byte pieces inside a row, applied on the
+// memory side: the lane that fills piece slot c of a row fetches piece c ^ (row % 16) of K, c ^ 4 (row % 4) of V.
+// These loads are inline asm (the compiler makes every LDS access after the builtin form wait for all of them), so the
+// wait -- vmcnt(0), once per tile, right before the barrier -- is explicit.
+typedef int desc_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ desc_t make_desc(const void *base, uint32_t bytes) {   // `base` and `bytes` wave-uniform
+  const uint64_t a = (uint64_t)(uintptr_t)base;
+  desc_t d;
+  d.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+  d.y = __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu));
+  d.z = __builtin_amdgcn_readfirstlane((int)bytes);
+  d.w = 0x00020000;
+  return d;
+}
+__device__ __forceinline__ uint32_t lds_offset_of(const void *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
+}
+__device__ __forceinline__ void dma_1k(uint32_t lds, desc_t d, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(lds), "v"(voff), "s"(d), "s"(soff) : "memory");
+}
+__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 struct PaSource {
-  rsrc_t k, v;
-  uint32_t k_lane, v_lane;   // this thread's byte offsets inside a tile
+  desc_t k, v;
+  uint32_t k_lane, v_lane;   // this thread's byte offsets inside a tile (row tid / 16, swizzled piece)
   uint32_t k_row, v_row;     // bytes between two keys
 };
-__device__ __forceinline__ uint4 buf_load16(rsrc_t r, uint32_t voff, uint32_t soff) {
-  typedef uint32_t v4u __attribute__((ext_vector_type(4)));
-  const v4u x = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
-  return make_uint4(x.x, x.y, x.z, x.w);
-}
-__device__ __forceinline__ void pa_tile_fetch(const PaSource &src, int k0, PaTileRegs &r) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) r.kr[i] = buf_load16(src.k, src.k_lane, (uint32_t)(k0 + 16 * i) * src.k_row);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) r.vr[j] = buf_load16(src.v, src.v_lane, (uint32_t)(k0 + j) * src.v_row);
-}
-__device__ __forceinline__ void pa_tile_store(const PaTileRegs &r, half_t *ks, half_t *vs) {
-  const int tid = threadIdx.x;
+// rows tid / 16 + 16 i of the tile; wave w's instruction i fills rows 16 i + 4 w .. + 3
+__device__ __forceinline__ void pa_tile_dma(const PaSource &src, int k0, const half_t *ks, const half_t *vs, int w) {
+  const uint32_t kb = lds_offset_of(ks) + (uint32_t)w * 1024u, vb = lds_offset_of(vs) + (uint32_t)w * 1024u;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int idx = tid + PA_THREADS * i, row = idx >> 4, c = idx & 15;
-    *reinterpret_cast<uint4 *>(ks + row * PA_KS + c * 8) = r.kr[i];
-  }
-  // 4 keys x 8 channels -> 8 channels x 4 keys; key quad = 4 t + 2 e + h: step t, first or second four of a lane's eight, lane half h
-  const int quad = tid >> 4, oct = tid & 15;
-  const uint32_t a[4] = {r.vr[0].x, r.vr[0].y, r.vr[0].z, r.vr[0].w}, b[4] = {r.vr[1].x, r.vr[1].y, r.vr[1].z, r.vr[1].w};
-  const uint32_t c[4] = {r.vr[2].x, r.vr[2].y, r.vr[2].z, r.vr[2].w}, e[4] = {r.vr[3].x, r.vr[3].y, r.vr[3].z, r.vr[3].w};
-  half_t *grp = vs + (2 * (quad >> 2) + (quad & 1)) * PA_VG + ((quad >> 1) & 1) * 4;
-  const int sw = (oct >> 1) & 7;   // ((d >> 4) & 7) for this thread's channels d = 8 oct + ch
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {   // channels 2p and 2p + 1 of this thread's eight
-    *reinterpret_cast<uint2 *>(grp + (8 * oct + ((2 * p) ^ sw)) * 8) = make_uint2(lo_pair(a[p], b[p]), lo_pair(c[p], e[p]));
-    *reinterpret_cast<uint2 *>(grp + (8 * oct + ((2 * p + 1) ^ sw)) * 8) = make_uint2(hi_pair(a[p], b[p]), hi_pair(c[p], e[p]));
+    dma_1k(kb + 4096u * i, src.k, src.k_lane, (uint32_t)(k0 + 16 * i) * src.k_row);
+    dma_1k(vb + 4096u * i, src.v, src.v_lane, (uint32_t)(k0 + 16 * i) * src.v_row);
   }
 }
 
 // S^T of one 64-key tile for the wave's 32 queries: two 32-key tiles, 16 fp32 values per lane each
-__device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8 - PA_QLDS], const h8_t *q_lds, int n, int h, f16_t &s0,
-                                          f16_t &s1) {
+__device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8], int n, int h, f16_t &s0, f16_t &s1) {
   s0 = s1 = (f16_t)(0.f);
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
-    const h8_t ka = *reinterpret_cast<const h8_t *>(ks + n * PA_KS + 16 * s + 8 * h);
-    const h8_t kb = *reinterpret_cast<const h8_t *>(ks + (32 + n) * PA_KS + 16 * s + 8 * h);
-    const h8_t qq = s < PA_QLDS ? q_lds[s * PA_THREADS] : qreg[s < PA_QLDS ? 0 : s - PA_QLDS];
-    s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qq, s0, 0, 0, 0);
-    s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb, qq, s1, 0, 0, 0);
+    const int piece = ((2 * s + h) ^ (n & 15)) * 8;   // (rows n and 32 + n share the swizzle)
+    const h8_t ka = *reinterpret_cast<const h8_t *>(ks + n * PA_D + piece);
+    const h8_t kb = *reinterpret_cast<const h8_t *>(ks + (32 + n) * PA_D + piece);
+    s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[s], s0, 0, 0, 0);
+    s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb, qreg[s], s1, 0, 0, 0);
   }
 }
 template <bool CAUSAL>
 __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a) {
-  __shared__ __align__(16) half_t ks_all[2][PA_BC * PA_KS];
-  __shared__ __align__(16) half_t vs_all[2][(PA_BC / 8) * PA_VG];
+  __shared__ __align__(16) half_t ks_all[2][PA_BC * PA_D];
+  __shared__ __align__(16) half_t vs_all[2][PA_BC * PA_D];
   const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;   // the longest rows first
@@ -116,20 +104,12 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   const half_t *kp = a.k + b * a.k_b + hkv * a.k_h;
   const half_t *vp = a.v + b * a.v_b + hkv * a.v_h;
   const int my_q = q0 + 32 * w + n;
-  // the lane's query row: 8 steps of 16 channels, of which it supplies 8 (by lane half); the first steps wait in a
-  // slot of LDS that only this lane touches (the registers are all spoken for: one spilled value costs a wait for
-  // every load in flight, every tile)
-  __shared__ __align__(16) h8_t q_slots[PA_QLDS > 0 ? PA_THREADS * PA_QLDS : 1];
-  h8_t *q_lds = q_slots + threadIdx.x;   // step s at q_lds[s * PA_THREADS]: adjacent lanes 16 bytes apart
-  h8_t qreg[8 - PA_QLDS];
+  // the lane's query row: 8 steps of 16 channels, of which it supplies 8 (by lane half)
+  h8_t qreg[8];
   {
     const half_t *qr = qp + (int64_t)min(my_q, T - 1) * a.q_t + 8 * h;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      const h8_t x = *reinterpret_cast<const h8_t *>(qr + 16 * s);
-      if (s < PA_QLDS) q_lds[s * PA_THREADS] = x;
-      else qreg[s < PA_QLDS ? 0 : s - PA_QLDS] = x;
-    }
+    for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const h8_t *>(qr + 16 * s);
   }
   f16_t o[4];
 #pragma unroll
@@ -139,28 +119,44 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   const int kend = CAUSAL ? min(T, q0 + PA_BR) : T;
   const int n_tiles = (kend + PA_BC - 1) / PA_BC;
   PaSource src;
-  src.k = make_rsrc(kp, (uint32_t)((int64_t)T * a.k_t * 2));   // (below 4 GiB: checked by the host)
-  src.v = make_rsrc(vp, (uint32_t)((int64_t)T * a.v_t * 2));
+  src.k = make_desc(kp, (uint32_t)((int64_t)T * a.k_t * 2));   // (below 4 GiB: checked by the host)
+  src.v = make_desc(vp, (uint32_t)((int64_t)T * a.v_t * 2));
   src.k_row = (uint32_t)a.k_t * 2u;
   src.v_row = (uint32_t)a.v_t * 2u;
-  src.k_lane = (uint32_t)(threadIdx.x >> 4) * src.k_row + (threadIdx.x & 15) * 16u;        // rows tid / 16 + 16 i
-  src.v_lane = (uint32_t)(threadIdx.x >> 4) * 4u * src.v_row + (threadIdx.x & 15) * 16u;   // rows 4 (tid / 16) + j
-  // Two tiles in LDS, one barrier per tile: iteration j parks tile j + 1 (requested during iteration j - 1) in the
-  // buffer that tile j - 1 was read from -- every wave has passed this iteration's barrier, so it has finished that
-  // tile -- requests tile j + 2 and works on tile j, which the barrier made visible.
-  PaTileRegs tr;
-  pa_tile_fetch(src, 0, tr);
-  pa_tile_store(tr, ks_all[0], vs_all[0]);
-  pa_tile_fetch(src, PA_BC, tr);   // (rows past the end of the prompt read as zeros; a tile past the last one is parked and never used)
+  {
+    const uint32_t row = threadIdx.x >> 4, slot = threadIdx.x & 15;
+    src.k_lane = row * src.k_row + ((slot ^ (row & 15)) * 16u);
+    src.v_lane = row * src.v_row + ((slot ^ (4 * (row & 3))) * 16u);
+  }
+  // Two tiles in LDS, one barrier per tile: iteration j waits for its own requests of tile j (made an iteration ago),
+  // passes the barrier -- now every wave's part of tile j is there and every wave has finished tile j - 1 -- requests
+  // tile j + 1 into the buffer that tile j - 1 was read from, and works on tile j.
+  // where this lane points the transposing reads of V: lane r of a group of 16 names key row 4h + r / 4 of a step and
+  // the 8 bytes of channels 32 dt + 16 (n / 16) + 4 (r % 4) ..; the row's pieces are swizzled by 4 (row % 4) = 4 (r / 4)
+  int v_off[4];
+  {
+    const int r = lane & 15, key = 4 * h + (r >> 2);
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      const int piece = 4 * dt + 2 * (n >> 4) + ((r & 3) >> 1);
+      v_off[dt] = key * PA_D + ((piece ^ (4 * (r >> 2))) * 8) + 4 * (r & 1);
+    }
+  }
+  // (rows past the end of the prompt are outside the buffer descriptors: whatever such a row holds in LDS -- zeros from
+  // this fill or an older tile's finite values -- meets an exponential that is exactly zero)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4 *>(&vs_all[0][0] + (threadIdx.x + PA_THREADS * i) * 8) = make_uint4(0, 0, 0, 0);
+  __syncthreads();
+  pa_tile_dma(src, 0, ks_all[0], vs_all[0], w);   // (a tile past the last one is fetched and never used)
   auto step = [&](int tile, const half_t *ks, const half_t *vs, half_t *ks_nxt, half_t *vs_nxt) {
     const int k0 = tile * PA_BC;
+    wait_all_loads();   // this wave's part of tile j, requested an iteration ago
     __syncthreads();
-    pa_tile_store(tr, ks_nxt, vs_nxt);
-    pa_tile_fetch(src, k0 + 2 * PA_BC, tr);   // in flight across the products
+    pa_tile_dma(src, k0 + PA_BC, ks_nxt, vs_nxt, w);   // in flight across the products
     // (a tile that lies after every query of this wave is worked through like any other: all its elements are masked,
     // the maximum stays and the exponentials are zeros; skipping it would cost a copy of the accumulators per tile)
     f16_t s[2];
-    pa_scores(ks, qreg, q_lds, n, h, s[0], s[1]);
+    pa_scores(ks, qreg, n, h, s[0], s[1]);
     const bool edge = (k0 + PA_BC > T) || (CAUSAL && k0 + PA_BC - 1 > q0 + 32 * w);   // some element of the tile is masked
     // the running maximum is kept in units of the scaled logit (base-2 exponent); a raw score enters as s * sl2
     if (edge) {   // (uniform per wave; one branch around all 32 selects)
@@ -205,8 +201,14 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
-        const int d = 32 * dt + n;
-        const h8_t av = *reinterpret_cast<const h8_t *>(vs + (2 * t + h) * PA_VG + (d ^ ((d >> 4) & 7)) * 8);
+        // V^T operand through the transposing LDS read: a group of 16 lanes names four key rows x 32 bytes and each
+        // lane receives four consecutive keys of one channel; two reads (keys 4h + j, 8 + 4h + j) make the operand
+        const half_t *src_lo = vs + v_off[dt] + 16 * t * PA_D;
+        const h4raw_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_h4_t *)(src_lo));
+        const h4raw_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_h4_t *)(src_lo + 8 * PA_D));
+        h8_t av;
+        __builtin_memcpy(&av, &lo, 8);
+        __builtin_memcpy(reinterpret_cast<char *>(&av) + 8, &hi, 8);
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, p[t], o[dt], 0, 0, 0);
       }
   };
