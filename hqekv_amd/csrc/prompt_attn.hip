@@ -217,6 +217,7 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     step(tile, ks_all[0], vs_all[0], ks_all[1], vs_all[1]);
     step(tile + 1, ks_all[1], vs_all[1], ks_all[0], vs_all[0]);
   }
+  wait_all_loads();   // the last request (a tile nobody reads) must have landed before this workgroup's LDS can go to another
   lsum += __shfl_xor(lsum, 32, 64);
   if (my_q < T) {
     const float inv = 1.0f / lsum;
