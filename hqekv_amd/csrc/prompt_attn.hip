@@ -25,7 +25,12 @@ constexpr int PA_D = 128;
 constexpr int PA_WAVES = 4;
 constexpr int PA_THREADS = 64 * PA_WAVES;
 constexpr int PA_BR = 32 * PA_WAVES;   // query rows per workgroup
-constexpr int PA_BC = 64;              // keys per tile
+#ifndef HQ_PA_BC
+#define HQ_PA_BC 32
+#endif
+constexpr int PA_BC = HQ_PA_BC;        // keys per tile: 32 (164 registers, 32 KB of LDS: three workgroups per CU) or 64 (two)
+constexpr int PA_NS = PA_BC / 32;      // 32-key score tiles per key tile
+constexpr int PA_WGS = PA_BC == 64 ? 2 : 3;
 
 struct PromptArgs {
   const half_t *q, *k, *v;
@@ -72,26 +77,28 @@ struct PaSource {
 __device__ __forceinline__ void pa_tile_dma(const PaSource &src, int k0, const half_t *ks, const half_t *vs, int w) {
   const uint32_t kb = lds_offset_of(ks) + (uint32_t)w * 1024u, vb = lds_offset_of(vs) + (uint32_t)w * 1024u;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < PA_BC / 16; ++i) {
     dma_1k(kb + 4096u * i, src.k, src.k_lane, (uint32_t)(k0 + 16 * i) * src.k_row);
     dma_1k(vb + 4096u * i, src.v, src.v_lane, (uint32_t)(k0 + 16 * i) * src.v_row);
   }
 }
 
-// S^T of one 64-key tile for the wave's 32 queries: two 32-key tiles, 16 fp32 values per lane each
-__device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8], int n, int h, f16_t &s0, f16_t &s1) {
-  s0 = s1 = (f16_t)(0.f);
+// S^T of one key tile for the wave's 32 queries: PA_NS score tiles of 32 keys, 16 fp32 values per lane each
+__device__ __forceinline__ void pa_scores(const half_t *ks, const h8_t (&qreg)[8], int n, int h, f16_t (&sc)[PA_NS]) {
+#pragma unroll
+  for (int mt = 0; mt < PA_NS; ++mt) sc[mt] = (f16_t)(0.f);
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
     const int piece = ((2 * s + h) ^ (n & 15)) * 8;   // (rows n and 32 + n share the swizzle)
-    const h8_t ka = *reinterpret_cast<const h8_t *>(ks + n * PA_D + piece);
-    const h8_t kb = *reinterpret_cast<const h8_t *>(ks + (32 + n) * PA_D + piece);
-    s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[s], s0, 0, 0, 0);
-    s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kb, qreg[s], s1, 0, 0, 0);
+#pragma unroll
+    for (int mt = 0; mt < PA_NS; ++mt) {
+      const h8_t kk = *reinterpret_cast<const h8_t *>(ks + (32 * mt + n) * PA_D + piece);
+      sc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kk, qreg[s], sc[mt], 0, 0, 0);
+    }
   }
 }
 template <bool CAUSAL>
-__global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a) {
+__global__ __launch_bounds__(PA_THREADS, PA_WGS) void prompt_attn_kernel(PromptArgs a) {
   __shared__ __align__(16) half_t ks_all[2][PA_BC * PA_D];
   __shared__ __align__(16) half_t vs_all[2][PA_BC * PA_D];
   const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -145,7 +152,7 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
   // (rows past the end of the prompt are outside the buffer descriptors: whatever such a row holds in LDS -- zeros from
   // this fill or an older tile's finite values -- meets an exponential that is exactly zero)
 #pragma unroll
-  for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4 *>(&vs_all[0][0] + (threadIdx.x + PA_THREADS * i) * 8) = make_uint4(0, 0, 0, 0);
+  for (int i = 0; i < PA_BC / 8; ++i) *reinterpret_cast<uint4 *>(&vs_all[0][0] + (threadIdx.x + PA_THREADS * i) * 8) = make_uint4(0, 0, 0, 0);
   __syncthreads();
   pa_tile_dma(src, 0, ks_all[0], vs_all[0], w);   // (a tile past the last one is fetched and never used)
   auto step = [&](int tile, const half_t *ks, const half_t *vs, half_t *ks_nxt, half_t *vs_nxt) {
@@ -155,21 +162,21 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
     pa_tile_dma(src, k0 + PA_BC, ks_nxt, vs_nxt, w);   // in flight across the products
     // (a tile that lies after every query of this wave is worked through like any other: all its elements are masked,
     // the maximum stays and the exponentials are zeros; skipping it would cost a copy of the accumulators per tile)
-    f16_t s[2];
-    pa_scores(ks, qreg, n, h, s[0], s[1]);
+    f16_t s[PA_NS];
+    pa_scores(ks, qreg, n, h, s);
     const bool edge = (k0 + PA_BC > T) || (CAUSAL && k0 + PA_BC - 1 > q0 + 32 * w);   // some element of the tile is masked
     // the running maximum is kept in units of the scaled logit (base-2 exponent); a raw score enters as s * sl2
     if (edge) {   // (uniform per wave; one branch around all 32 selects)
       const int last_key = (CAUSAL ? min(my_q, T - 1) : T - 1) - k0 - 4 * h;   // the last visible key, relative to element r's base
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
+      for (int mt = 0; mt < PA_NS; ++mt)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           if (32 * mt + 8 * (r >> 2) + (r & 3) > last_key) s[mt][r] = -INFINITY;
     }
     float raw = -INFINITY;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < PA_NS; ++mt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) raw = fmaxf(raw, s[mt][r]);
     float mx = fmaxf(m, raw * sl2);   // (sl2 > 0)
@@ -187,9 +194,9 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
       m = mx;
     }
     float part = 0.f;
-    h8_t p[4];
+    h8_t p[2 * PA_NS];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < PA_NS; ++mt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][r], sl2, -mx));
@@ -198,7 +205,7 @@ __global__ __launch_bounds__(PA_THREADS, 2) void prompt_attn_kernel(PromptArgs a
       }
     lsum += part;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 2 * PA_NS; ++t)
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
         // V^T operand through the transposing LDS read: a group of 16 lanes names four key rows x 32 bytes and each
