@@ -95,15 +95,16 @@ struct FuseArgs {
   uint32_t *arrive;
   half_t *out;         // (B*Hq, D) attention output, written by the last workgroup of each (b, kv head)
   int32_t two_step;    // never fold the bias removal of a code into its multiply (HQEKV_TWO_STEP_DEQUANT)
-  // More than eight query heads per KV head are served in slices of at most eight, one launch each: the launch's NREP
-  // heads are heads head_off .. head_off + NREP - 1 of the head_group query heads of their KV head.  head_group 0: the
-  // launch covers all NREP heads (the usual case).
-  int32_t head_group, head_off;
 };
-// first query head (inside its batch row) that a workgroup of KV head `hkv` works on
-__device__ __forceinline__ int first_head(const FuseArgs &fz, int hkv, int nrep) {
-  return fz.head_group ? hkv * fz.head_group + fz.head_off : hkv * nrep;
-}
+// More than eight query heads per KV head are served in slices of at most eight, one launch each: the launch's NREP
+// heads are heads `off` .. `off` + NREP - 1 of the `group` query heads of their KV head (a launch that covers all
+// heads: group = NREP, off = 0).  Group and offset ride in the upper half of the kernels' head-count argument,
+// hq_slice = Hq | group << 16 | off << 24, and are used without a branch: as two members at the end of FuseArgs, or
+// behind a test for "no slices", the kernel's other scalar loads ended up behind a first, dependent one -- half a
+// microsecond in every workgroup -- and even one more plain argument moved the launches by a quarter.
+// -> first query head (inside its batch row) that a workgroup of KV head `hkv` works on
+__device__ __forceinline__ int first_head(int hq_slice, int hkv) { return hkv * ((hq_slice >> 16) & 0xff) + (int)((uint32_t)hq_slice >> 24); }
+__host__ __device__ constexpr int hq_with_slice(int Hq, int group, int off) { return Hq | group << 16 | off << 24; }
 
 // What the caller of a decode step does next to the attention (model/llama_hqe.py:131-133, 200), folded into the
 // step's last launch: the row of the importance ring -- the probabilities summed over the batch, rounded to fp16,
@@ -602,7 +603,7 @@ __device__ __forceinline__ void qk_f16_cm_accumulate(const SegDev &sg, uint32_t 
 // all of a wave's loads are in flight together and a token's dot product is reduced across 8 lanes.
 // Other D: a wave walks its tokens one by one, lanes split the channels.
 template <int NREP, int QK_WAVES>
-__device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int bh, int b, int hkv, int D,
+__device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int bh, int b, int head0, int D,
                                                int Hq, int64_t Tall, int wave, int lane, const half2_t *q2s,
                                                half_t *__restrict__ scores, const FuseArgs &fz, float *red) {
   const int64_t n = sg.n_tokens;
@@ -650,7 +651,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
           l_run[h] = l_run[h] * keep + wave_sum(e);
           m_run[h] = mn;
         }
-        if (valid && lg == 0) scores[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall + pos] = rr;
+        if (valid && lg == 0) scores[((int64_t)b * Hq + head0 + h) * Tall + pos] = rr;
       }
     }
   } else {
@@ -676,7 +677,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
           l_run[h] = l_run[h] * __expf(m_run[h] - mn) + __expf(x - mn);
           m_run[h] = mn;
         }
-        if (lane == 0) scores[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall + pos] = r;
+        if (lane == 0) scores[((int64_t)b * Hq + head0 + h) * Tall + pos] = r;
       }
     }
   }
@@ -697,7 +698,7 @@ __device__ __forceinline__ void qk_f16_tm_tile(const SegDev &sg, int tile, int b
         const float lw = red[(w * NREP + h) * 2 + 1];
         if (lw > 0.f) l += lw * __expf(red[(w * NREP + h) * 2] - m);
       }
-      fz.stats[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+      fz.stats[((int64_t)b * Hq + head0 + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
     }
   }
 }
@@ -720,7 +721,7 @@ struct QkReduce {
 //
 template <int NREP, int QK_WAVES, bool MF = false>
 __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void qk_hybrid_kernel(SegTable tb, const half_t *__restrict__ q,
-                                                               half_t *__restrict__ scores, int Hq,
+                                                               half_t *__restrict__ scores, int hq_slice,
                                                                int Hkv, int D, int64_t Tall, FuseArgs fz, int tpw) {
   using R = QkReduce<NREP, QK_WAVES>;
   constexpr int RH = R::RH, VPT = R::VPT, WPH = R::WPH;
@@ -731,6 +732,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int bh = blockIdx.x;
   const int b = bh / Hkv, hkv = bh % Hkv;
+  const int Hq = hq_slice & 0xffff, head0 = first_head(hq_slice, hkv);
   if (fz.arrive && blockIdx.y == 0 && threadIdx.x == 0) fz.arrive[bh] = 0;  // for the p.V launch that follows
   // grid.y counts workgroups; a workgroup takes `tpw` consecutive tiles of one class (1 unless the
   // environment asks for more: longer-lived workgroups stage the query once, but measured no faster)
@@ -740,7 +742,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
   const int tile_end = min(tile_begin + tpw, (int)sg.n_units);
   const bool tm = sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR;
   const uint32_t n = (uint32_t)sg.n_tokens;
-  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + first_head(fz, hkv, NREP)) * D);
+  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + head0) * D);
   // The query is staged by the first tile only; for every tile the call is the workgroup barrier between
   // "first loads requested" and "arithmetic starts", and between two tiles' uses of the reduction buffer.
   bool staged = false;
@@ -758,7 +760,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
 #pragma unroll 1
     for (int tile = tile_begin; tile < tile_end; ++tile) {
       stage_q();
-      qk_f16_tm_tile<NREP, QK_WAVES>(sg, tile, bh, b, hkv, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
+      qk_f16_tm_tile<NREP, QK_WAVES>(sg, tile, bh, b, head0, D, Hq, Tall, wave, lane, q2s, scores, fz, red);
     }
     return;
   }
@@ -851,7 +853,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
           if (lane == 0) wave_ml[h][wave - hl * WPH] = make_float2(m, l);
         }
         if (tok < n) {
-          half_t *srow = scores + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall;
+          half_t *srow = scores + ((int64_t)b * Hq + head0 + h) * Tall;
           // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one
           // vector store; otherwise 2-byte scatters through idx
           if (contig && (((uintptr_t)(srow + pos[0])) & (VPT * 2 - 1)) == 0) {
@@ -873,7 +875,7 @@ __global__ __launch_bounds__(QK_WAVES * 64, NREP <= 4 ? 16 / QK_WAVES : 1) void 
 #pragma unroll
           for (int w = 0; w < WPH; ++w)
             if (wave_ml[h][w].y > 0.f) l += wave_ml[h][w].y * __expf(wave_ml[h][w].x - m);
-          fz.stats[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+          fz.stats[((int64_t)b * Hq + head0 + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
         }
       }
     }
@@ -1273,7 +1275,7 @@ __device__ __forceinline__ void qw_f16_accumulate(const SegDev &sg, uint32_t ts,
 
 template <int NREP, int TPL, bool MF = false>
 __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wave_kernel(SegTable tb, const half_t *__restrict__ q,
-                                                                              half_t *__restrict__ scores, int Hq, int Hkv,
+                                                                              half_t *__restrict__ scores, int hq_slice, int Hkv,
                                                                               int64_t Tall, FuseArgs fz) {
   using G = QwGeom<TPL>;
   // [row pair][head]: (q[d], q[d+1]); matrix-core form: [head][row pair], QW_QH_STRIDE pairs per head
@@ -1283,12 +1285,13 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
   const int lane = threadIdx.x;
   const int bh = blockIdx.x;
   const int b = bh / Hkv, hkv = bh % Hkv;
+  const int Hq = hq_slice & 0xffff, head0 = first_head(hq_slice, hkv);
   if (fz.arrive && blockIdx.y == 0 && lane == 0) fz.arrive[bh] = 0;  // for the p.V launch that follows
   const int si = seg_of_unit(tb, blockIdx.y);
   const SegDev sg = tb.seg[si];
   const int tile = (int)blockIdx.y - begin_of_seg(tb, si);
 
-  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + first_head(fz, hkv, NREP)) * 128);
+  const uint32_t *qsrc = reinterpret_cast<const uint32_t *>(q + ((int64_t)b * Hq + head0) * 128);
   auto stage_q_pairs = [&]() {
 #pragma unroll
     for (int h = 0; h < NREP; ++h) q2s[lane * NREP + h] = as_h2(qsrc[h * 64 + lane]);
@@ -1304,7 +1307,7 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
   if (sg.bits == 16 && sg.layout == HQEKV_LAYOUT_TOKEN_MAJOR) {
     stage_q_pairs();
     __syncthreads();
-    qk_f16_tm_tile<NREP, 1>(sg, tile, bh, b, hkv, 128, Hq, Tall, 0, lane, q2s, scores, fz, red);
+    qk_f16_tm_tile<NREP, 1>(sg, tile, bh, b, head0, 128, Hq, Tall, 0, lane, q2s, scores, fz, red);
     return;
   }
   const uint32_t n = (uint32_t)sg.n_tokens;
@@ -1381,10 +1384,10 @@ __global__ __launch_bounds__(64, NREP <= 4 ? (TPL == 8 ? 4 : 6) : 2) void qk_wav
       if (!valid) l_lane = 0.f;
       const float l = wave_sum(l_lane);
       if (lane == 0)
-        fz.stats[((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
+        fz.stats[((int64_t)b * Hq + head0 + h) * fz.n_stat + sg.unit_begin + tile] = make_float2(m, l);
     }
     if (valid) {
-      half_t *srow = scores + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall;
+      half_t *srow = scores + ((int64_t)b * Hq + head0 + h) * Tall;
       // consecutive positions (classes are made of 32-token blocks) and an aligned destination: one vector
       // store; otherwise 2-byte scatters through idx
       if (contig && (((uintptr_t)(srow + pos[0])) & (2 * TPL - 1)) == 0) {
@@ -1818,7 +1821,7 @@ __device__ __forceinline__ void pv_chunk(const SegDev &sg, int64_t c0, int64_t c
 #endif
 template <int NREP, int D, bool MF = false>
 __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid_kernel(SegTable tb, half_t *__restrict__ p,
-                                                               float *__restrict__ partial, int Hq, int Hkv,
+                                                               float *__restrict__ partial, int hq_slice, int Hkv,
                                                                int64_t Tall, int64_t chunk_tokens,
                                                                int64_t n_bhq, FuseArgs fz) {
   __shared__ float red[PV_WAVES * NREP * D];
@@ -1829,13 +1832,14 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   const int ux = (int)blockIdx.y - sg.unit_begin;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = bh / Hkv, hkv = bh % Hkv;
+  const int Hq = hq_slice & 0xffff, head0 = first_head(hq_slice, hkv);
   const int chunk_id = sg.unit_begin + ux;
   const int64_t c0 = (int64_t)ux * chunk_tokens;
   const int64_t c1 = min(c0 + chunk_tokens, sg.n_tokens);
   const bool fused = fz.stats != nullptr;
   half_t *prow[NREP];
 #pragma unroll
-  for (int h = 0; h < NREP; ++h) prow[h] = p + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * Tall;
+  for (int h = 0; h < NREP; ++h) prow[h] = p + ((int64_t)b * Hq + head0 + h) * Tall;
   // The positions of the first block are asked for before anything else: what is read AT them (the logits) is the
   // longest chain of dependent loads at the start of a workgroup's life, and the statistics below wait in its shadow.
   PvPair<NREP, D / 32> first;
@@ -1844,7 +1848,7 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
     // merge the per-tile (m, l) pairs of each head: wave w serves heads w, w+4, ...; up to 128 tiles are read once
     // and kept in registers between the maximum and the sum
     for (int h = wave; h < NREP; h += PV_WAVES) {
-      const float2 *sp = fz.stats + ((int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * fz.n_stat;
+      const float2 *sp = fz.stats + ((int64_t)b * Hq + head0 + h) * fz.n_stat;
       const float2 none = make_float2(-INFINITY, 0.f);
       const float2 v0 = lane < fz.n_stat ? sp[lane] : none;
       const float2 v1 = lane + 64 < fz.n_stat ? sp[lane + 64] : none;
@@ -1916,7 +1920,7 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   for (int k = threadIdx.x; k < NREP * D; k += PV_THREADS) {
     const float v = red[k] + red[NREP * D + k] + red[2 * NREP * D + k] + red[3 * NREP * D + k];
     const int h = k / D, d = k % D;
-    float *dst = partial + ((int64_t)chunk_id * n_bhq + (int64_t)b * Hq + first_head(fz, hkv, NREP) + h) * D + d;
+    float *dst = partial + ((int64_t)chunk_id * n_bhq + (int64_t)b * Hq + head0 + h) * D + d;
     if (fold) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // write-through
     else *dst = v;
   }
@@ -1948,7 +1952,7 @@ __global__ __launch_bounds__(PV_THREADS, MF ? HQ_PV_MF_WAVES : 1) void pv_hybrid
   static_assert(D % 2 == 0, "channel pairs");
   for (int o = threadIdx.x; o < NREP * (D / 2); o += PV_THREADS) {
     const int h = o / (D / 2), d = 2 * (o % (D / 2));
-    const int64_t row = (int64_t)b * Hq + first_head(fz, hkv, NREP) + h;
+    const int64_t row = (int64_t)b * Hq + head0 + h;
     const uint64_t *src = reinterpret_cast<const uint64_t *>(partial + row * D + d);
     const int64_t cstride = n_bhq * D / 2;  // in 8-byte units
     float t0 = 0.f, t1 = 0.f;
@@ -2280,6 +2284,7 @@ static int check_heads(const char *who, int64_t B, int64_t Hq, int64_t Hkv, int6
                 (long long)Hq, (long long)Hkv);
   const int64_t nrep = Hq / Hkv;
   if (nrep > 64) return fail(HQEKV_E_UNSUPPORTED, "%s: Hq/Hkv=%lld (supported: up to 64)", who, (long long)nrep);
+  if (Hq > 0xffff) return fail(HQEKV_E_UNSUPPORTED, "%s: Hq=%lld (supported: up to 65535)", who, (long long)Hq);
   if (B * Hkv > 0x7fffffffLL) return fail(HQEKV_E_ARG, "%s: B*Hkv too large", who);
   if (D <= 0 || D % 32 != 0) return fail(HQEKV_E_ARG, "%s: D=%lld must be a positive multiple of 32", who, (long long)D);
   return HQEKV_OK;
@@ -2347,31 +2352,31 @@ static HeadSlices head_slices(int64_t nrep) {
   return hs;
 }
 static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
-                           int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf, int nrep);
+                           int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf, int nrep,
+                           int head_slice);
 
 static int launch_qk(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
                      int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf) {
   if (tb.total_units == 0) return HQEKV_OK;
   const int64_t nrep = Hq / Hkv;
-  if (one_slice(nrep)) return launch_qk_heads(tb, q, scores, B, Hq, Hkv, D, Tall, fz, st, tiling, mf, (int)nrep);
+  if (one_slice(nrep)) return launch_qk_heads(tb, q, scores, B, Hq, Hkv, D, Tall, fz, st, tiling, mf, (int)nrep, (int)(nrep << 16));
   const HeadSlices hs = head_slices(nrep);
   for (int k = 0; k < hs.n; ++k) {
-    FuseArgs f = fz;
-    f.head_group = (int32_t)nrep;
-    f.head_off = hs.off[k];
-    const int rc = launch_qk_heads(tb, q, scores, B, Hq, Hkv, D, Tall, f, st, tiling, mf, hs.size[k]);
+    const int rc = launch_qk_heads(tb, q, scores, B, Hq, Hkv, D, Tall, fz, st, tiling, mf, hs.size[k],
+                                   (int)(nrep << 16) | hs.off[k]);
     if (rc) return rc;
   }
   return HQEKV_OK;
 }
 
 static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int64_t B, int64_t Hq, int64_t Hkv,
-                           int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf, int nrep) {
+                           int64_t D, int64_t Tall, const FuseArgs &fz, hipStream_t st, int tiling, bool mf, int nrep,
+                           int head_slice) {
   dim3 grid((unsigned)(B * Hkv), (unsigned)tb.total_units);
   if (tiling >= 3) {
 #define LAUNCH(N_, TPL_, MF_)                                                                                        \
   hipLaunchKernelGGL((qk_wave_kernel<N_, TPL_, MF_>), grid, dim3(64), 0, st, tb, (const half_t *)q, (half_t *)scores, \
-                     (int)Hq, (int)Hkv, Tall, fz)
+                     hq_with_slice((int)Hq, head_slice >> 16, head_slice & 0xffff), (int)Hkv, Tall, fz)
 #define LAUNCH_DS(N_) \
   if (tiling == 3) LAUNCH(N_, 8, false); else LAUNCH(N_, 4, false)
     switch (nrep) {
@@ -2399,7 +2404,7 @@ static int launch_qk_heads(const SegTable &tb, const void *q, void *scores, int6
   const size_t shmem = (size_t)(nrep * D / 2 + waves * rh * QK_TILE) * sizeof(float);
 #define LAUNCH(N_, W_, MF_)                                                                                        \
   hipLaunchKernelGGL((qk_hybrid_kernel<N_, W_, MF_>), grid, block, shmem, st, tb, (const half_t *)q, (half_t *)scores, \
-                     (int)Hq, (int)Hkv, (int)D, Tall, fz, tpw)
+                     hq_with_slice((int)Hq, head_slice >> 16, head_slice & 0xffff), (int)Hkv, (int)D, Tall, fz, tpw)
 #define LAUNCH_W(N_) \
   if (waves == 8) LAUNCH(N_, 8, false); else LAUNCH(N_, 4, false)
   switch (nrep) {
@@ -2452,14 +2457,10 @@ static int launch_pv(const SegTable &tb, int64_t chunk, void *p, void *out, floa
     HeadSlices hs = head_slices(Hq / Hkv);
     if (whole) hs = HeadSlices{1, {0}, {(int)(Hq / Hkv)}};
     for (int k = 0; k < hs.n; ++k) {
-      FuseArgs f = fz;
-      if (!whole) {
-        f.head_group = (int32_t)(Hq / Hkv);
-        f.head_off = hs.off[k];
-      }
+      const int head_slice = ((int)(Hq / Hkv) << 16) | (whole ? 0 : hs.off[k]);
 #define LAUNCH(N_, D_, MF_)                                                                                   \
-  hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_, MF_>), grid, block, 0, st, tb, (half_t *)p, partial, (int)Hq, \
-                     (int)Hkv, Tall, chunk, n_bhq, f)
+  hipLaunchKernelGGL((pv_hybrid_kernel<N_, D_, MF_>), grid, block, 0, st, tb, (half_t *)p, partial,          \
+                     hq_with_slice((int)Hq, head_slice >> 16, head_slice & 0xffff), (int)Hkv, Tall, chunk, n_bhq, fz)
 #define LAUNCH_D(N_) LAUNCH(N_, 128, false)
       switch (hs.size[k]) {
         case 1: LAUNCH_D(1); break;

@@ -264,7 +264,7 @@ int hqekv_pv_hybrid(const hqekv_seg *segs, int nseg, const void *p, void *out, i
  * instruction per four elements of the reduction axis and lane, in place of eight two-element dot products on the
  * vector ALU.  The dequantised values are the same bits either way, products are exact and accumulation is fp32 in
  * both; only the order of the additions differs.  Neither flag: the library's default for the shape.
- * Head ratios: the kernels exist for 1 to 8 query heads per KV head; a larger ratio, up to 64, is served in slices of
+ * Head ratios (Hq up to 65535): the kernels exist for 1 to 8 query heads per KV head; a larger ratio, up to 64, is served in slices of
  * at most eight heads (12 = 8 + 4, 13 = 8 + 5, ...), one launch per slice and GEMV (each reads the cache again), a
  * slice of four in the form the flags name.  HQEKV_DOT_MFMA with a ratio of 1-3 or 5-8 returns HQEKV_E_UNSUPPORTED. */
 #define HQEKV_DOT_MFMA 0x800
