@@ -723,9 +723,10 @@ def main():
             out["extra"] = {"skipped": f"configuration 4 does not fit: {e}"}
 
     if args.workload == "c2" and not args.no_extra:
-        # the prompt side beside the headline: a short run of the causal prompt attention (16384 tokens)
+        # the prompt side beside the headline: a short run of the causal prompt attention at the size of
+        # `--workload prompt` (32768 tokens)
         try:
-            out["extra_prompt"] = measure_prompt(16384, 5, 2)
+            out["extra_prompt"] = measure_prompt(32768, 4, 2)
         except (torch.OutOfMemoryError, RuntimeError) as e:
             out["extra_prompt"] = {"skipped": str(e)[:200]}
 
